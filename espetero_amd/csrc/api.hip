@@ -1,0 +1,222 @@
+// The C ABI (include/espetero_attn.h): argument checks, workspace carving and
+// kernel selection. Nothing here allocates device memory or synchronises.
+#include <cstdarg>
+#include <cstdio>
+#include <cstring>
+
+#include "common.hpp"
+
+namespace esp {
+hipError_t launch_stream(int dt, int HD, int NC, const KArgs& a, int n_tiles, hipStream_t st);
+hipError_t launch_combine(int dt, int HD, const KArgs& a, const esp_combine* jobs, int n_jobs, hipStream_t st);
+hipError_t launch_tiled(int dt, int HD, const KArgs& a, int n_tiles, hipStream_t st);
+hipError_t launch_kv_save(const esp_attn_params* p, const void* Kb, const void* Vb, void* pool, const esp_kvsave* e, int n,
+                          hipStream_t st);
+hipError_t launch_kv_copy_blocks(const esp_attn_params* p, void* pool, const int32_t* pairs, int n_pairs, int n_layers,
+                                 uint64_t region_elems, hipStream_t st);
+hipError_t launch_kv_gather(const esp_attn_params* p, const void* pool, const int32_t* blocks, int n, void* K_out,
+                            void* V_out, hipStream_t st);
+hipError_t launch_kv_relayout(const esp_attn_params* p, const void* src, void* dst, int to_native, int n_blocks,
+                              hipStream_t st);
+hipError_t launch_vt_stage(const esp_attn_params* p, const void* Vb, void* vt, int n_rows, hipStream_t st);
+}  // namespace esp
+
+namespace {
+
+int fail(char* err, size_t errlen, int code, const char* fmt, ...) {
+  if (err && errlen) {
+    va_list ap;
+    va_start(ap, fmt);
+    vsnprintf(err, errlen, fmt, ap);
+    va_end(ap);
+  }
+  return code;
+}
+
+int hip_fail(char* err, size_t errlen, const char* what, hipError_t e) {
+  return fail(err, errlen, ESP_ELAUNCH, "%s: %s", what, hipGetErrorString(e));
+}
+
+// Checks shared by every entry point. Returns 0 or an error code.
+int check_params(const esp_attn_params* p, char* err, size_t errlen) {
+  if (!p) return fail(err, errlen, ESP_EINVAL, "params is NULL");
+  if (p->H <= 0 || p->Hkv <= 0 || p->H % p->Hkv) return fail(err, errlen, ESP_EINVAL, "H=%d Hkv=%d: H must be a positive multiple of Hkv", p->H, p->Hkv);
+  if (p->head_dim != 128 && p->head_dim != 256) return fail(err, errlen, ESP_EUNSUPPORTED, "head_dim %d (128 or 256)", p->head_dim);
+  if (p->dtype != ESP_F16 && p->dtype != ESP_BF16) return fail(err, errlen, ESP_EINVAL, "dtype %d", p->dtype);
+  if (p->bt <= 0 || p->bt % 16) return fail(err, errlen, ESP_EINVAL, "bt %d: tokens per block must be a positive multiple of 16", p->bt);
+  if (p->q_ld < p->H * p->head_dim || p->q_ld % 8) return fail(err, errlen, ESP_EINVAL, "q_ld %d", p->q_ld);
+  if (p->kv_ld < p->Hkv * p->head_dim || p->kv_ld % 8) return fail(err, errlen, ESP_EINVAL, "kv_ld %d", p->kv_ld);
+  if (p->kv_base % 8) return fail(err, errlen, ESP_EINVAL, "kv_base must be a multiple of 8 elements");
+  if (p->window < 0 || p->ring < 0) return fail(err, errlen, ESP_EINVAL, "window / ring negative");
+  return ESP_OK;
+}
+
+// Which kernel family serves rows_per_tile x G packed rows: 0 none, else the
+// streaming kernel's column tiles (1, 2) or -1 for the tiled kernel.
+int family(const esp_attn_params* p) {
+  const int packed = p->rows_per_tile * (p->H / p->Hkv);
+  const int nc = (packed + 15) / 16;
+  if (nc <= 2 && nc * p->head_dim <= 256) return nc;
+  return -1;
+}
+
+struct Carve {
+  size_t parts_o, parts_ml, vt_stage, total;
+};
+Carve carve(const esp_attn_params* p, int n_rows, int n_parts) {
+  const size_t cols = size_t(p->rows_per_tile) * size_t(p->H / p->Hkv);
+  const size_t recs = size_t(n_parts > 0 ? n_parts : 0) * p->Hkv * cols;
+  auto up = [](size_t x) { return (x + 255) & ~size_t(255); };
+  Carve c;
+  c.parts_o = 0;
+  c.parts_ml = up(recs * p->head_dim * sizeof(float));
+  c.vt_stage = c.parts_ml + up(recs * 2 * sizeof(float));
+  const size_t groups = size_t(n_rows > 0 ? (n_rows + 15) / 16 : 0);
+  c.total = c.vt_stage + (family(p) < 0 ? up(groups * 16 * p->Hkv * p->head_dim * sizeof(uint16_t)) : 0);
+  if (c.total == 0) c.total = 256;
+  return c;
+}
+
+}  // namespace
+
+extern "C" {
+
+int esp_attn_abi_version(void) { return ESP_ABI_VERSION; }
+
+int esp_attn_init(int device, char* err, size_t errlen) {
+  hipDeviceProp_t prop;
+  hipError_t e = hipGetDeviceProperties(&prop, device);
+  if (e != hipSuccess) return hip_fail(err, errlen, "hipGetDeviceProperties", e);
+  if (strncmp(prop.gcnArchName, "gfx950", 6) != 0)
+    return fail(err, errlen, ESP_EUNSUPPORTED, "device %d is %s; this library is built for gfx950 only", device, prop.gcnArchName);
+  return ESP_OK;
+}
+
+size_t esp_attn_workspace_bytes(const esp_attn_params* p, int32_t n_rows, int32_t n_parts) {
+  if (!p || p->Hkv <= 0 || p->H <= 0 || p->rows_per_tile <= 0) return 0;
+  return carve(p, n_rows, n_parts).total;
+}
+
+int esp_attn_forward(const esp_attn_params* p, const void* Q, const void* Kb, const void* Vb, const void* kv_pool,
+                     const int32_t* blocks, const int32_t* desc, const int32_t* pos, void* O, const esp_tile* tiles,
+                     int32_t n_tiles, const esp_tree* trees, int32_t n_trees, const esp_combine* jobs, int32_t n_jobs,
+                     int32_t n_parts, int32_t n_rows, void* workspace, size_t workspace_bytes, void* stream, char* err,
+                     size_t errlen) {
+  if (int rc = check_params(p, err, errlen)) return rc;
+  if (n_tiles < 0 || n_trees < 0 || n_jobs < 0 || n_parts < 0 || n_rows < 0) return fail(err, errlen, ESP_EINVAL, "negative count");
+  if (n_tiles == 0) return ESP_OK;
+  if (!Q || !Kb || !Vb || !O || !tiles || !trees) return fail(err, errlen, ESP_EINVAL, "Q, Kb, Vb, O, tiles, trees must not be NULL");
+  if (!kv_pool) return fail(err, errlen, ESP_EINVAL, "kv_pool is NULL");
+  if (!p->ring && !blocks) return fail(err, errlen, ESP_EINVAL, "blocks is NULL on a layer without rings");
+  if (p->window > 0 && !pos) return fail(err, errlen, ESP_EINVAL, "pos is NULL on a sliding-window layer");
+  if (p->rows_per_tile <= 0) return fail(err, errlen, ESP_EINVAL, "rows_per_tile %d", p->rows_per_tile);
+  if (n_jobs > 0 && !jobs) return fail(err, errlen, ESP_EINVAL, "jobs is NULL");
+  if ((n_jobs > 0) != (n_parts > 0)) return fail(err, errlen, ESP_EINVAL, "n_jobs %d and n_parts %d disagree", n_jobs, n_parts);
+  if (!(p->scale > 0.0f)) return fail(err, errlen, ESP_EINVAL, "scale must be positive");
+  const int fam = family(p);
+  if (fam < 0 && p->rows_per_tile > 128)
+    return fail(err, errlen, ESP_EUNSUPPORTED, "rows_per_tile %d: the tiled kernel takes at most 128 rows per tile", p->rows_per_tile);
+  const Carve c = carve(p, n_rows, n_parts);
+  if (!workspace || workspace_bytes < c.total)
+    return fail(err, errlen, ESP_EWORKSPACE, "workspace %zu bytes, %zu needed", workspace_bytes, c.total);
+  if (reinterpret_cast<uintptr_t>(workspace) % 16) return fail(err, errlen, ESP_EINVAL, "workspace must be 16-byte aligned");
+
+  hipStream_t st = static_cast<hipStream_t>(stream);
+  char* ws = static_cast<char*>(workspace);
+  esp::KArgs a{};
+  a.Q = static_cast<const uint16_t*>(Q);
+  a.Kb = static_cast<const uint16_t*>(Kb);
+  a.Vb = static_cast<const uint16_t*>(Vb);
+  a.pool = static_cast<const uint16_t*>(kv_pool);
+  a.blocks = blocks;
+  a.desc = reinterpret_cast<const int4*>(desc);
+  a.pos = reinterpret_cast<const int4*>(pos);
+  a.O = static_cast<uint16_t*>(O);
+  a.tiles = tiles;
+  a.trees = trees;
+  a.parts_o = reinterpret_cast<float*>(ws + c.parts_o);
+  a.parts_ml = reinterpret_cast<float*>(ws + c.parts_ml);
+  a.vt_stage = reinterpret_cast<uint16_t*>(ws + c.vt_stage);
+  a.gate = p->gate;
+  a.gate_ld = p->gate_ld;
+  a.gate_hs = p->gate_hs;
+  a.gate_off = p->gate_off;
+  a.H = p->H;
+  a.Hkv = p->Hkv;
+  a.G = p->H / p->Hkv;
+  a.q_ld = p->q_ld;
+  a.kv_ld = p->kv_ld;
+  a.bt = p->bt;
+  a.window = p->window;
+  a.ring = p->ring;
+  a.bidi = p->bidi;
+  a.R = p->rows_per_tile;
+  a.cols = a.R * a.G;
+  a.n_rows = n_rows;
+  a.scale_log2 = p->scale * esp::kLog2e;
+  a.kv_base = p->kv_base;
+
+  hipError_t e;
+  if (fam > 0) {
+    e = esp::launch_stream(p->dtype, p->head_dim, fam, a, n_tiles, st);
+    if (e != hipSuccess) return hip_fail(err, errlen, "attn_stream launch", e);
+  } else {
+    if (n_rows > 0) {
+      e = esp::launch_vt_stage(p, Vb, a.vt_stage, n_rows, st);
+      if (e != hipSuccess) return hip_fail(err, errlen, "vt_stage launch", e);
+    }
+    e = esp::launch_tiled(p->dtype, p->head_dim, a, n_tiles, st);
+    if (e != hipSuccess) return hip_fail(err, errlen, "attn_tiled launch", e);
+  }
+  if (n_jobs > 0) {
+    e = esp::launch_combine(p->dtype, p->head_dim, a, jobs, n_jobs, st);
+    if (e != hipSuccess) return hip_fail(err, errlen, "attn_combine launch", e);
+  }
+  return ESP_OK;
+}
+
+int esp_kv_save(const esp_attn_params* p, const void* Kb, const void* Vb, void* kv_pool, const esp_kvsave* entries,
+                int32_t n_entries, void* stream, char* err, size_t errlen) {
+  if (int rc = check_params(p, err, errlen)) return rc;
+  if (n_entries < 0) return fail(err, errlen, ESP_EINVAL, "n_entries negative");
+  if (n_entries == 0) return ESP_OK;
+  if (!Kb || !Vb || !kv_pool || !entries) return fail(err, errlen, ESP_EINVAL, "NULL argument");
+  hipError_t e = esp::launch_kv_save(p, Kb, Vb, kv_pool, entries, n_entries, static_cast<hipStream_t>(stream));
+  return e == hipSuccess ? ESP_OK : hip_fail(err, errlen, "kv_save launch", e);
+}
+
+int esp_kv_copy_blocks(const esp_attn_params* p, void* kv_pool, const int32_t* pairs, int32_t n_pairs, int32_t n_layers,
+                       uint64_t region_elems, void* stream, char* err, size_t errlen) {
+  if (int rc = check_params(p, err, errlen)) return rc;
+  if (n_pairs < 0 || n_layers < 0) return fail(err, errlen, ESP_EINVAL, "negative count");
+  if (n_pairs == 0 || n_layers == 0) return ESP_OK;
+  if (!kv_pool || !pairs) return fail(err, errlen, ESP_EINVAL, "NULL argument");
+  if (region_elems % 8) return fail(err, errlen, ESP_EINVAL, "region_elems must be a multiple of 8");
+  hipError_t e = esp::launch_kv_copy_blocks(p, kv_pool, pairs, n_pairs, n_layers, region_elems, static_cast<hipStream_t>(stream));
+  return e == hipSuccess ? ESP_OK : hip_fail(err, errlen, "kv_copy_blocks launch", e);
+}
+
+int esp_kv_gather(const esp_attn_params* p, const void* kv_pool, const int32_t* blocks, int32_t n_tokens, void* K_out,
+                  void* V_out, void* stream, char* err, size_t errlen) {
+  if (int rc = check_params(p, err, errlen)) return rc;
+  if (n_tokens < 0) return fail(err, errlen, ESP_EINVAL, "n_tokens negative");
+  if (n_tokens == 0) return ESP_OK;
+  if (!kv_pool || !blocks || !K_out || !V_out) return fail(err, errlen, ESP_EINVAL, "NULL argument");
+  hipError_t e = esp::launch_kv_gather(p, kv_pool, blocks, n_tokens, K_out, V_out, static_cast<hipStream_t>(stream));
+  return e == hipSuccess ? ESP_OK : hip_fail(err, errlen, "kv_gather launch", e);
+}
+
+int esp_kv_relayout(const esp_attn_params* p, const void* src_pool, int32_t src_layout, void* dst_pool, int32_t dst_layout,
+                    int32_t n_blocks, void* stream, char* err, size_t errlen) {
+  if (int rc = check_params(p, err, errlen)) return rc;
+  if (n_blocks < 0) return fail(err, errlen, ESP_EINVAL, "n_blocks negative");
+  if (!((src_layout == ESP_LAYOUT_REFERENCE && dst_layout == ESP_LAYOUT_NATIVE) ||
+        (src_layout == ESP_LAYOUT_NATIVE && dst_layout == ESP_LAYOUT_REFERENCE)))
+    return fail(err, errlen, ESP_EINVAL, "layouts %d -> %d: one side reference, the other native", src_layout, dst_layout);
+  if (n_blocks == 0) return ESP_OK;
+  if (!src_pool || !dst_pool) return fail(err, errlen, ESP_EINVAL, "NULL argument");
+  hipError_t e = esp::launch_kv_relayout(p, src_pool, dst_pool, dst_layout == ESP_LAYOUT_NATIVE, n_blocks, static_cast<hipStream_t>(stream));
+  return e == hipSuccess ? ESP_OK : hip_fail(err, errlen, "kv_relayout launch", e);
+}
+
+}  // extern "C"

@@ -1,0 +1,454 @@
+// Split-K streaming attention for passes with few query rows per tree: decode
+// (one row) and speculative verify (a handful of rows). Bandwidth bound: the
+// job of this kernel is to keep KV pages in flight.
+//
+// Semantics: the reference's single-row decode kernels and its 8-row tiles on
+// small trees (kernels/40_attention.metal:597-781, kernels/80_gemma.metal:157-342,
+// :371-550): cached keys [k0, k1) through the block table (or ring), the batch
+// keys of the tree on the `last` tile with the tree mask and the window, online
+// softmax in fp32 with P rounded to the storage type before P.V, a partial
+// record (O unnormalised, m, l) or the normalised (optionally gated) output.
+//
+// Mapping to gfx950. One workgroup = one tile x one KV head, 4 wavefronts. The
+// G query heads of the KV head times the tile's rows are packed into the 16 (or
+// 32) columns of the MFMA tiles ("packed rows": col = row_in_tile * G + head),
+// so K and V are read from HBM once for all of them. Per 32 keys a wavefront
+//   S^T[32 keys][cols]  = K[32][HD] . Q^T          v_mfma_f32_16x16x32 (A = K straight from HBM, 16-byte loads)
+//   P^T = exp2(S^T - m) rounded to fp16 / bf16    (D layout of S^T == B layout of P^T: no shuffles)
+//   O^T[HD][cols]      += V^T[HD][32] . P^T        v_mfma_f32_16x16x32 (A = V^T straight from HBM: the pool keeps V transposed)
+// with no LDS on the way. The 4 wavefronts take 32-key units round robin and
+// merge their (m, l, O) through LDS in wave order at the end. Loads for the
+// next unit are issued before the current unit's math (two register sets).
+#include "common.hpp"
+
+namespace esp {
+
+template <int HD, int SBU>
+struct Unit {  // operands of one unit of SBU 16-key sub-blocks
+  u32x4 k[SBU][HD / 32];  // [sub-block][32-dim group]: key = lane % 16, dims 32 kk + 8 (lane / 16) ..
+  u32x2 v[SBU][HD / 16];  // [sub-block][16-dim group]: dim = 16 mt + lane % 16, keys 4 (lane / 16) ..
+};
+
+// SBU: 16-key sub-blocks per unit (2: P.V on 16x16x32 tiles; 1: on 16x16x16 tiles, for
+// head dims whose operands would not fit two register sets otherwise).
+template <int DT, int HD, int NC, int SBU, int OCC>
+__global__ __launch_bounds__(256, OCC) void attn_stream_kernel(const KArgs a) {
+  constexpr int KK = HD / 32, MT = HD / 16, LDO = HD + 4, UK = 16 * SBU, USH = SBU == 2 ? 5 : 4;
+  extern __shared__ float smem[];  // [4 waves][NC * 16 cols][LDO] O, then [4][NC * 16][2] m, l
+
+  const int kvh = blockIdx.x;
+  const int lane = threadIdx.x & 63;
+  const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+  const int c16 = lane & 15, q4 = lane >> 4;
+  const esp_tile tile = a.tiles[blockIdx.y];
+  const esp_tree tree = a.trees[tile.tree];
+  const int end = tree.base + tree.M;
+  const int rows_live = min(a.R, end - tile.r0);
+  const int rr0 = tile.r0 - tree.base;
+
+  // ---- this lane's packed rows: Q fragments, position, descriptor
+  u32x4 qf[NC][KK];
+  int rr[NC], qpos[NC];
+  int4 dsc[NC];
+  bool ok[NC];
+#pragma unroll
+  for (int c = 0; c < NC; ++c) {
+    const int col = 16 * c + c16;
+    const int m = col / a.G, hg = col - m * a.G;
+    ok[c] = col < a.cols && m < rows_live;
+    rr[c] = rr0 + m;
+    const int row = ok[c] ? tile.r0 + m : tile.r0;
+    qpos[c] = (a.window > 0) ? a.pos[row].x : 0;
+    dsc[c] = a.desc ? a.desc[row] : make_int4(0, 0, 0, 0);
+    const uint16_t* qp = a.Q + size_t(row) * a.q_ld + size_t(kvh * a.G + (ok[c] ? hg : 0)) * HD + 8 * q4;
+#pragma unroll
+    for (int kk = 0; kk < KK; ++kk)
+      qf[c][kk] = ok[c] ? *reinterpret_cast<const u32x4*>(qp + 32 * kk) : u32x4{0, 0, 0, 0};
+  }
+
+  // ---- units of UK keys: the cached range, then the tree's batch rows
+  const int cp0 = tile.k0 >> USH;
+  const int n_cached = tile.k1 > tile.k0 ? ((tile.k1 + UK - 1) >> USH) - cp0 : 0;
+  int k_last = -1, bp0 = 0, n_batch = 0;
+  if (tile.last) {
+    // Last batch key any row of the tile sees: its last row, a root it sees whole
+    // (anc_len), the end of its image (bidi).
+    int kl = -1;
+#pragma unroll
+    for (int c = 0; c < NC; ++c)
+      if (ok[c]) kl = max(kl, max(rr[c], max(dsc[c].z - 1, a.bidi ? dsc[c].w - 1 : -1)));
+#pragma unroll
+    for (int o = 32; o >= 1; o >>= 1) kl = max(kl, __shfl_xor(kl, o));
+    k_last = __builtin_amdgcn_readfirstlane(min(kl, tree.M - 1));
+    bp0 = tile.b0 >> USH;
+    n_batch = max(0, ((k_last + UK) >> USH) - bp0);
+  }
+  const int n_units = n_cached + n_batch;
+
+  f32x4 acc[NC][MT];
+  float m_run[NC], l_run[NC];
+#pragma unroll
+  for (int c = 0; c < NC; ++c) {
+    m_run[c] = -INFINITY;
+    l_run[c] = 0.0f;
+#pragma unroll
+    for (int mt = 0; mt < MT; ++mt) acc[c][mt] = f32x4{0, 0, 0, 0};
+  }
+
+  // Cached units: K rows and V^T rows straight from the pool.
+  auto load_cached = [&](int u, Unit<HD, SBU>& U) {
+    const int j0 = (cp0 + u) << USH;
+#pragma unroll
+    for (int sb = 0; sb < SBU; ++sb) {
+      const int js = j0 + 16 * sb;  // first key of the sub-block
+      // A sub-block wholly outside the range is not read (its page may not exist).
+      const bool live = js < tile.k1 && js + 16 > tile.k0;
+      if (live) {
+        const int b = block_of(a, tree.table, js);
+        const uint16_t* hb = a.pool + head_base(a, HD, b, kvh);
+        const int t0 = js % a.bt;
+        const uint16_t* kp = hb + size_t(t0 + c16) * HD + 8 * q4;
+        const uint16_t* vp = hb + size_t(a.bt) * HD + size_t(c16) * a.bt + t0 + 4 * q4;
+#pragma unroll
+        for (int kk = 0; kk < KK; ++kk) U.k[sb][kk] = *reinterpret_cast<const u32x4*>(kp + 32 * kk);
+#pragma unroll
+        for (int mt = 0; mt < MT; ++mt) U.v[sb][mt] = *reinterpret_cast<const u32x2*>(vp + size_t(16 * mt) * a.bt);
+      } else {
+#pragma unroll
+        for (int kk = 0; kk < KK; ++kk) U.k[sb][kk] = u32x4{0, 0, 0, 0};
+#pragma unroll
+        for (int mt = 0; mt < MT; ++mt) U.v[sb][mt] = u32x2{0, 0};
+      }
+    }
+  };
+
+  // Batch units: rows of the pass (row major Kb / Vb); V gathered element by element.
+  auto load_batch = [&](int u, Unit<HD, SBU>& U) {
+    const int j0 = (bp0 + (u - n_cached)) << USH;
+#pragma unroll
+    for (int sb = 0; sb < SBU; ++sb) {
+      const int js = j0 + 16 * sb;
+      const int jk = js + c16;
+      const bool k_ok = jk <= k_last;
+      const uint16_t* kp = a.Kb + size_t(tree.base + (k_ok ? jk : 0)) * a.kv_ld + size_t(kvh) * HD + 8 * q4;
+#pragma unroll
+      for (int kk = 0; kk < KK; ++kk)
+        U.k[sb][kk] = k_ok ? *reinterpret_cast<const u32x4*>(kp + 32 * kk) : u32x4{0, 0, 0, 0};
+      const int jv = js + 4 * q4;
+#pragma unroll
+      for (int mt = 0; mt < MT; ++mt) U.v[sb][mt] = u32x2{0, 0};
+#pragma unroll
+      for (int i = 0; i < 4; ++i) {
+        if (jv + i > k_last) continue;
+        const uint16_t* vp = a.Vb + size_t(tree.base + jv + i) * a.kv_ld + size_t(kvh) * HD + c16;
+#pragma unroll
+        for (int mt = 0; mt < MT; ++mt) {
+          const uint32_t e = uint32_t(vp[16 * mt]) << (16 * (i & 1));
+          if (i < 2) U.v[sb][mt].x |= e;
+          else U.v[sb][mt].y |= e;
+        }
+      }
+    }
+  };
+
+  // edge: the unit needs per-key visibility (range ends, window, batch rows).
+  auto compute_unit = [&](int u, Unit<HD, SBU>& U, const bool edge) {
+    const bool cached = u < n_cached;
+    const int j0 = cached ? (cp0 + u) << USH : (bp0 + (u - n_cached)) << USH;
+    if (edge && cached) {
+      // Keys outside [k0, k1) may be memory never written: their V must not reach the products.
+#pragma unroll
+      for (int sb = 0; sb < SBU; ++sb) {
+        const int jv = j0 + 16 * sb + 4 * q4;
+        const uint32_t m0 = (jv >= tile.k0 && jv < tile.k1) ? 0xffffu : 0u;
+        const uint32_t m1 = (jv + 1 >= tile.k0 && jv + 1 < tile.k1) ? 0xffff0000u : 0u;
+        const uint32_t m2 = (jv + 2 >= tile.k0 && jv + 2 < tile.k1) ? 0xffffu : 0u;
+        const uint32_t m3 = (jv + 3 >= tile.k0 && jv + 3 < tile.k1) ? 0xffff0000u : 0u;
+#pragma unroll
+        for (int mt = 0; mt < MT; ++mt) {
+          U.v[sb][mt].x &= (m0 | m1);
+          U.v[sb][mt].y &= (m2 | m3);
+        }
+      }
+    }
+    f32x4 s[NC][SBU];
+#pragma unroll
+    for (int c = 0; c < NC; ++c)
+#pragma unroll
+      for (int sb = 0; sb < SBU; ++sb) {
+        s[c][sb] = f32x4{0, 0, 0, 0};
+#pragma unroll
+        for (int kk = 0; kk < KK; ++kk) s[c][sb] = mfma16x32<DT>(U.k[sb][kk], qf[c][kk], s[c][sb]);
+      }
+    int kpos[SBU][4];
+    if (edge && !cached && a.window > 0) {
+#pragma unroll
+      for (int sb = 0; sb < SBU; ++sb)
+#pragma unroll
+        for (int e = 0; e < 4; ++e) {
+          const int j = j0 + 16 * sb + 4 * q4 + e;
+          kpos[sb][e] = a.pos[tree.base + min(j, tree.M - 1)].x;
+        }
+    }
+    bool any_change = false;
+    u32x2 pb[NC][SBU];
+    float corr[NC];
+#pragma unroll
+    for (int c = 0; c < NC; ++c) {
+      float mx = -INFINITY;
+#pragma unroll
+      for (int sb = 0; sb < SBU; ++sb)
+#pragma unroll
+        for (int e = 0; e < 4; ++e) {
+          float x = s[c][sb][e] * a.scale_log2;
+          if (edge) {
+            const int j = j0 + 16 * sb + 4 * q4 + e;
+            bool vis;
+            if (cached) {
+              vis = j >= tile.k0 && j < tile.k1;
+              if (a.window > 0) vis = vis && (qpos[c] - j < a.window);
+            } else {
+              vis = j <= k_last && ((j < dsc[c].z) || (j >= dsc[c].x && (j <= rr[c] || (a.bidi && j < dsc[c].w))));
+              if (a.window > 0) vis = vis && (qpos[c] - kpos[sb][e] < a.window);
+            }
+            x = vis ? x : -INFINITY;
+          }
+          s[c][sb][e] = x;
+          mx = fmaxf(mx, x);
+        }
+      mx = fmaxf(mx, __shfl_xor(mx, 16));
+      mx = fmaxf(mx, __shfl_xor(mx, 32));
+      const float m_new = fmaxf(m_run[c], mx);
+      const float m_safe = (m_new == -INFINITY) ? 0.0f : m_new;
+      corr[c] = fast_exp2(m_run[c] - m_safe);  // -inf -> 0: nothing accumulated yet
+      any_change = any_change || (m_new > m_run[c]);
+      m_run[c] = m_new;
+      float ps = 0.0f;
+#pragma unroll
+      for (int sb = 0; sb < SBU; ++sb) {
+        float p[4];
+#pragma unroll
+        for (int e = 0; e < 4; ++e) {
+          p[e] = fast_exp2(s[c][sb][e] - m_safe);
+          ps += p[e];
+        }
+        pb[c][sb] = u32x2{pack2<DT>(p[0], p[1]), pack2<DT>(p[2], p[3])};
+      }
+      l_run[c] = l_run[c] * corr[c] + ps;
+    }
+    if (__any(any_change)) {
+#pragma unroll
+      for (int c = 0; c < NC; ++c)
+#pragma unroll
+        for (int mt = 0; mt < MT; ++mt) acc[c][mt] *= corr[c];
+    }
+#pragma unroll
+    for (int mt = 0; mt < MT; ++mt) {
+      if constexpr (SBU == 2) {
+        const u32x4 va = {U.v[0][mt].x, U.v[0][mt].y, U.v[1][mt].x, U.v[1][mt].y};
+#pragma unroll
+        for (int c = 0; c < NC; ++c)
+          acc[c][mt] = mfma16x32<DT>(va, u32x4{pb[c][0].x, pb[c][0].y, pb[c][1].x, pb[c][1].y}, acc[c][mt]);
+      } else {
+#pragma unroll
+        for (int c = 0; c < NC; ++c) acc[c][mt] = mfma16x16<DT>(U.v[0][mt], pb[c][0], acc[c][mt]);
+      }
+    }
+  };
+  // Interior cached units of an unwindowed layer see every key.
+  auto is_edge = [&](int u) {
+    const int j0 = (cp0 + u) << USH;
+    return a.window > 0 || j0 < tile.k0 || j0 + UK > tile.k1;
+  };
+
+  // ---- stream the cached range: two register sets, the next unit's loads in
+  // flight during the math. Wavefront w takes units w, w + 4, ...
+  {
+    Unit<HD, SBU> A, B;
+    int u = wave;
+    if (u < n_cached) load_cached(u, A);
+    for (; u < n_cached; u += 8) {
+      if (u + 4 < n_cached) load_cached(u + 4, B);
+      if (is_edge(u)) compute_unit(u, A, true);
+      else compute_unit(u, A, false);
+      if (u + 4 < n_cached) {
+        if (u + 8 < n_cached) load_cached(u + 8, A);
+        if (is_edge(u + 4)) compute_unit(u + 4, B, true);
+        else compute_unit(u + 4, B, false);
+      }
+    }
+    // ---- then the batch rows (few: this kernel serves short trees)
+    for (u = n_cached + ((wave + 4 - (n_cached & 3)) & 3); u < n_units; u += 4) {
+      load_batch(u, A);
+      compute_unit(u, A, true);
+    }
+  }
+
+  // ---- merge the 4 wavefronts in wave order
+  float* o_sh = smem;                          // [4][NC * 16][LDO]
+  float* ml_sh = smem + 4 * NC * 16 * LDO;     // [4][NC * 16][2]
+#pragma unroll
+  for (int c = 0; c < NC; ++c) {
+    float l = l_run[c];
+    l += __shfl_xor(l, 16);
+    l += __shfl_xor(l, 32);
+    l_run[c] = l;
+    if (q4 == 0) {
+      ml_sh[(wave * NC * 16 + 16 * c + c16) * 2] = m_run[c];
+      ml_sh[(wave * NC * 16 + 16 * c + c16) * 2 + 1] = l;
+    }
+  }
+  __syncthreads();
+#pragma unroll
+  for (int c = 0; c < NC; ++c) {
+    const int col = 16 * c + c16;
+    float M = -INFINITY;
+#pragma unroll
+    for (int w = 0; w < 4; ++w) M = fmaxf(M, ml_sh[(w * NC * 16 + col) * 2]);
+    const float f = (m_run[c] == -INFINITY) ? 0.0f : fast_exp2(m_run[c] - M);
+    float* dst = o_sh + size_t(wave * NC * 16 + col) * LDO + 4 * q4;
+#pragma unroll
+    for (int mt = 0; mt < MT; ++mt) *reinterpret_cast<f32x4*>(dst + 16 * mt) = acc[c][mt] * f;
+  }
+  __syncthreads();
+  // Each thread finishes 4 dims of one packed row at a time.
+  for (int i = threadIdx.x; i < NC * 16 * (HD / 4); i += 256) {
+    const int col = i / (HD / 4), d = (i % (HD / 4)) * 4;
+    const int m = col / a.G, hg = col - m * a.G;
+    if (col >= a.cols || m >= rows_live) continue;
+    float M = -INFINITY;
+#pragma unroll
+    for (int w = 0; w < 4; ++w) M = fmaxf(M, ml_sh[(w * NC * 16 + col) * 2]);
+    float L = 0.0f;
+    f32x4 o = {0, 0, 0, 0};
+#pragma unroll
+    for (int w = 0; w < 4; ++w) {
+      const float mw = ml_sh[(w * NC * 16 + col) * 2];
+      const float f = (mw == -INFINITY) ? 0.0f : fast_exp2(mw - M);
+      L += f * ml_sh[(w * NC * 16 + col) * 2 + 1];
+      o += *reinterpret_cast<const f32x4*>(o_sh + size_t(w * NC * 16 + col) * LDO + d);
+    }
+    if (tile.part >= 0) {
+      const size_t rec = (size_t(tile.part) * a.Hkv + kvh) * a.cols + col;
+      *reinterpret_cast<f32x4*>(a.parts_o + rec * HD + d) = o;
+      if (d == 0) {
+        a.parts_ml[rec * 2] = M;
+        a.parts_ml[rec * 2 + 1] = L;
+      }
+    } else {
+      const int row = tile.r0 + m, h = kvh * a.G + hg;
+      const float inv = L > 0.0f ? 1.0f / L : 0.0f;
+      o *= inv;
+      if (a.gate) {
+        const float* g = a.gate + size_t(row) * a.gate_ld + size_t(h) * a.gate_hs + a.gate_off + d;
+#pragma unroll
+        for (int e = 0; e < 4; ++e) o[e] = o[e] / (1.0f + __expf(-g[e]));
+      }
+      u32x2 out = {pack2<DT>(o[0], o[1]), pack2<DT>(o[2], o[3])};
+      *reinterpret_cast<u32x2*>(a.O + size_t(row) * a.q_ld + size_t(h) * HD + d) = out;
+    }
+  }
+}
+
+// Merge the split partial records of a tile group in part order
+// (attention_combine, kernels/40_attention.metal:811-864): one thread per
+// (job, row, head, 4 dims).
+template <int DT, int HD>
+__global__ __launch_bounds__(256) void attn_combine_kernel(const KArgs a, const esp_combine* jobs, int n_jobs) {
+  const int per_job = a.R * a.H * (HD / 4);
+  const long gid = long(blockIdx.x) * 256 + threadIdx.x;
+  if (gid >= long(n_jobs) * per_job) return;
+  const int ji = int(gid / per_job);
+  int rem = int(gid % per_job);
+  const int r = rem / (a.H * (HD / 4));
+  rem -= r * a.H * (HD / 4);
+  const int h = rem / (HD / 4), d = (rem % (HD / 4)) * 4;
+  const esp_combine job = jobs[ji];
+  if (r >= job.rows) return;
+  const int kvh = h / a.G, hg = h - kvh * a.G;
+  const int col = r * a.G + hg;
+  const size_t stride = size_t(a.Hkv) * a.cols;  // records from one part to the next
+  const size_t rec0 = (size_t(job.part0) * a.Hkv + kvh) * a.cols + col;
+  float M = -INFINITY;
+  for (int s = 0; s < job.nparts; ++s) M = fmaxf(M, a.parts_ml[(rec0 + s * stride) * 2]);
+  float L = 0.0f;
+  f32x4 o = {0, 0, 0, 0};
+  int s = 0;
+  for (; s + 4 <= job.nparts; s += 4) {  // 4 records in flight, summed in order
+    float m4[4], l4[4];
+    f32x4 o4[4];
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+      const size_t rec = rec0 + size_t(s + i) * stride;
+      m4[i] = a.parts_ml[rec * 2];
+      l4[i] = a.parts_ml[rec * 2 + 1];
+      o4[i] = *reinterpret_cast<const f32x4*>(a.parts_o + rec * HD + d);
+    }
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+      const float w = (m4[i] == -INFINITY) ? 0.0f : fast_exp2(m4[i] - M);
+      L += w * l4[i];
+      o += o4[i] * w;
+    }
+  }
+  for (; s < job.nparts; ++s) {
+    const size_t rec = rec0 + size_t(s) * stride;
+    const float ms = a.parts_ml[rec * 2];
+    const float w = (ms == -INFINITY) ? 0.0f : fast_exp2(ms - M);
+    L += w * a.parts_ml[rec * 2 + 1];
+    o += *reinterpret_cast<const f32x4*>(a.parts_o + rec * HD + d) * w;
+  }
+  const int row = job.r0 + r;
+  const float inv = L > 0.0f ? 1.0f / L : 0.0f;
+  o *= inv;
+  if (a.gate) {
+    const float* g = a.gate + size_t(row) * a.gate_ld + size_t(h) * a.gate_hs + a.gate_off + d;
+#pragma unroll
+    for (int e = 0; e < 4; ++e) o[e] = o[e] / (1.0f + __expf(-g[e]));
+  }
+  u32x2 out = {pack2<DT>(o[0], o[1]), pack2<DT>(o[2], o[3])};
+  *reinterpret_cast<u32x2*>(a.O + size_t(row) * a.q_ld + size_t(h) * HD + d) = out;
+}
+
+size_t stream_smem_bytes(int HD, int NC) { return size_t(4 * NC * 16) * (HD + 4 + 2) * sizeof(float); }
+
+template <int DT, int HD, int NC>
+static hipError_t launch_stream_t(const KArgs& a, int n_tiles, hipStream_t st) {
+  constexpr int SBU = HD == 128 ? 2 : 1;
+  constexpr int OCC = (HD == 128 && NC == 1) ? 2 : 1;
+  const size_t smem = stream_smem_bytes(HD, NC);
+  auto k = attn_stream_kernel<DT, HD, NC, SBU, OCC>;
+  if (smem > 48 * 1024) {
+    hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(k), hipFuncAttributeMaxDynamicSharedMemorySize, int(smem));
+    if (e != hipSuccess) return e;
+  }
+  hipLaunchKernelGGL(k, dim3(a.Hkv, n_tiles), dim3(256), smem, st, a);
+  return hipGetLastError();
+}
+
+// dt, HD, NC are validated by the caller: HD in {128, 256}, NC in {1, 2}, NC * HD <= 256.
+hipError_t launch_stream(int dt, int HD, int NC, const KArgs& a, int n_tiles, hipStream_t st) {
+  if (dt == ESP_F16) {
+    if (HD == 128 && NC == 1) return launch_stream_t<ESP_F16, 128, 1>(a, n_tiles, st);
+    if (HD == 128 && NC == 2) return launch_stream_t<ESP_F16, 128, 2>(a, n_tiles, st);
+    if (HD == 256 && NC == 1) return launch_stream_t<ESP_F16, 256, 1>(a, n_tiles, st);
+  } else {
+    if (HD == 128 && NC == 1) return launch_stream_t<ESP_BF16, 128, 1>(a, n_tiles, st);
+    if (HD == 128 && NC == 2) return launch_stream_t<ESP_BF16, 128, 2>(a, n_tiles, st);
+    if (HD == 256 && NC == 1) return launch_stream_t<ESP_BF16, 256, 1>(a, n_tiles, st);
+  }
+  return hipErrorInvalidValue;
+}
+
+hipError_t launch_combine(int dt, int HD, const KArgs& a, const esp_combine* jobs, int n_jobs, hipStream_t st) {
+  const long n = long(n_jobs) * a.R * a.H * (HD / 4);
+  const dim3 grid((unsigned)((n + 255) / 256));
+  if (dt == ESP_F16 && HD == 128) hipLaunchKernelGGL((attn_combine_kernel<ESP_F16, 128>), grid, dim3(256), 0, st, a, jobs, n_jobs);
+  else if (dt == ESP_F16 && HD == 256) hipLaunchKernelGGL((attn_combine_kernel<ESP_F16, 256>), grid, dim3(256), 0, st, a, jobs, n_jobs);
+  else if (dt == ESP_BF16 && HD == 128) hipLaunchKernelGGL((attn_combine_kernel<ESP_BF16, 128>), grid, dim3(256), 0, st, a, jobs, n_jobs);
+  else if (dt == ESP_BF16 && HD == 256) hipLaunchKernelGGL((attn_combine_kernel<ESP_BF16, 256>), grid, dim3(256), 0, st, a, jobs, n_jobs);
+  else return hipErrorInvalidValue;
+  return hipGetLastError();
+}
+
+}  // namespace esp

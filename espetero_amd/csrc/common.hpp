@@ -1,0 +1,117 @@
+// Shared device helpers of the gfx950 attention kernels: vector types, MFMA
+// wrappers for fp16 / bf16 operands, storage conversions, the native KV pool
+// addressing and the kernel argument block.
+#pragma once
+
+#include <hip/hip_runtime.h>
+#include <stdint.h>
+
+#include "../../include/espetero_attn.h"
+
+namespace esp {
+
+using f32x4 = float __attribute__((ext_vector_type(4)));
+using f32x16 = float __attribute__((ext_vector_type(16)));
+using f16x8 = _Float16 __attribute__((ext_vector_type(8)));
+using f16x4 = _Float16 __attribute__((ext_vector_type(4)));
+using f16x2 = _Float16 __attribute__((ext_vector_type(2)));
+using i16x4 = short __attribute__((ext_vector_type(4)));
+using bf16x8 = __bf16 __attribute__((ext_vector_type(8)));
+using bf16x2 = __bf16 __attribute__((ext_vector_type(2)));
+using u32x4 = uint32_t __attribute__((ext_vector_type(4)));
+using u32x2 = uint32_t __attribute__((ext_vector_type(2)));
+
+constexpr float kLog2e = 1.4426950408889634f;
+
+// D(16x16) += A(16x32) * B(32x16). Lane l holds A[l % 16][8 (l / 16) .. + 7],
+// B[8 (l / 16) .. + 7][l % 16] and D[4 (l / 16) .. + 3][l % 16].
+template <int DT>
+__device__ __forceinline__ f32x4 mfma16x32(u32x4 a, u32x4 b, f32x4 c) {
+  if constexpr (DT == ESP_F16) {
+    return __builtin_amdgcn_mfma_f32_16x16x32_f16(__builtin_bit_cast(f16x8, a), __builtin_bit_cast(f16x8, b), c, 0, 0, 0);
+  } else {
+    return __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(bf16x8, a), __builtin_bit_cast(bf16x8, b), c, 0, 0, 0);
+  }
+}
+
+// D(16x16) += A(16x16) * B(16x16). Lane l holds A[l % 16][4 (l / 16) .. + 3],
+// B[4 (l / 16) .. + 3][l % 16] and D[4 (l / 16) .. + 3][l % 16].
+template <int DT>
+__device__ __forceinline__ f32x4 mfma16x16(u32x2 a, u32x2 b, f32x4 c) {
+  if constexpr (DT == ESP_F16) {
+    return __builtin_amdgcn_mfma_f32_16x16x16f16(__builtin_bit_cast(f16x4, a), __builtin_bit_cast(f16x4, b), c, 0, 0, 0);
+  } else {
+    return __builtin_amdgcn_mfma_f32_16x16x16bf16_1k(__builtin_bit_cast(i16x4, a), __builtin_bit_cast(i16x4, b), c, 0, 0, 0);
+  }
+}
+
+// D(32x32) += A(32x16) * B(16x32). Lane l holds A[l % 32][8 (l / 32) .. + 7],
+// B[8 (l / 32) .. + 7][l % 32] and D[8 i + 4 (l / 32) + j][l % 32] at index 4 i + j.
+template <int DT>
+__device__ __forceinline__ f32x16 mfma32x16(u32x4 a, u32x4 b, f32x16 c) {
+  if constexpr (DT == ESP_F16) {
+    return __builtin_amdgcn_mfma_f32_32x32x16_f16(__builtin_bit_cast(f16x8, a), __builtin_bit_cast(f16x8, b), c, 0, 0, 0);
+  } else {
+    return __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(bf16x8, a), __builtin_bit_cast(bf16x8, b), c, 0, 0, 0);
+  }
+}
+
+// Two fp32 -> one dword of two storage elements, round to nearest even.
+template <int DT>
+__device__ __forceinline__ uint32_t pack2(float lo, float hi) {
+  if constexpr (DT == ESP_F16) {
+    f16x2 v = {(_Float16)lo, (_Float16)hi};
+    return __builtin_bit_cast(uint32_t, v);
+  } else {
+    bf16x2 v = {(__bf16)lo, (__bf16)hi};
+    return __builtin_bit_cast(uint32_t, v);
+  }
+}
+
+template <int DT>
+__device__ __forceinline__ uint16_t pack1(float x) {
+  if constexpr (DT == ESP_F16) {
+    return __builtin_bit_cast(uint16_t, (_Float16)x);
+  } else {
+    return __builtin_bit_cast(uint16_t, (__bf16)x);
+  }
+}
+
+__device__ __forceinline__ float fast_exp2(float x) { return __builtin_amdgcn_exp2f(x); }
+
+// Everything a kernel of this library reads: the call's device pointers and
+// the per-layer constants, passed by value.
+struct KArgs {
+  const uint16_t* Q;
+  const uint16_t* Kb;
+  const uint16_t* Vb;
+  const uint16_t* pool;
+  const int32_t* blocks;
+  const int4* desc;
+  const int4* pos;
+  uint16_t* O;
+  const esp_tile* tiles;
+  const esp_tree* trees;
+  float* parts_o;   // [part][Hkv][cols][HD]   unnormalised O
+  float* parts_ml;  // [part][Hkv][cols][2]    running max (log2 units), sum
+  uint16_t* vt_stage;  // batch V transposed: [Hkv][n_rows16 / 16][HD][16]
+  const float* gate;
+  int32_t gate_ld, gate_hs, gate_off;
+  int32_t H, Hkv, G, q_ld, kv_ld, bt, window, ring, bidi, R, cols, n_rows;
+  float scale_log2;
+  uint64_t kv_base;
+};
+
+// Native pool: element offset of (block b, KV head h); K rows follow at
+// t * HD + d, V transposed at bt * HD + d * bt + t.
+__device__ __forceinline__ size_t head_base(const KArgs& a, int HD, int b, int kvh) {
+  return size_t(a.kv_base) + (size_t(b) * size_t(a.Hkv) + size_t(kvh)) * size_t(2 * a.bt * HD);
+}
+
+// Block holding cached key j of a tree: its block list, or its slot's ring.
+__device__ __forceinline__ int block_of(const KArgs& a, int table, int j) {
+  const int bi = j / a.bt;
+  return a.ring ? table + bi % a.ring : a.blocks[table + bi];
+}
+
+}  // namespace esp

@@ -1,0 +1,170 @@
+// Pool maintenance kernels over the native block layout: append rows, copy
+// blocks (copy on write), gather a block list into contiguous rows, convert
+// blocks between the reference's layout and the native one, and stage a
+// pass's batch V rows transposed for the tiled attention kernel. All are bit
+// copies of 16-bit storage elements.
+#include "common.hpp"
+
+namespace esp {
+
+// kv_save (kernels/40_attention.metal:875-889): entry = (source row, block,
+// position). One thread per (entry, 8 elements of the KV row).
+__global__ __launch_bounds__(256) void kv_save_kernel(const uint16_t* Kb, const uint16_t* Vb, uint16_t* pool,
+                                                      const esp_kvsave* entries, int n, int Hkv, int HD, int kv_ld, int bt,
+                                                      uint64_t kv_base) {
+  const int per = Hkv * HD / 8;
+  const long gid = long(blockIdx.x) * 256 + threadIdx.x;
+  if (gid >= long(n) * per) return;
+  const esp_kvsave e = entries[gid / per];
+  const int x = int(gid % per) * 8;
+  const int kvh = x / HD, d = x % HD;
+  const size_t src = size_t(e.src_row) * kv_ld + x;
+  uint16_t* hb = pool + kv_base + (size_t(e.block) * Hkv + kvh) * size_t(2 * bt * HD);
+  *reinterpret_cast<u32x4*>(hb + size_t(e.pos) * HD + d) = *reinterpret_cast<const u32x4*>(Kb + src);
+  const u32x4 v = *reinterpret_cast<const u32x4*>(Vb + src);
+  uint16_t* vt = hb + size_t(bt) * HD + size_t(d) * bt + e.pos;
+#pragma unroll
+  for (int i = 0; i < 4; ++i) {
+    vt[size_t(2 * i) * bt] = uint16_t(v[i] & 0xffffu);
+    vt[size_t(2 * i + 1) * bt] = uint16_t(v[i] >> 16);
+  }
+}
+
+// kv_copy_blocks (40_:894-905): a block is one contiguous run of
+// 2 * bt * Hkv * HD elements in the native layout as well.
+__global__ __launch_bounds__(256) void kv_copy_blocks_kernel(uint16_t* pool, const int2* pairs, uint64_t blk2,
+                                                             uint64_t region_elems) {
+  const uint64_t x = (uint64_t(blockIdx.x) * 256 + threadIdx.x) * 8;
+  if (x >= blk2) return;
+  const int2 pr = pairs[blockIdx.y];
+  uint16_t* base = pool + uint64_t(blockIdx.z) * region_elems;
+  *reinterpret_cast<u32x4*>(base + uint64_t(pr.y) * blk2 + x) = *reinterpret_cast<const u32x4*>(base + uint64_t(pr.x) * blk2 + x);
+}
+
+// Tokens [0, n) of a block list -> K_out / V_out [n][Hkv * HD].
+__global__ __launch_bounds__(256) void kv_gather_kernel(const uint16_t* pool, const int32_t* blocks, int n, uint16_t* K_out,
+                                                        uint16_t* V_out, int Hkv, int HD, int bt, uint64_t kv_base) {
+  const int per = Hkv * HD / 8;
+  const long gid = long(blockIdx.x) * 256 + threadIdx.x;
+  if (gid >= long(n) * per) return;
+  const int j = int(gid / per);
+  const int x = int(gid % per) * 8;
+  const int kvh = x / HD, d = x % HD;
+  const int b = blocks[j / bt], t = j % bt;
+  const uint16_t* hb = pool + kv_base + (size_t(b) * Hkv + kvh) * size_t(2 * bt * HD);
+  *reinterpret_cast<u32x4*>(K_out + size_t(j) * Hkv * HD + x) = *reinterpret_cast<const u32x4*>(hb + size_t(t) * HD + d);
+  const uint16_t* vt = hb + size_t(bt) * HD + size_t(d) * bt + t;
+  u32x4 v;
+#pragma unroll
+  for (int i = 0; i < 4; ++i) v[i] = uint32_t(vt[size_t(2 * i) * bt]) | (uint32_t(vt[size_t(2 * i + 1) * bt]) << 16);
+  *reinterpret_cast<u32x4*>(V_out + size_t(j) * Hkv * HD + x) = v;
+}
+
+// Whole blocks between layouts. Reference block: [K | V][t][h][d] (40_:245-247).
+// One thread per (block, which, t, 8 elements of the row).
+__global__ __launch_bounds__(256) void kv_relayout_kernel(const uint16_t* src, uint16_t* dst, int to_native, int n_blocks,
+                                                          int Hkv, int HD, int bt) {
+  const int w = Hkv * HD;
+  const long per_block = long(2) * bt * (w / 8);
+  const long gid = long(blockIdx.x) * 256 + threadIdx.x;
+  if (gid >= long(n_blocks) * per_block) return;
+  const int b = int(gid / per_block);
+  long rem = gid % per_block;
+  const int which = int(rem / (long(bt) * (w / 8)));
+  rem -= long(which) * bt * (w / 8);
+  const int t = int(rem / (w / 8));
+  const int x = int(rem % (w / 8)) * 8;
+  const int kvh = x / HD, d = x % HD;
+  const size_t ref_off = size_t(b) * 2 * bt * w + (size_t(which) * bt + t) * w + x;
+  const size_t hb = (size_t(b) * Hkv + kvh) * size_t(2 * bt * HD);
+  if (which == 0) {
+    const size_t nat = hb + size_t(t) * HD + d;
+    if (to_native) *reinterpret_cast<u32x4*>(dst + nat) = *reinterpret_cast<const u32x4*>(src + ref_off);
+    else *reinterpret_cast<u32x4*>(dst + ref_off) = *reinterpret_cast<const u32x4*>(src + nat);
+  } else {
+    const size_t nat = hb + size_t(bt) * HD + size_t(d) * bt + t;
+    if (to_native) {
+      const u32x4 v = *reinterpret_cast<const u32x4*>(src + ref_off);
+#pragma unroll
+      for (int i = 0; i < 4; ++i) {
+        dst[nat + size_t(2 * i) * bt] = uint16_t(v[i] & 0xffffu);
+        dst[nat + size_t(2 * i + 1) * bt] = uint16_t(v[i] >> 16);
+      }
+    } else {
+      u32x4 v;
+#pragma unroll
+      for (int i = 0; i < 4; ++i) v[i] = uint32_t(src[nat + size_t(2 * i) * bt]) | (uint32_t(src[nat + size_t(2 * i + 1) * bt]) << 16);
+      *reinterpret_cast<u32x4*>(dst + ref_off) = v;
+    }
+  }
+}
+
+// Batch V rows [n_rows][kv_ld] -> vt_stage [Hkv][n_rows16 / 16][HD][16]
+// (16-row groups, rows past n_rows zero). One workgroup per (16-row group, KV
+// head): the 16 x HD tile is transposed through LDS.
+__global__ __launch_bounds__(256) void vt_stage_kernel(const uint16_t* Vb, uint16_t* vt, int n_rows, int n_groups, int HD,
+                                                       int kv_ld) {
+  __shared__ uint16_t sh[16][256 + 2];
+  const int g = blockIdx.x, kvh = blockIdx.y;
+  for (int i = threadIdx.x; i < 16 * (HD / 8); i += 256) {
+    const int r = i / (HD / 8), x = (i % (HD / 8)) * 8;
+    const int row = 16 * g + r;
+    u32x4 v = {0, 0, 0, 0};
+    if (row < n_rows) v = *reinterpret_cast<const u32x4*>(Vb + size_t(row) * kv_ld + size_t(kvh) * HD + x);
+#pragma unroll
+    for (int e = 0; e < 4; ++e) {
+      sh[r][x + 2 * e] = uint16_t(v[e] & 0xffffu);
+      sh[r][x + 2 * e + 1] = uint16_t(v[e] >> 16);
+    }
+  }
+  __syncthreads();
+  uint16_t* out = vt + (size_t(kvh) * n_groups + g) * size_t(HD) * 16;
+  for (int i = threadIdx.x; i < HD * 2; i += 256) {  // (dim, half of the 16 rows): 16 bytes each
+    const int d = i >> 1, h8 = (i & 1) * 8;
+    u32x4 v;
+#pragma unroll
+    for (int e = 0; e < 4; ++e) v[e] = uint32_t(sh[h8 + 2 * e][d]) | (uint32_t(sh[h8 + 2 * e + 1][d]) << 16);
+    *reinterpret_cast<u32x4*>(out + size_t(d) * 16 + h8) = v;
+  }
+}
+
+hipError_t launch_kv_save(const esp_attn_params* p, const void* Kb, const void* Vb, void* pool, const esp_kvsave* e, int n,
+                          hipStream_t st) {
+  const long total = long(n) * (p->Hkv * p->head_dim / 8);
+  hipLaunchKernelGGL(kv_save_kernel, dim3((unsigned)((total + 255) / 256)), dim3(256), 0, st, (const uint16_t*)Kb,
+                     (const uint16_t*)Vb, (uint16_t*)pool, e, n, p->Hkv, p->head_dim, p->kv_ld, p->bt, p->kv_base);
+  return hipGetLastError();
+}
+
+hipError_t launch_kv_copy_blocks(const esp_attn_params* p, void* pool, const int32_t* pairs, int n_pairs, int n_layers,
+                                 uint64_t region_elems, hipStream_t st) {
+  const uint64_t blk2 = uint64_t(2) * p->bt * p->Hkv * p->head_dim;
+  hipLaunchKernelGGL(kv_copy_blocks_kernel, dim3((unsigned)((blk2 / 8 + 255) / 256), n_pairs, n_layers), dim3(256), 0, st,
+                     (uint16_t*)pool, (const int2*)pairs, blk2, region_elems);
+  return hipGetLastError();
+}
+
+hipError_t launch_kv_gather(const esp_attn_params* p, const void* pool, const int32_t* blocks, int n, void* K_out,
+                            void* V_out, hipStream_t st) {
+  const long total = long(n) * (p->Hkv * p->head_dim / 8);
+  hipLaunchKernelGGL(kv_gather_kernel, dim3((unsigned)((total + 255) / 256)), dim3(256), 0, st, (const uint16_t*)pool, blocks,
+                     n, (uint16_t*)K_out, (uint16_t*)V_out, p->Hkv, p->head_dim, p->bt, p->kv_base);
+  return hipGetLastError();
+}
+
+hipError_t launch_kv_relayout(const esp_attn_params* p, const void* src, void* dst, int to_native, int n_blocks,
+                              hipStream_t st) {
+  const long total = long(n_blocks) * 2 * p->bt * (p->Hkv * p->head_dim / 8);
+  hipLaunchKernelGGL(kv_relayout_kernel, dim3((unsigned)((total + 255) / 256)), dim3(256), 0, st, (const uint16_t*)src,
+                     (uint16_t*)dst, to_native, n_blocks, p->Hkv, p->head_dim, p->bt);
+  return hipGetLastError();
+}
+
+hipError_t launch_vt_stage(const esp_attn_params* p, const void* Vb, void* vt, int n_rows, hipStream_t st) {
+  const int n_groups = (n_rows + 15) / 16;
+  hipLaunchKernelGGL(vt_stage_kernel, dim3(n_groups, p->Hkv), dim3(256), 0, st, (const uint16_t*)Vb, (uint16_t*)vt, n_rows,
+                     n_groups, p->head_dim, p->kv_ld);
+  return hipGetLastError();
+}
+
+}  // namespace esp

@@ -1,0 +1,99 @@
+"""Calls into libespetero_attn.so with torch tensors as device memory.
+
+torch is plumbing here (allocation, streams, host<->device copies); every
+computation happens behind the C ABI. There is no fallback path: a missing or
+failing library raises.
+"""
+import ctypes as C
+
+import numpy as np
+import torch
+
+from . import abi
+
+_ERRLEN = 512
+
+
+def _ptr(t):
+    return None if t is None else C.c_void_p(t.data_ptr())
+
+
+def _stream(stream):
+    if stream is None:
+        stream = torch.cuda.current_stream()
+    return C.c_void_p(stream.cuda_stream)
+
+
+def init(device=0):
+    err = C.create_string_buffer(_ERRLEN)
+    abi.check(abi.attn_lib().esp_attn_init(device, err, _ERRLEN), err)
+
+
+def to_dev(a, device="cuda"):
+    """numpy array (any dtype, incl. structured records) -> device tensor of raw bytes / ints."""
+    a = np.ascontiguousarray(a)
+    if a.dtype.fields is not None or a.dtype == np.uint16:
+        flat = a.view(np.uint8).reshape(-1)
+        return torch.from_numpy(flat.copy()).to(device)
+    return torch.from_numpy(a.copy()).to(device)
+
+
+def workspace_bytes(params, n_rows, n_parts):
+    return abi.attn_lib().esp_attn_workspace_bytes(C.byref(params), n_rows, n_parts)
+
+
+def forward(params, Q, Kb, Vb, pool, blocks, desc, pos, O, tiles, n_tiles, trees, n_trees, jobs, n_jobs, n_parts, n_rows,
+            workspace, stream=None):
+    """All tensors are device tensors (records as byte tensors). Enqueues on `stream`."""
+    err = C.create_string_buffer(_ERRLEN)
+    rc = abi.attn_lib().esp_attn_forward(
+        C.byref(params), _ptr(Q), _ptr(Kb), _ptr(Vb), _ptr(pool), _ptr(blocks), _ptr(desc), _ptr(pos), _ptr(O),
+        _ptr(tiles), n_tiles, _ptr(trees), n_trees, _ptr(jobs), n_jobs, n_parts, n_rows, _ptr(workspace),
+        0 if workspace is None else workspace.numel() * workspace.element_size(), _stream(stream), err, _ERRLEN)
+    abi.check(rc, err)
+
+
+def kv_save(params, Kb, Vb, pool, entries, n_entries, stream=None):
+    err = C.create_string_buffer(_ERRLEN)
+    abi.check(abi.attn_lib().esp_kv_save(C.byref(params), _ptr(Kb), _ptr(Vb), _ptr(pool), _ptr(entries), n_entries,
+                                         _stream(stream), err, _ERRLEN), err)
+
+
+def kv_copy_blocks(params, pool, pairs, n_pairs, n_layers, region_elems, stream=None):
+    err = C.create_string_buffer(_ERRLEN)
+    abi.check(abi.attn_lib().esp_kv_copy_blocks(C.byref(params), _ptr(pool), _ptr(pairs), n_pairs, n_layers,
+                                                C.c_uint64(region_elems), _stream(stream), err, _ERRLEN), err)
+
+
+def kv_gather(params, pool, blocks, n_tokens, K_out, V_out, stream=None):
+    err = C.create_string_buffer(_ERRLEN)
+    abi.check(abi.attn_lib().esp_kv_gather(C.byref(params), _ptr(pool), _ptr(blocks), n_tokens, _ptr(K_out), _ptr(V_out),
+                                           _stream(stream), err, _ERRLEN), err)
+
+
+def kv_relayout(params, src, src_layout, dst, dst_layout, n_blocks, stream=None):
+    err = C.create_string_buffer(_ERRLEN)
+    abi.check(abi.attn_lib().esp_kv_relayout(C.byref(params), _ptr(src), src_layout, _ptr(dst), dst_layout, n_blocks,
+                                             _stream(stream), err, _ERRLEN), err)
+
+
+class DevicePass:
+    """One planned pass resident on the device: uploads the records once and
+    replays esp_attn_forward (what a decode chain does between host syncs)."""
+
+    def __init__(self, params, trees, tiles, jobs, n_parts, n_rows, blocks, desc=None, pos=None, device="cuda"):
+        self.params = params
+        self.n_trees, self.n_tiles, self.n_jobs = len(trees), len(tiles), len(jobs)
+        self.n_parts, self.n_rows = n_parts, n_rows
+        self.trees = to_dev(np.ascontiguousarray(trees, dtype=abi.TREE_DT), device)
+        self.tiles = to_dev(np.ascontiguousarray(tiles, dtype=abi.TILE_DT), device)
+        self.jobs = to_dev(np.ascontiguousarray(jobs, dtype=abi.COMBINE_DT), device) if len(jobs) else None
+        self.blocks = to_dev(np.ascontiguousarray(blocks, dtype=np.int32), device) if blocks is not None else None
+        self.desc = to_dev(np.ascontiguousarray(desc, dtype=np.int32), device) if desc is not None else None
+        self.pos = to_dev(np.ascontiguousarray(pos, dtype=np.int32), device) if pos is not None else None
+        nbytes = workspace_bytes(params, n_rows, n_parts)
+        self.workspace = torch.empty(nbytes, dtype=torch.uint8, device=device)
+
+    def run(self, Q, Kb, Vb, pool, O, stream=None):
+        forward(self.params, Q, Kb, Vb, pool, self.blocks, self.desc, self.pos, O, self.tiles, self.n_tiles, self.trees,
+                self.n_trees, self.jobs, self.n_jobs, self.n_parts, self.n_rows, self.workspace, stream)

@@ -1,0 +1,133 @@
+// Attention tile planner: which (tree, row tile, cached-key range) units a pass
+// runs and how split ranges merge. Host code, no device calls.
+//
+// Two rules share one implementation:
+//   * reference rule  -- PlanOptions::reference(): the records are identical,
+//     field for field, to what the reference's planner emits
+//     (plan_tiles, src/model/impl/forest.h:1378-1433 without the sparse branch;
+//      g4_plan_tiles, src/model/impl/gemma.h:77-116): 8-row tiles, every tree
+//     gets the same split budget 256 / (groups * tiles), 32-key boundaries.
+//   * balanced rule   -- PlanOptions::mi355x(): one chunk size for the whole
+//     pass, derived from the pass's total key count, so every workgroup
+//     streams about the same number of KV bytes whatever its sequence length
+//     (the reference rule gives a 512-token and an 8192-token sequence the same
+//     number of splits, which leaves most of 256 CUs idle while the longest
+//     sequence finishes). Boundaries stay on page multiples.
+// Only the algebra is contractual: the ranges of a tile group partition
+// [k0, P), the last range owns the batch keys, parts merge in range order.
+#pragma once
+
+#include <algorithm>
+#include <climits>
+#include <cstdint>
+#include <vector>
+
+#include "../../include/espetero_attn.h"
+
+namespace espetero::engine {
+
+struct PlanOptions {
+  int rows_per_tile = 8;    // query rows per tile
+  int groups_target = 256;  // workgroups a few-tile pass is split up to
+  int split = 512;          // reference rule: largest chunk a split tile is sized to; 0: never split
+  int min_chunk = 32;       // fewest cached keys a split tile takes
+  int granule = 32;         // split boundaries are multiples of this
+  int max_splits = 64;      // parts per tile group
+  int min_span = 64;        // shorter cached ranges are not split
+  bool balanced = false;    // false: reference rule; true: equal keys per workgroup
+
+  static PlanOptions reference() { return PlanOptions{}; }
+  // rows: query rows per tile (decode 1..8 -> 8-row budget is irrelevant; prefill 64/128).
+  static PlanOptions mi355x(int rows, int workgroups) {
+    PlanOptions o;
+    o.rows_per_tile = rows;
+    o.groups_target = workgroups;
+    o.split = 0;
+    o.min_chunk = 64;
+    o.granule = 32;
+    o.max_splits = 256;
+    o.min_span = 128;
+    o.balanced = true;
+    return o;
+  }
+};
+
+struct AttnPlan {
+  std::vector<esp_tree> trees;
+  std::vector<esp_tile> tiles;
+  std::vector<esp_combine> combine;
+  int parts = 0;
+  int rows_per_tile = 8;
+};
+
+// groups: workgroups per tile (KV heads, or KV heads x head splits).
+// window > 0 needs pos (4 ints per row, pos[4 * row] = position).
+inline void plan_tiles(AttnPlan& A, int groups, int window, const int32_t* pos, const PlanOptions& o) {
+  A.tiles.clear();
+  A.combine.clear();
+  A.parts = 0;
+  A.rows_per_tile = o.rows_per_tile;
+  const int R = o.rows_per_tile;
+  struct RowTile {
+    int tree, r, k0, b0, span;
+  };
+  std::vector<RowTile> rts;
+  long long total_span = 0;
+  for (int ti = 0; ti < int(A.trees.size()); ++ti) {
+    const esp_tree& t = A.trees[size_t(ti)];
+    for (int r = 0; r < t.M; r += R) {
+      int k0 = 0, b0 = 0;
+      if (window > 0) {
+        // The tile's earliest row bounds what any of its rows can still see:
+        // cached key j sits at position j, root row j at P + j (gemma.h:88-94).
+        int minpos = INT32_MAX;
+        for (int i = r; i < std::min(t.M, r + R); ++i) minpos = std::min(minpos, pos[4 * (t.base + i)]);
+        k0 = std::clamp(minpos - window + 1, 0, t.P);
+        b0 = std::max(0, minpos - window + 1 - t.P);
+      }
+      rts.push_back({ti, r, k0, b0, t.P - k0});
+      total_span += t.P - k0;
+    }
+  }
+  const int n_tiles = int(rts.size());
+  const int budget = std::max(1, o.groups_target / std::max(1, groups * n_tiles));
+  int chunk_all = 0;  // balanced rule: keys per workgroup
+  if (o.balanced && budget > 1) {
+    const long long want = (total_span * groups + o.groups_target - 1) / o.groups_target;
+    chunk_all = int(std::max<long long>(o.min_chunk, (want + o.granule - 1) / o.granule * o.granule));
+  }
+  for (const RowTile& rt : rts) {
+    const esp_tree& t = A.trees[size_t(rt.tree)];
+    const int span = rt.span;
+    int ns = 1;
+    if (budget > 1 && span >= o.min_span) {
+      if (o.balanced) {
+        ns = std::min((span + chunk_all - 1) / chunk_all, o.max_splits);
+      } else if (o.split > 0) {
+        const int chunk =
+            std::max(std::max(32, o.min_chunk),
+                     std::min(o.split, ((span + budget - 1) / budget + o.granule - 1) / o.granule * o.granule));
+        ns = std::min({(span + chunk - 1) / chunk, budget, o.max_splits});
+      }
+    }
+    if (ns <= 1) {
+      A.tiles.push_back({rt.tree, t.base + rt.r, rt.k0, t.P, -1, 1, rt.b0, 0});
+      continue;
+    }
+    const int per = (span + ns - 1) / ns;
+    const int step = (per + o.granule - 1) / o.granule * o.granule;
+    const int part0 = A.parts;
+    int used = 0;
+    for (int k = rt.k0; k < t.P; ++used) {
+      int k1 = std::min(t.P, k + step);
+      // Balanced rule: a windowed range starts anywhere, its inner boundaries still fall on page multiples.
+      if (o.balanced && k1 < t.P) k1 = std::max(k + o.granule, k1 / o.granule * o.granule);
+      k1 = std::min(t.P, k1);
+      A.tiles.push_back({rt.tree, t.base + rt.r, k, k1, A.parts++, k1 >= t.P ? 1 : 0, rt.b0, 0});
+      k = k1;
+    }
+    A.combine.push_back({t.base + rt.r, std::min(R, t.M - rt.r), part0, used});
+  }
+}
+
+}  // namespace espetero::engine

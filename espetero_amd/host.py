@@ -1,0 +1,192 @@
+"""ctypes binding of the host engine (include/espetero_engine.h): tile planner,
+KV block pool, slots and the pass builder. Host memory only."""
+import ctypes as C
+import os
+
+import numpy as np
+
+from . import abi
+
+
+class PlanOptions(C.Structure):
+    _fields_ = [("rows_per_tile", C.c_int32), ("groups_target", C.c_int32), ("split", C.c_int32),
+                ("min_chunk", C.c_int32), ("granule", C.c_int32), ("max_splits", C.c_int32),
+                ("min_span", C.c_int32), ("balanced", C.c_int32)]
+
+
+class TreeSpec(C.Structure):
+    _fields_ = [("parent", C.c_int32), ("save", C.c_int32), ("work", C.c_int32), ("root_len", C.c_int32),
+                ("save_len", C.c_int32), ("n_leaves", C.c_int32), ("leaf_offsets", C.POINTER(C.c_int32)),
+                ("leaf_tokens", C.POINTER(C.c_int32)), ("commit_chain", C.c_int32), ("noncausal", C.c_int32)]
+
+
+_V, _I = C.c_void_p, C.c_int32
+_ERR = (C.c_char_p, C.c_size_t)
+_PO = C.POINTER(PlanOptions)
+_TS = C.POINTER(TreeSpec)
+_IP = C.POINTER(C.c_int32)
+ENGINE_SYMBOLS = {
+    "esp_plan_options_reference": (None, (_PO,)),
+    "esp_plan_options_mi355x": (None, (_PO, _I, _I)),
+    "esp_plan_tiles": (C.c_int, (_V, _I, _I, _I, _V, _PO, _V, _I, _IP, _V, _I, _IP, _IP) + _ERR),
+    "esp_engine_create": (_V, (_I, _I, _I, _I)),
+    "esp_engine_destroy": (None, (_V,)),
+    "esp_engine_slot_alloc": (C.c_int, (_V,)),
+    "esp_engine_slot_free": (C.c_int, (_V, _I)),
+    "esp_engine_slot_reset": (C.c_int, (_V, _I)),
+    "esp_engine_slot_fork": (C.c_int, (_V, _I, _I)),
+    "esp_engine_slot_len": (C.c_int, (_V, _I)),
+    "esp_engine_slot_blocks": (C.c_int, (_V, _I, _V, _I)),
+    "esp_engine_free_blocks": (C.c_int, (_V,)),
+    "esp_engine_block_ref": (C.c_int, (_V, _I)),
+    "esp_engine_pass_blocks": (C.c_int, (_V, _TS, _I)),
+    "esp_engine_pass_begin": (C.c_int, (_V, _TS, _I) + _ERR),
+    "esp_engine_pass_rows": (C.c_int, (_V,)),
+    "esp_engine_pass_counts": (C.c_int, (_V, _IP, _IP, _IP)),
+    "esp_engine_pass_trees": (C.c_int, (_V, _V)),
+    "esp_engine_pass_desc": (C.c_int, (_V, _V)),
+    "esp_engine_pass_pos": (C.c_int, (_V, _V)),
+    "esp_engine_pass_table": (C.c_int, (_V, _V)),
+    "esp_engine_pass_saves": (C.c_int, (_V, _V)),
+    "esp_engine_pass_cow": (C.c_int, (_V, _V)),
+    "esp_engine_pass_commit": (C.c_int, (_V,)),
+    "esp_engine_pass_abort": (C.c_int, (_V,)),
+}
+
+_lib = None
+
+
+def engine_lib():
+    global _lib
+    if _lib is None:
+        if not os.path.exists(abi.ENGINE_LIB_PATH):
+            raise abi.EspError(f"{abi.ENGINE_LIB_PATH} is not built (run __graft_entry__.build())")
+        lib = C.CDLL(abi.ENGINE_LIB_PATH)
+        for name, (res, args) in ENGINE_SYMBOLS.items():
+            fn = getattr(lib, name)
+            fn.restype = res
+            fn.argtypes = list(args)
+        _lib = lib
+    return _lib
+
+
+def options_reference():
+    o = PlanOptions()
+    engine_lib().esp_plan_options_reference(C.byref(o))
+    return o
+
+
+def options_mi355x(rows, workgroups):
+    o = PlanOptions()
+    engine_lib().esp_plan_options_mi355x(C.byref(o), rows, workgroups)
+    return o
+
+
+def plan_tiles(trees, groups, window, pos, options):
+    """trees: TREE_DT array. Returns (tiles TILE_DT, jobs COMBINE_DT, n_parts)."""
+    lib = engine_lib()
+    trees = np.ascontiguousarray(trees, dtype=abi.TREE_DT)
+    pos_a = None if pos is None else np.ascontiguousarray(pos, dtype=np.int32)
+    err = C.create_string_buffer(256)
+    nt, nj, npart = C.c_int32(0), C.c_int32(0), C.c_int32(0)
+    rc = lib.esp_plan_tiles(trees.ctypes.data, len(trees), groups, window, None if pos_a is None else pos_a.ctypes.data,
+                            C.byref(options), None, 0, C.byref(nt), None, 0, C.byref(nj), C.byref(npart), err, 256)
+    if rc not in (0, 4):
+        abi.check(rc, err)
+    tiles = np.zeros(nt.value, abi.TILE_DT)
+    jobs = np.zeros(nj.value, abi.COMBINE_DT)
+    rc = lib.esp_plan_tiles(trees.ctypes.data, len(trees), groups, window, None if pos_a is None else pos_a.ctypes.data,
+                            C.byref(options), tiles.ctypes.data, len(tiles), C.byref(nt), jobs.ctypes.data, len(jobs),
+                            C.byref(nj), C.byref(npart), err, 256)
+    abi.check(rc, err)
+    return tiles, jobs, npart.value
+
+
+def make_spec(parent=-1, save=-1, work=-1, root_len=0, save_len=0, leaves=(), commit_chain=0, noncausal=0):
+    """leaves: list of token lists. Keeps the arrays alive on the returned struct."""
+    s = TreeSpec(parent, save, work, root_len, save_len, len(leaves), None, None, commit_chain, noncausal)
+    if leaves:
+        offs = np.zeros(len(leaves) + 1, np.int32)
+        offs[1:] = np.cumsum([len(x) for x in leaves])
+        toks = np.ascontiguousarray(np.concatenate([np.asarray(x, np.int32) for x in leaves]), dtype=np.int32)
+        s._keep = (offs, toks)
+        s.leaf_offsets = offs.ctypes.data_as(_IP)
+        s.leaf_tokens = toks.ctypes.data_as(_IP)
+    return s
+
+
+class Engine:
+    """KV pool + slots + pass builder (C++ KvEngine)."""
+
+    def __init__(self, n_blocks, bt, n_slots, max_ctx=1 << 30):
+        self.lib = engine_lib()
+        self.h = self.lib.esp_engine_create(n_blocks, bt, n_slots, max_ctx)
+        if not self.h:
+            raise abi.EspError("esp_engine_create failed")
+        self.bt = bt
+
+    def __del__(self):
+        if getattr(self, "h", None):
+            self.lib.esp_engine_destroy(self.h)
+            self.h = None
+
+    def slot_alloc(self):
+        return self.lib.esp_engine_slot_alloc(self.h)
+
+    def slot_free(self, s):
+        return self.lib.esp_engine_slot_free(self.h, s)
+
+    def slot_reset(self, s):
+        return self.lib.esp_engine_slot_reset(self.h, s)
+
+    def slot_fork(self, a, b):
+        return self.lib.esp_engine_slot_fork(self.h, a, b)
+
+    def slot_len(self, s):
+        return self.lib.esp_engine_slot_len(self.h, s)
+
+    def slot_blocks(self, s):
+        n = self.lib.esp_engine_slot_blocks(self.h, s, None, 0)
+        out = np.zeros(max(n, 1), np.int32)
+        self.lib.esp_engine_slot_blocks(self.h, s, out.ctypes.data, n)
+        return out[:n].copy()
+
+    def free_blocks(self):
+        return self.lib.esp_engine_free_blocks(self.h)
+
+    def block_ref(self, b):
+        return self.lib.esp_engine_block_ref(self.h, b)
+
+    def pass_blocks(self, specs):
+        arr = (TreeSpec * len(specs))(*specs)
+        return self.lib.esp_engine_pass_blocks(self.h, arr, len(specs))
+
+    def pass_begin(self, specs):
+        """Returns dict(trees, desc, pos, table, saves, cow, M). Raises EspError on a refused pass."""
+        arr = (TreeSpec * len(specs))(*specs)
+        err = C.create_string_buffer(256)
+        rc = self.lib.esp_engine_pass_begin(self.h, arr, len(specs), err, 256)
+        abi.check(rc, err)
+        nt, ns, nc = C.c_int32(0), C.c_int32(0), C.c_int32(0)
+        n = self.lib.esp_engine_pass_counts(self.h, C.byref(nt), C.byref(ns), C.byref(nc))
+        M = self.lib.esp_engine_pass_rows(self.h)
+        trees = np.zeros(n, abi.TREE_DT)
+        desc = np.zeros((max(M, 1), 4), np.int32)
+        pos = np.zeros((max(M, 1), 4), np.int32)
+        table = np.zeros(max(nt.value, 1), np.int32)
+        saves = np.zeros(max(ns.value, 1), abi.KVSAVE_DT)
+        cow = np.zeros((max(nc.value, 1), 2), np.int32)
+        self.lib.esp_engine_pass_trees(self.h, trees.ctypes.data)
+        self.lib.esp_engine_pass_desc(self.h, desc.ctypes.data)
+        self.lib.esp_engine_pass_pos(self.h, pos.ctypes.data)
+        self.lib.esp_engine_pass_table(self.h, table.ctypes.data)
+        self.lib.esp_engine_pass_saves(self.h, saves.ctypes.data)
+        self.lib.esp_engine_pass_cow(self.h, cow.ctypes.data)
+        return dict(trees=trees, desc=desc[:M], pos=pos[:M], table=table[:nt.value], saves=saves[:ns.value],
+                    cow=cow[:nc.value], M=M)
+
+    def pass_commit(self):
+        return self.lib.esp_engine_pass_commit(self.h)
+
+    def pass_abort(self):
+        return self.lib.esp_engine_pass_abort(self.h)

@@ -1,0 +1,164 @@
+/* espetero_attn.h -- C ABI of the MI355X (gfx950) paged-KV attention path.
+ *
+ * This is the boundary a host engine binds instead of the reference's
+ * per-dispatch kernel ABI (pipeline name + buffers 0..11 + by-value params):
+ *   reference kernels   kernels/40_attention.metal:155-905,
+ *                       kernels/80_gemma.metal:157-601,
+ *                       kernels/82_qwen3_omni.metal:97-106
+ *   reference bindings  src/model/impl/forest.h:2855-2947,
+ *                       src/model/impl/gemma.h:223-303,
+ *                       src/model/impl/qwen3_omni.h:96-161
+ *   host record structs src/model/impl/forest.h:1308-1345, gemma.h:29-35
+ *
+ * Conventions (the reference's dlopen'd C ABI uses the same ones,
+ * tests/parity_test.mm:37-57): every function returns 0 on success or a
+ * non-zero ESP_E* code and writes a NUL-terminated message into `err`
+ * (may be NULL). No function throws, allocates or frees device memory, or
+ * synchronises the device: work is enqueued on `stream` (a hipStream_t passed
+ * as void*; NULL = the default stream) and the caller orders it. All pointer
+ * arguments other than `p`, `err` are DEVICE pointers unless stated. Like the
+ * reference's model object (src/model/api.h:4-6) the library is driven from
+ * one thread at a time.
+ *
+ * KV pool layout ("native", ESP_LAYOUT_NATIVE). One region per attention
+ * layer starting at element offset kv_base, n_blocks blocks per region, each
+ * block 2 * bt * Hkv * head_dim elements (the reference's block size,
+ * src/model/impl/model.h:396), arranged for 64-wide wavefronts as
+ *   block b, KV head h : base = kv_base + (b * Hkv + h) * 2 * bt * head_dim
+ *   K[token t][dim d]  : base + t * head_dim + d                (row major)
+ *   V[token t][dim d]  : base + bt * head_dim + d * bt + t      (transposed)
+ * so one (block, head) is a single contiguous run and V is already the
+ * k-contiguous operand of the P.V matrix product. The reference's layout
+ * (ESP_LAYOUT_REFERENCE, kernels/40_attention.metal:245-247) is
+ *   K/V[which][t][h][d]: kv_base + (2 b + which) * bt * kv_ld + t * kv_ld + h * head_dim + d
+ * and is accepted only by esp_kv_relayout (import / export of blocks).
+ */
+#ifndef ESPETERO_ATTN_H
+#define ESPETERO_ATTN_H
+
+#include <stddef.h>
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+#define ESP_ABI_VERSION 1
+
+enum { ESP_OK = 0, ESP_EINVAL = 1, ESP_EUNSUPPORTED = 2, ESP_ELAUNCH = 3, ESP_EWORKSPACE = 4 };
+enum { ESP_F16 = 0, ESP_BF16 = 1 };
+enum { ESP_LAYOUT_REFERENCE = 0, ESP_LAYOUT_NATIVE = 1 };
+
+/* One sequence-in-pass. Field for field AttnTree (kernels/40_attention.metal:134-139,
+ * host AttnTreeRec src/model/impl/forest.h:1308-1310). */
+typedef struct esp_tree {
+  int32_t base;  /* absolute first row of the tree in Q/Kb/Vb/O/desc/pos */
+  int32_t P;     /* cached keys [0, P) */
+  int32_t table; /* first entry of its block list in `blocks`; ring layers: first ring block */
+  int32_t M;     /* rows of the tree in this pass */
+} esp_tree;
+
+/* One unit of GPU work. Field for field G4Tile (kernels/80_gemma.metal:146-155,
+ * host G4TileRec src/model/impl/gemma.h:29-31); AttnTile (40_:141-150) is the
+ * same record with b0 = pad = 0. */
+typedef struct esp_tile {
+  int32_t tree;
+  int32_t r0;   /* absolute first query row; the tile covers rows_per_tile rows (fewer at the tree's end) */
+  int32_t k0;   /* cached-key range [k0, k1) */
+  int32_t k1;
+  int32_t part; /* -1: write O; else index of the partial record this tile writes */
+  int32_t last; /* also scan the tree's batch keys (this pass's own rows) */
+  int32_t b0;   /* first batch key (relative row) any row of the tile may see */
+  int32_t pad;
+} esp_tile;
+
+/* Merge job of one split tile group. Field for field AttnCombine (40_:804-809). */
+typedef struct esp_combine {
+  int32_t r0;     /* absolute first row */
+  int32_t rows;   /* live rows */
+  int32_t part0;  /* first partial record */
+  int32_t nparts; /* records, merged in order part0, part0 + 1, ... */
+} esp_combine;
+
+/* KV append entry. Field for field KVSave (40_:868-873, forest.h:1317-1319). */
+typedef struct esp_kvsave {
+  int32_t src_row;
+  int32_t block;
+  int32_t pos; /* token index within the block */
+  int32_t pad;
+} esp_kvsave;
+
+/* Per-layer constants: G4AttnParams (80_:134-144) + AttnParams' gate stride
+ * (40_:124-132) + what the Metal templates fix at compile time (head_dim,
+ * element type, score scale). */
+typedef struct esp_attn_params {
+  int32_t H;             /* query heads */
+  int32_t Hkv;           /* KV heads; H % Hkv == 0, group G = H / Hkv */
+  int32_t head_dim;      /* 128 or 256 */
+  int32_t dtype;         /* ESP_F16 | ESP_BF16: element type of Q, Kb, Vb, pool and O */
+  int32_t q_ld;          /* Q / O row stride in elements (>= H * head_dim) */
+  int32_t kv_ld;         /* Kb / Vb row stride in elements (>= Hkv * head_dim) */
+  int32_t bt;            /* tokens per KV block, a multiple of 16 */
+  int32_t window;        /* sliding window (0: none): key visible iff qpos - kpos < window */
+  int32_t ring;          /* blocks per slot ring on sliding layers (0: block lists) */
+  int32_t bidi;          /* image rows see their whole image (desc.w) */
+  int32_t rows_per_tile; /* query rows per tile the planner used (the reference: 8) */
+  float scale;           /* multiplies q.k (1 when q arrives pre-scaled) */
+  uint64_t kv_base;      /* element offset of this layer's region in the pool */
+  const float* gate;     /* optional sigmoid output gate (40_:334-342), NULL: none */
+  int32_t gate_ld;       /* gate[row * gate_ld + h * gate_hs + gate_off + d] */
+  int32_t gate_hs;
+  int32_t gate_off;
+  int32_t reserved;
+} esp_attn_params;
+
+/* Library / device check. Safe to call more than once. */
+int esp_attn_init(int device, char* err, size_t errlen);
+int esp_attn_abi_version(void);
+
+/* Bytes of `workspace` esp_attn_forward needs for a pass of n_rows batch rows
+ * whose plan holds n_parts partial records (replaces the reference's `parts`
+ * sizing, forest.h:2716, gemma.h:162-165). Host-only arithmetic. */
+size_t esp_attn_workspace_bytes(const esp_attn_params* p, int32_t n_rows, int32_t n_parts);
+
+/* Attention of one layer over a planned pass, then the split-K merge:
+ * replaces the dispatch of flash_attention / attn_decode_gqa / g4_attention /
+ * g4_attention_dec and attention_combine (forest.h:2895-2933, gemma.h:249-284).
+ * Q [n_rows][q_ld], Kb/Vb [n_rows][kv_ld] (this pass's rows, not yet cached),
+ * desc/pos: int32[4] per row (desc = seg_start, 0, anc_len, img_end; pos.x =
+ * position); desc may be NULL (plain causal rows), pos may be NULL when
+ * window == 0. O [n_rows][q_ld]. The kernel family is chosen from
+ * rows_per_tile * G (streaming split-K kernel up to 64 packed rows, tiled
+ * MFMA kernel above), as the reference chooses from its plan (forest.h:2863-2868). */
+int esp_attn_forward(const esp_attn_params* p, const void* Q, const void* Kb, const void* Vb, const void* kv_pool,
+                     const int32_t* blocks, const int32_t* desc, const int32_t* pos, void* O, const esp_tile* tiles,
+                     int32_t n_tiles, const esp_tree* trees, int32_t n_trees, const esp_combine* jobs, int32_t n_jobs,
+                     int32_t n_parts, int32_t n_rows, void* workspace, size_t workspace_bytes, void* stream, char* err,
+                     size_t errlen);
+
+/* Append batch rows to the pool: replaces kv_save (40_:875-889; forest.h:2935-2947). */
+int esp_kv_save(const esp_attn_params* p, const void* Kb, const void* Vb, void* kv_pool, const esp_kvsave* entries,
+                int32_t n_entries, void* stream, char* err, size_t errlen);
+
+/* Copy whole blocks src -> dst in every layer region (copy on write): replaces
+ * kv_copy_blocks (40_:894-905; forest.h:1438-1449). pairs: int32[2] per pair;
+ * region_elems: elements per layer region. */
+int esp_kv_copy_blocks(const esp_attn_params* p, void* kv_pool, const int32_t* pairs, int32_t n_pairs, int32_t n_layers,
+                       uint64_t region_elems, void* stream, char* err, size_t errlen);
+
+/* Gather a block list's first n_tokens tokens into contiguous rows
+ * K_out / V_out [n_tokens][Hkv * head_dim] (the order of the reference's slot
+ * files, src/model/model.mm:600-752: logical token order, K then V). Bit copy. */
+int esp_kv_gather(const esp_attn_params* p, const void* kv_pool, const int32_t* blocks, int32_t n_tokens, void* K_out,
+                  void* V_out, void* stream, char* err, size_t errlen);
+
+/* Convert n_blocks whole blocks of one layer region between the reference's
+ * block layout and the native one (src and dst regions must not overlap).
+ * src_layout / dst_layout: ESP_LAYOUT_*. Bit copy. */
+int esp_kv_relayout(const esp_attn_params* p, const void* src_pool, int32_t src_layout, void* dst_pool, int32_t dst_layout,
+                    int32_t n_blocks, void* stream, char* err, size_t errlen);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* ESPETERO_ATTN_H */

@@ -1,0 +1,102 @@
+/* espetero_engine.h -- C view of the host-side attention call surface
+ * (espetero_amd/engine/ *.hpp, C++20, no device calls): the tile planner, the
+ * refcounted KV block pool with copy-on-write block lists, and the builder
+ * that turns a pass's trees into the device records esp_attn_forward reads.
+ *
+ * It replaces, for this path only, what the reference keeps in
+ *   plan_tiles / g4_plan_tiles     src/model/impl/forest.h:1378-1433, gemma.h:77-116
+ *   kv_alloc / retain / release    src/model/impl/model.h:722-737
+ *   Forest::target_blocks          src/model/impl/forest.h:1785-1811
+ *   target_new_blocks              src/model/impl/forest.h:1821-1829
+ *   leaf hosting, row descriptors  src/model/impl/forest.h:2201-2220, 2374-2443
+ *   block tables, kv_save entries  src/model/impl/forest.h:2483-2520
+ *   slot commit / PassGuard        src/model/impl/forest.h:2468-2482, 4743-4754
+ *   slot_alloc/free/reset/fork/len src/model/model.mm:520-553
+ * The C++ headers are the interface a C++ engine includes; these functions
+ * exist so that other languages (and the tests) can drive the same code.
+ * Errors: 0 / non-zero + message in err, as in espetero_attn.h. Host memory only.
+ */
+#ifndef ESPETERO_ENGINE_H
+#define ESPETERO_ENGINE_H
+
+#include "espetero_attn.h"
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+typedef struct esp_plan_options {
+  int32_t rows_per_tile; /* query rows per tile (reference: 8) */
+  int32_t groups_target; /* workgroups a few-tile pass is split up to (reference: 256) */
+  int32_t split;         /* reference rule: largest chunk a split is sized to (attn_split, 512) */
+  int32_t min_chunk;     /* fewest cached keys of a split tile (attn_min_chunk, 32) */
+  int32_t granule;       /* split boundaries are multiples of this (32) */
+  int32_t max_splits;    /* parts per tile group (64) */
+  int32_t min_span;      /* shorter cached ranges are not split (64) */
+  int32_t balanced;      /* 0: the reference's per-tree budget rule; 1: equal keys per workgroup */
+} esp_plan_options;
+
+/* The reference's constants. */
+void esp_plan_options_reference(esp_plan_options* o);
+/* Tuned for 256 CUs: rows query rows per tile, workgroups the split target. */
+void esp_plan_options_mi355x(esp_plan_options* o, int32_t rows, int32_t workgroups);
+
+/* Plan a pass. trees[n_trees] in; tiles / jobs out (capacities given; on
+ * ESP_EWORKSPACE the needed counts are still written). groups: workgroups per
+ * tile (KV heads). window > 0 needs pos (4 ints per row). */
+int esp_plan_tiles(const esp_tree* trees, int32_t n_trees, int32_t groups, int32_t window, const int32_t* pos,
+                   const esp_plan_options* o, esp_tile* tiles, int32_t tiles_cap, int32_t* n_tiles, esp_combine* jobs,
+                   int32_t jobs_cap, int32_t* n_jobs, int32_t* n_parts, char* err, size_t errlen);
+
+/* ---- KV engine: pool + slots + pass builder ---- */
+typedef struct esp_engine esp_engine;
+
+/* One tree of a pass: the attention-relevant part of the reference's TreeSpec
+ * (src/model/api.h:105-176). Slots: -1 = none. */
+typedef struct esp_tree_spec {
+  int32_t parent;     /* slot whose cached keys the tree reads */
+  int32_t save;       /* slot that receives parent + root[0, save_len) */
+  int32_t work;       /* slot that receives parent + whole root */
+  int32_t root_len;
+  int32_t save_len;   /* 0: whole root */
+  int32_t n_leaves;
+  const int32_t* leaf_offsets; /* n_leaves + 1 */
+  const int32_t* leaf_tokens;
+  int32_t commit_chain; /* leaves [0, k) are one chain whose rows are also saved */
+  int32_t noncausal;
+} esp_tree_spec;
+
+esp_engine* esp_engine_create(int32_t n_blocks, int32_t bt, int32_t n_slots, int32_t max_ctx);
+void esp_engine_destroy(esp_engine* e);
+int esp_engine_slot_alloc(esp_engine* e);                 /* slot or -1 */
+int esp_engine_slot_free(esp_engine* e, int32_t slot);
+int esp_engine_slot_reset(esp_engine* e, int32_t slot);
+int esp_engine_slot_fork(esp_engine* e, int32_t src, int32_t dst);
+int esp_engine_slot_len(const esp_engine* e, int32_t slot);
+int esp_engine_slot_blocks(const esp_engine* e, int32_t slot, int32_t* out, int32_t cap); /* count */
+int esp_engine_free_blocks(const esp_engine* e);
+int esp_engine_block_ref(const esp_engine* e, int32_t block);
+/* Blocks a pass of these trees would take from the free list (pass_kv_tokens / bt). */
+int esp_engine_pass_blocks(const esp_engine* e, const esp_tree_spec* specs, int32_t n);
+
+/* Build a pass: validates every tree before touching anything, then plans
+ * rows, descriptors, positions, the block table, kv_save entries and
+ * copy-on-write pairs. The pass stays pending until committed or aborted. */
+int esp_engine_pass_begin(esp_engine* e, const esp_tree_spec* specs, int32_t n, char* err, size_t errlen);
+int esp_engine_pass_rows(const esp_engine* e);      /* M */
+int esp_engine_pass_counts(const esp_engine* e, int32_t* n_table, int32_t* n_saves, int32_t* n_cow);
+int esp_engine_pass_trees(const esp_engine* e, esp_tree* out);          /* n trees */
+int esp_engine_pass_desc(const esp_engine* e, int32_t* out);            /* 4 * M */
+int esp_engine_pass_pos(const esp_engine* e, int32_t* out);             /* 4 * M */
+int esp_engine_pass_table(const esp_engine* e, int32_t* out);
+int esp_engine_pass_saves(const esp_engine* e, esp_kvsave* out);
+int esp_engine_pass_cow(const esp_engine* e, int32_t* out);             /* 2 * n_cow */
+/* The slots take their new block lists (after the device work completed). */
+int esp_engine_pass_commit(esp_engine* e);
+/* Give the pass's new blocks back; slots are as before the pass. */
+int esp_engine_pass_abort(esp_engine* e);
+
+#ifdef __cplusplus
+}
+#endif
+#endif

@@ -1,0 +1,184 @@
+"""ctypes binding of the CPU checker (oracle/attn_oracle.c) plus a float64
+brute force. TEST INFRASTRUCTURE: imported only by tests/, the smoke check
+and the bench's cpu_baseline leg; the product never touches it.
+"""
+import ctypes as C
+import os
+import subprocess
+
+import numpy as np
+
+from espetero_amd import abi
+
+_DIR = os.path.dirname(os.path.abspath(__file__))
+LIB_PATH = os.path.join(_DIR, "libattn_oracle.so")
+_lib = None
+
+
+def build():
+    subprocess.run(["make", "-s", "-C", _DIR, "-B"], check=True)
+
+
+def lib():
+    global _lib
+    if _lib is None:
+        if not os.path.exists(LIB_PATH):
+            build()
+        L = C.CDLL(LIB_PATH)
+        L.esp_oracle_h2f.restype = C.c_float
+        L.esp_oracle_h2f.argtypes = [C.c_uint16]
+        L.esp_oracle_f2h.restype = C.c_uint16
+        L.esp_oracle_f2h.argtypes = [C.c_float]
+        L.esp_oracle_bf2f.restype = C.c_float
+        L.esp_oracle_bf2f.argtypes = [C.c_uint16]
+        L.esp_oracle_f2bf.restype = C.c_uint16
+        L.esp_oracle_f2bf.argtypes = [C.c_float]
+        _lib = L
+    return _lib
+
+
+def _p(a):
+    return None if a is None else a.ctypes.data_as(C.c_void_p)
+
+
+def _u16(a):
+    a = np.ascontiguousarray(a)
+    assert a.dtype == np.uint16
+    return a
+
+
+def _i32(a):
+    if a is None:
+        return None
+    a = np.ascontiguousarray(a, dtype=np.int32)
+    return a
+
+
+def attn_direct(params, Q, Kb, Vb, pool, blocks, desc, pos, trees, n_threads=1):
+    """Row-by-row semantics. Q/Kb/Vb/pool: uint16 storage bits. Returns O (uint16)."""
+    Q, Kb, Vb, pool = _u16(Q), _u16(Kb), _u16(Vb), _u16(pool)
+    blocks, desc, pos = _i32(blocks), _i32(desc), _i32(pos)
+    trees = np.ascontiguousarray(trees, dtype=abi.TREE_DT)
+    O = np.zeros_like(Q)
+    rc = lib().esp_oracle_attn_direct(C.byref(params), _p(Q), _p(Kb), _p(Vb), _p(pool), _p(blocks), _p(desc), _p(pos),
+                                      _p(O), _p(trees), C.c_int(len(trees)), C.c_int(n_threads))
+    assert rc == 0
+    return O
+
+
+def attn_tiles(params, Q, Kb, Vb, pool, blocks, desc, pos, tiles, trees, jobs, n_parts):
+    """Through tiles, partial records and the merge, as the reference kernels are structured."""
+    Q, Kb, Vb, pool = _u16(Q), _u16(Kb), _u16(Vb), _u16(pool)
+    blocks, desc, pos = _i32(blocks), _i32(desc), _i32(pos)
+    trees = np.ascontiguousarray(trees, dtype=abi.TREE_DT)
+    tiles = np.ascontiguousarray(tiles, dtype=abi.TILE_DT)
+    jobs = np.ascontiguousarray(jobs, dtype=abi.COMBINE_DT)
+    G = params.H // params.Hkv
+    parts = np.zeros(max(1, n_parts) * params.Hkv * params.rows_per_tile * G * (params.head_dim + 2), np.float32)
+    O = np.zeros_like(Q)
+    rc = lib().esp_oracle_attn_tiles(C.byref(params), _p(Q), _p(Kb), _p(Vb), _p(pool), _p(blocks), _p(desc), _p(pos),
+                                     _p(O), _p(tiles), C.c_int(len(tiles)), _p(trees), C.c_int(len(trees)), _p(jobs),
+                                     C.c_int(len(jobs)), _p(parts))
+    assert rc == 0
+    return O
+
+
+def kv_save(params, Kb, Vb, pool, entries):
+    entries = np.ascontiguousarray(entries, dtype=abi.KVSAVE_DT)
+    lib().esp_oracle_kv_save(C.byref(params), _p(_u16(Kb)), _p(_u16(Vb)), _p(pool), _p(entries), C.c_int(len(entries)))
+
+
+def kv_copy_blocks(params, pool, pairs, n_layers, region_elems):
+    pairs = np.ascontiguousarray(pairs, dtype=np.int32).reshape(-1, 2)
+    lib().esp_oracle_kv_copy_blocks(C.byref(params), _p(pool), _p(pairs), C.c_int(len(pairs)), C.c_int(n_layers),
+                                    C.c_uint64(region_elems))
+
+
+def kv_gather(params, pool, blocks, n_tokens):
+    w = params.Hkv * params.head_dim
+    K = np.zeros((n_tokens, w), np.uint16)
+    V = np.zeros((n_tokens, w), np.uint16)
+    blocks = _i32(blocks)
+    lib().esp_oracle_kv_gather(C.byref(params), _p(_u16(pool)), _p(blocks), C.c_int(n_tokens), _p(K), _p(V))
+    return K, V
+
+
+# ---- storage conversions (numpy side) ----
+def to_f32(bits, dtype):
+    bits = np.asarray(bits, dtype=np.uint16)
+    if dtype == abi.ESP_BF16:
+        return (bits.astype(np.uint32) << 16).view(np.float32)
+    return bits.view(np.float16).astype(np.float32)
+
+
+def from_f32(x, dtype):
+    x = np.ascontiguousarray(x, dtype=np.float32)
+    if dtype == abi.ESP_BF16:
+        u = x.view(np.uint32)
+        return ((u + 0x7FFF + ((u >> 16) & 1)) >> 16).astype(np.uint16)
+    return x.astype(np.float16).view(np.uint16)
+
+
+# ---- float64 brute force: dense mask, no paging, no online softmax ----
+def visible_mask(params, tree, desc, pos):
+    """bool [M][P + M]: row rr of the tree sees cached key j (col j) / batch key j (col P + j).
+    The textual rule at kernels/40_attention.metal:104-113 and 80_gemma.metal:283-285."""
+    base, P, M = int(tree["base"]), int(tree["P"]), int(tree["M"])
+    vis = np.zeros((M, P + M), bool)
+    for rr in range(M):
+        row = base + rr
+        d = desc[row] if desc is not None else (0, 0, 0, 0)
+        qpos = pos[row][0] if pos is not None else 0
+        for j in range(P):
+            vis[rr, j] = (qpos - j < params.window) if params.window > 0 else True
+        for j in range(M):
+            v = (j < d[2]) or (j >= d[0] and (j <= rr or (params.bidi and j < d[3])))
+            if params.window > 0 and v:
+                v = qpos - pos[base + j][0] < params.window
+            vis[rr, P + j] = v
+    return vis
+
+
+def gather_tree_kv(params, tree, pool, blocks, Kb, Vb):
+    """K, V float64 [P + M][Hkv][HD] of one tree (cached via the reference-layout pool, then batch)."""
+    base, P, M, table = int(tree["base"]), int(tree["P"]), int(tree["M"]), int(tree["table"])
+    HD, Hkv, bt, kv_ld = params.head_dim, params.Hkv, params.bt, params.kv_ld
+    K = np.zeros((P + M, Hkv, HD), np.float64)
+    V = np.zeros((P + M, Hkv, HD), np.float64)
+    blk = bt * kv_ld
+    for j in range(P):
+        b = table + (j // bt) % params.ring if params.ring else int(blocks[table + j // bt])
+        for which, out in ((0, K), (1, V)):
+            a = params.kv_base + (2 * b + which) * blk + (j % bt) * kv_ld
+            out[j] = to_f32(pool[a:a + Hkv * HD], params.dtype).reshape(Hkv, HD)
+    for j in range(M):
+        K[P + j] = to_f32(Kb[base + j, :Hkv * HD], params.dtype).reshape(Hkv, HD)
+        V[P + j] = to_f32(Vb[base + j, :Hkv * HD], params.dtype).reshape(Hkv, HD)
+    return K, V
+
+
+def brute_force(params, Q, Kb, Vb, pool, blocks, desc, pos, trees, gate=None):
+    """O in float64, [n_rows][H][HD]; rows of no tree stay 0. No rounding of P."""
+    HD, H, Hkv = params.head_dim, params.H, params.Hkv
+    G = H // Hkv
+    n_rows = Q.shape[0]
+    O = np.zeros((n_rows, H, HD), np.float64)
+    for tree in trees:
+        base, P, M = int(tree["base"]), int(tree["P"]), int(tree["M"])
+        K, V = gather_tree_kv(params, tree, pool, blocks, Kb, Vb)
+        vis = visible_mask(params, tree, desc, pos)
+        q = to_f32(Q[base:base + M, :H * HD], params.dtype).astype(np.float64).reshape(M, H, HD)
+        for h in range(H):
+            kvh = h // G
+            s = (q[:, h, :] @ K[:, kvh, :].T) * float(params.scale)
+            s = np.where(vis, s, -np.inf)
+            m = s.max(axis=1, keepdims=True)
+            m = np.where(np.isfinite(m), m, 0.0)
+            p = np.exp(s - m)
+            l = p.sum(axis=1, keepdims=True)
+            o = p @ V[:, kvh, :]
+            o = np.where(l > 0, o / np.where(l > 0, l, 1.0), 0.0)
+            if gate is not None:
+                o = o / (1.0 + np.exp(-gate[base:base + M, h, :].astype(np.float64)))
+            O[base:base + M, h, :] = o
+    return O

@@ -1,0 +1,48 @@
+"""Runs synthetic cases through the C ABI on the GPU (used by the -m gpu tests)."""
+import numpy as np
+import torch
+
+from espetero_amd import abi, device, host
+
+
+def dev_u16(a):
+    return torch.from_numpy(np.ascontiguousarray(a).view(np.int16).copy()).to("cuda")
+
+
+def to_host_u16(t):
+    return t.cpu().numpy().view(np.uint16)
+
+
+def native_pool(case, nan_fill=False):
+    """Device pool in the native layout, made from the case's reference-layout pool by esp_kv_relayout."""
+    ref = dev_u16(case.pool_ref)
+    nat = torch.empty_like(ref)
+    device.kv_relayout(case.params, ref, abi.ESP_LAYOUT_REFERENCE, nat, abi.ESP_LAYOUT_NATIVE, case.n_blocks)
+    torch.cuda.synchronize()
+    return nat
+
+
+def default_options(case, workgroups=1024):
+    return host.options_mi355x(case.params.rows_per_tile, workgroups)
+
+
+def plan(case, options):
+    p = case.params
+    p.rows_per_tile = options.rows_per_tile
+    return host.plan_tiles(case.trees, p.Hkv, p.window, case.pos if p.window > 0 else None, options)
+
+
+def run_case(case, options=None, pool=None, with_desc=True):
+    """Returns O as storage bits [n_rows][H * HD]."""
+    device.init(0)
+    options = options or default_options(case)
+    tiles, jobs, n_parts = plan(case, options)
+    if pool is None:
+        pool = native_pool(case)
+    dp = device.DevicePass(case.params, case.trees, tiles, jobs, n_parts, case.n_rows, case.blocks,
+                           case.desc if with_desc else None, case.pos)
+    Q, Kb, Vb = dev_u16(case.Q), dev_u16(case.Kb), dev_u16(case.Vb)
+    O = torch.zeros_like(Q)
+    dp.run(Q, Kb, Vb, pool, O)
+    torch.cuda.synchronize()
+    return to_host_u16(O).reshape(case.n_rows, -1)

@@ -1,0 +1,75 @@
+"""The C-ABI libraries load and export every symbol the headers declare.
+No compute calls: these run without a GPU."""
+import ctypes as C
+import os
+import re
+
+from espetero_amd import abi, host
+
+ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+
+
+def _declared(header):
+    text = open(os.path.join(ROOT, "include", header)).read()
+    text = re.sub(r"/\*.*?\*/", "", text, flags=re.S)
+    return sorted(set(re.findall(r"\b(esp_[a-z0-9_]+)\s*\(", text)))
+
+
+def test_attn_library_exports_every_declared_symbol():
+    names = _declared("espetero_attn.h")
+    assert set(names) == set(abi.ATTN_SYMBOLS), "the ctypes table must name exactly what the header declares"
+    lib = C.CDLL(abi.ATTN_LIB_PATH)
+    for n in names:
+        assert hasattr(lib, n), n
+    lib.esp_attn_abi_version.restype = C.c_int
+    assert lib.esp_attn_abi_version() == abi.ESP_ABI_VERSION
+
+
+def test_engine_library_exports_every_declared_symbol():
+    names = _declared("espetero_engine.h")
+    assert set(names) == set(host.ENGINE_SYMBOLS)
+    lib = C.CDLL(abi.ENGINE_LIB_PATH)
+    for n in names:
+        assert hasattr(lib, n), n
+
+
+def test_record_layouts_match_the_reference_structs():
+    """AttnTree 16 B, tile 32 B, combine 16 B, KVSave 16 B (kernels/40_attention.metal:134-150,
+    804-809, 868-873): field order is part of the contract."""
+    assert [f[0] for f in abi.Tree._fields_] == ["base", "P", "table", "M"]
+    assert [f[0] for f in abi.Tile._fields_] == ["tree", "r0", "k0", "k1", "part", "last", "b0", "pad"]
+    assert [f[0] for f in abi.Combine._fields_] == ["r0", "rows", "part0", "nparts"]
+    assert [f[0] for f in abi.KVSave._fields_] == ["src_row", "block", "pos", "pad"]
+
+
+def test_workspace_bytes_is_host_arithmetic():
+    from espetero_amd import synth
+    lib = abi.attn_lib()
+    p = synth.make_params(32, 4, 128, abi.ESP_F16, 16, rows_per_tile=1)
+    assert lib.esp_attn_workspace_bytes(C.byref(p), 16, 0) >= 1
+    n = lib.esp_attn_workspace_bytes(C.byref(p), 16, 100)
+    assert n >= 100 * 4 * 8 * (128 + 2) * 4          # parts x Hkv x packed rows x (O, m, l) floats
+    p2 = synth.make_params(40, 8, 128, abi.ESP_BF16, 16, rows_per_tile=128)
+    n2 = lib.esp_attn_workspace_bytes(C.byref(p2), 2048, 0)
+    assert n2 >= 2048 * 8 * 128 * 2                   # the transposed staging copy of the batch V rows
+
+
+def test_argument_errors_come_back_as_codes_not_crashes():
+    """Checked on the host before any launch."""
+    from espetero_amd import synth
+    lib = abi.attn_lib()
+    err = C.create_string_buffer(256)
+    p = synth.make_params(32, 5, 128, abi.ESP_F16, 16)
+    rc = lib.esp_attn_forward(C.byref(p), None, None, None, None, None, None, None, None, None, 1, None, 1, None, 0, 0, 1,
+                              None, 0, None, err, 256)
+    assert rc == 1 and b"multiple of Hkv" in err.value
+    p = synth.make_params(32, 4, 96, abi.ESP_F16, 16)
+    rc = lib.esp_kv_save(C.byref(p), None, None, None, None, 1, None, err, 256)
+    assert rc == 2 and b"head_dim" in err.value
+    p = synth.make_params(32, 4, 128, abi.ESP_F16, 24)
+    rc = lib.esp_kv_gather(C.byref(p), None, None, 1, None, None, None, err, 256)
+    assert rc == 1 and b"multiple of 16" in err.value
+    p = synth.make_params(32, 4, 128, abi.ESP_F16, 16)
+    rc = lib.esp_attn_forward(C.byref(p), None, None, None, None, None, None, None, None, None, 1, None, 1, None, 0, 0, 1,
+                              None, 0, None, err, 256)
+    assert rc == 1 and b"must not be NULL" in err.value

@@ -1,0 +1,286 @@
+"""Host engine (C++ planner, KV pool, pass builder) against the integer
+restatement of the reference's formulas in oracle/host_oracle.py, plus the
+properties those formulas must keep. Integer work: every comparison is exact.
+"""
+import numpy as np
+import pytest
+
+from espetero_amd import abi, host
+from oracle import host_oracle as ho
+
+
+def _trees(rng, n, max_p=9000, max_m=1):
+    out, base = [], 0
+    for _ in range(n):
+        P = int(rng.integers(0, max_p))
+        M = int(rng.integers(1, max_m + 1))
+        out.append((base, P, int(rng.integers(0, 100)), M))
+        base += M
+    return out
+
+
+def _as_tuples(recs):
+    return [tuple(int(x) for x in r) for r in recs]
+
+
+# ---------------------------------------------------------------- planner, reference rule
+@pytest.mark.parametrize("seed", range(12))
+def test_reference_rule_is_bit_identical_to_plan_tiles(seed):
+    rng = np.random.default_rng(seed)
+    n = int(rng.integers(1, 20))
+    trees = _trees(rng, n, max_m=int(rng.choice([1, 1, 4, 40, 300])))
+    Hkv = int(rng.choice([1, 2, 4, 8]))
+    split = int(rng.choice([0, 256, 512, 1024]))
+    o = host.options_reference()
+    o.split = split
+    tiles, jobs, parts = host.plan_tiles(np.array(trees, abi.TREE_DT), Hkv, 0, None, o)
+    wt, wj, wp = ho.plan_tiles(trees, Hkv, split)
+    assert _as_tuples(tiles) == wt and _as_tuples(jobs) == wj and parts == wp
+    # the windowless Gemma planner is the same rule (gemma.h:77-116 with window 0)
+    gt, gj, gp, rows = ho.g4_plan_tiles(trees, Hkv, split, 0, None)
+    assert rows == 8 and _as_tuples(tiles) == gt and _as_tuples(jobs) == gj and parts == gp
+
+
+@pytest.mark.parametrize("seed", range(8))
+def test_reference_rule_with_window_matches_g4_plan_tiles(seed):
+    rng = np.random.default_rng(100 + seed)
+    trees = _trees(rng, int(rng.integers(1, 10)), max_p=20000, max_m=int(rng.choice([1, 3, 30])))
+    M = sum(t[3] for t in trees)
+    pos = np.zeros((M, 4), np.int32)
+    for base, P, _, m in trees:
+        pos[base:base + m, 0] = P + np.arange(m)
+    window = int(rng.choice([64, 1024, 4096]))
+    o = host.options_reference()
+    tiles, jobs, parts = host.plan_tiles(np.array(trees, abi.TREE_DT), 8, window, pos, o)
+    wt, wj, wp, _ = ho.g4_plan_tiles(trees, 8, 512, window, pos.reshape(-1).tolist())
+    assert _as_tuples(tiles) == wt and _as_tuples(jobs) == wj and parts == wp
+
+
+def test_reference_rule_on_the_benchmark_shapes():
+    """What the reference's planner does with its own constants on the benchmark shapes
+    (256-threadgroup target, attn_split 512, 32-key granularity)."""
+    o = host.options_reference()
+    # single decode at 1024 keys, 4 KV heads: 32 tiles of 32 keys
+    t, j, p = host.plan_tiles(np.array([(0, 1024, 0, 1)], abi.TREE_DT), 4, 0, None, o)
+    assert len(t) == 32 and p == 32 and all(int(x["k1"] - x["k0"]) == 32 for x in t) and _as_tuples(j) == [(0, 1, 0, 32)]
+    # 8 verify trees of 4 rows at 32K, 4 KV heads: 8 splits of 4096 keys each
+    trees = [(4 * i, 32768, 2048 * i, 4) for i in range(8)]
+    t, j, p = host.plan_tiles(np.array(trees, abi.TREE_DT), 4, 0, None, o)
+    assert len(t) == 64 and p == 64 and all(int(x["k1"] - x["k0"]) == 4096 for x in t)
+    assert all(int(x["nparts"]) == 8 and int(x["rows"]) == 4 for x in j)
+    # one 2048-row prefill chunk, 8 KV heads: 256 unsplit 8-row tiles
+    t, j, p = host.plan_tiles(np.array([(0, 4096, 0, 2048)], abi.TREE_DT), 8, 0, None, o)
+    assert len(t) == 256 and p == 0 and len(j) == 0 and all(int(x["part"]) == -1 and int(x["last"]) == 1 for x in t)
+
+
+# ---------------------------------------------------------------- planner, contractual algebra under any options
+@pytest.mark.parametrize("seed", range(10))
+def test_split_algebra_holds_for_both_rules(seed):
+    rng = np.random.default_rng(200 + seed)
+    trees = _trees(rng, int(rng.integers(1, 24)), max_p=40000, max_m=int(rng.choice([1, 4, 9])))
+    M = sum(t[3] for t in trees)
+    pos = np.zeros((M, 4), np.int32)
+    for base, P, _, m in trees:
+        pos[base:base + m, 0] = P + np.arange(m)
+    window = int(rng.choice([0, 0, 512]))
+    R = int(rng.choice([1, 4, 8]))
+    for o in (host.options_reference(), host.options_mi355x(R, int(rng.choice([256, 512, 1024])))):
+        tiles, jobs, parts = host.plan_tiles(np.array(trees, abi.TREE_DT), 4, window, pos if window else None, o)
+        R_ = o.rows_per_tile
+        # every (tree, row tile) is covered once; its ranges partition [k0, P); the last owns the batch keys
+        by = {}
+        for x in tiles:
+            by.setdefault((int(x["tree"]), int(x["r0"])), []).append(x)
+        want_keys = {(ti, base + r) for ti, (base, P, _, m) in enumerate(trees) for r in range(0, m, R_)}
+        assert set(by) == want_keys
+        used_parts = []
+        for (ti, r0), xs in by.items():
+            base, P, _, m = trees[ti]
+            k = int(xs[0]["k0"])
+            if window == 0:
+                assert k == 0
+            for i, x in enumerate(xs):
+                assert int(x["k0"]) == k and int(x["k1"]) > k or P == k
+                k = int(x["k1"])
+                assert int(x["last"]) == (1 if i == len(xs) - 1 else 0)
+                if len(xs) > 1:
+                    used_parts.append(int(x["part"]))
+                    if i:
+                        # reference rule: steps from k0 (gemma.h:109); balanced rule: absolute page multiples
+                        off = 0 if o.balanced else int(xs[0]["k0"])
+                        assert (int(x["k0"]) - off) % o.granule == 0
+                else:
+                    assert int(x["part"]) == -1
+            assert k == P
+        assert sorted(used_parts) == list(range(parts))
+        # merge jobs name consecutive parts in range order
+        seen = 0
+        for jb in jobs:
+            assert int(jb["part0"]) == seen and int(jb["nparts"]) >= 2
+            seen += int(jb["nparts"])
+        assert seen == parts
+
+
+def test_balanced_rule_equalises_keys_per_workgroup():
+    """16 sequences of 512..8192 keys: the reference rule gives every sequence the same
+    number of splits; the balanced rule gives every workgroup about the same key count."""
+    rng = np.random.default_rng(2)
+    lens = rng.integers(512, 8193, 16)
+    trees = np.array([(i, int(L), 0, 1) for i, L in enumerate(lens)], abi.TREE_DT)
+    ref_t, _, _ = host.plan_tiles(trees, 4, 0, None, host.options_reference())
+    bal_t, _, _ = host.plan_tiles(trees, 4, 0, None, host.options_mi355x(1, 1024))
+    ref_sz = np.array([int(x["k1"] - x["k0"]) for x in ref_t])
+    bal_sz = np.array([int(x["k1"] - x["k0"]) for x in bal_t])
+    assert ref_sz.max() / ref_sz.min() > 4
+    assert bal_sz.max() / np.median(bal_sz) < 1.3
+    assert 0.5 * 1024 / 4 <= len(bal_t) <= 1.5 * 1024 / 4
+
+
+# ---------------------------------------------------------------- pool: allocator and copy-on-write lists
+def _conservation(e, n_blocks, slots):
+    """Sum of refcounts == sum of list memberships; free + live == n_blocks."""
+    member = np.zeros(n_blocks, int)
+    for s in slots:
+        if e.slot_len(s) >= 0:
+            for b in e.slot_blocks(s):
+                member[b] += 1
+    refs = np.array([e.block_ref(b) for b in range(n_blocks)])
+    assert (refs == member).all()
+    assert e.free_blocks() + int((refs > 0).sum()) == n_blocks
+
+
+def test_allocator_hands_out_block_zero_first_and_conserves():
+    e = host.Engine(8, 16, 4)
+    s = e.slot_alloc()
+    e.pass_begin([host.make_spec(parent=-1, save=s, root_len=40)])
+    e.pass_commit()
+    assert list(e.slot_blocks(s)) == [0, 1, 2] and e.slot_len(s) == 40 and e.free_blocks() == 5
+    _conservation(e, 8, [s])
+    e.slot_reset(s)
+    assert e.free_blocks() == 8 and e.slot_len(s) == 0
+    # released blocks are reused last-in first-out (model.h:731-733)
+    e.pass_begin([host.make_spec(save=s, root_len=16)])
+    e.pass_commit()
+    assert list(e.slot_blocks(s)) == [2]
+
+
+def test_target_blocks_cases_match_the_restatement():
+    """In place with sole ownership / shared partial block (copy on write) / block-aligned append."""
+    for (P, n_new, fork, in_place) in [(40, 1, False, True), (40, 1, True, True), (40, 30, True, False), (32, 5, True, True),
+                                       (32, 5, False, True), (0, 20, False, False), (47, 1, False, True), (48, 1, False, True)]:
+        e = host.Engine(32, 16, 4)
+        pool = ho.Pool(32, 16)
+        a, b = e.slot_alloc(), e.slot_alloc()
+        parent_blocks = []
+        if P:
+            e.pass_begin([host.make_spec(save=a, root_len=P)])
+            e.pass_commit()
+            parent_blocks, _ = ho.target_blocks(pool, [], 0, 0, P, False)
+        assert list(e.slot_blocks(a)) == parent_blocks
+        if fork:
+            e.slot_fork(a, b)
+            for blk in parent_blocks:
+                pool.retain(blk)
+        dst = a if in_place else b
+        if not in_place and not fork:
+            pass
+        want_new = ho.target_new_blocks(pool, parent_blocks if P else None, P, P, P + n_new, in_place)
+        spec = host.make_spec(parent=a if P else -1, save=dst, root_len=n_new)
+        assert e.pass_blocks([spec]) == want_new
+        free0 = e.free_blocks()
+        ps = e.pass_begin([spec])
+        want_blocks, want_cow = ho.target_blocks(pool, parent_blocks, P, P, P + n_new, in_place and P > 0)
+        assert free0 - e.free_blocks() == want_new            # pass_kv_tokens == blocks actually taken
+        assert [tuple(x) for x in ps["cow"].tolist()] == want_cow
+        assert _as_tuples(ps["saves"]) == ho.kv_saves(0, P, n_new, want_blocks, 16)
+        assert list(ps["table"]) == parent_blocks[:(P + 15) // 16]
+        e.pass_commit()
+        assert list(e.slot_blocks(dst)) == want_blocks and e.slot_len(dst) == P + n_new
+        _conservation(e, 32, [a, b])
+
+
+def test_failed_pass_leaves_slots_and_pool_untouched():
+    e = host.Engine(6, 16, 4)
+    a, b = e.slot_alloc(), e.slot_alloc()
+    e.pass_begin([host.make_spec(save=a, root_len=50)])
+    e.pass_commit()
+    before = (list(e.slot_blocks(a)), e.slot_len(a), e.free_blocks())
+    with pytest.raises(abi.EspError, match="KV cache full"):
+        e.pass_begin([host.make_spec(parent=a, save=b, root_len=64)])
+    with pytest.raises(abi.EspError, match="two trees save into one slot"):
+        e.pass_begin([host.make_spec(parent=a, save=b, root_len=1), host.make_spec(parent=a, save=b, root_len=1)])
+    with pytest.raises(abi.EspError, match="work slot must differ"):
+        e.pass_begin([host.make_spec(parent=a, save=a, work=a, root_len=1)])
+    with pytest.raises(abi.EspError, match="invalid parent slot"):
+        e.pass_begin([host.make_spec(parent=3, root_len=1)])
+    with pytest.raises(abi.EspError, match="empty tree"):
+        e.pass_begin([host.make_spec(parent=a)])
+    assert (list(e.slot_blocks(a)), e.slot_len(a), e.free_blocks()) == before
+    # an aborted pass (the device work failed) gives its blocks back
+    e.pass_begin([host.make_spec(parent=a, save=b, root_len=20)])
+    assert e.free_blocks() < before[2]
+    e.pass_abort()
+    assert (list(e.slot_blocks(a)), e.slot_len(a), e.free_blocks()) == before and e.slot_len(b) == 0
+    _conservation(e, 6, [a, b])
+
+
+def test_fork_shares_blocks_and_copy_on_write_diverges():
+    e = host.Engine(16, 16, 4)
+    a, b = e.slot_alloc(), e.slot_alloc()
+    e.pass_begin([host.make_spec(save=a, root_len=40)])
+    e.pass_commit()
+    e.slot_fork(a, b)
+    assert list(e.slot_blocks(a)) == list(e.slot_blocks(b))
+    assert all(e.block_ref(x) == 2 for x in e.slot_blocks(a))
+    ps = e.pass_begin([host.make_spec(parent=a, save=a, root_len=1), host.make_spec(parent=b, save=b, root_len=1)])
+    # both partial blocks are shared: each append copies block 2 into a fresh one
+    assert len(ps["cow"]) == 2 and all(src == 2 for src, _ in ps["cow"].tolist())
+    e.pass_commit()
+    la, lb = list(e.slot_blocks(a)), list(e.slot_blocks(b))
+    assert la[:2] == lb[:2] and la[2] != lb[2] and e.block_ref(2) == 0
+    _conservation(e, 16, [a, b])
+
+
+# ---------------------------------------------------------------- rows of verify trees
+def test_leaf_hosting_and_descriptors_match_the_restatement():
+    rng = np.random.default_rng(5)
+    for _ in range(30):
+        NL = int(rng.integers(1, 6))
+        leaves = []
+        for _ in range(NL):
+            n = int(rng.integers(1, 5))
+            leaves.append([int(x) for x in rng.integers(0, 3, n)])
+        Tr = int(rng.integers(0, 4))
+        e = host.Engine(64, 16, 2)
+        s = e.slot_alloc()
+        e.pass_begin([host.make_spec(save=s, root_len=33)])
+        e.pass_commit()
+        toks = [t for lf in leaves for t in lf]
+        offs = [0]
+        for lf in leaves:
+            offs.append(offs[-1] + len(lf))
+        ps = e.pass_begin([host.make_spec(parent=s, root_len=Tr, leaves=leaves)])
+        desc, pos, M = ho.tree_rows(0, Tr, 33, toks, offs)
+        assert ps["M"] == M
+        assert ps["desc"].tolist() == [list(d) for d in desc]
+        assert ps["pos"].tolist() == [list(p) for p in pos]
+        e.pass_abort()
+
+
+def test_verify_chain_is_one_tree_of_root_plus_k_rows():
+    """MTP verify: leaf i = first i + 1 drafts; prefixes are hosted by the longest leaf, so the
+    tree has root + k rows, not k (k + 1) / 2 (forest.h:2201-2220)."""
+    e = host.Engine(64, 16, 2)
+    s = e.slot_alloc()
+    e.pass_begin([host.make_spec(save=s, root_len=100)])
+    e.pass_commit()
+    drafts = [5, 6, 7]
+    leaves = [drafts[:i + 1] for i in range(3)]
+    ps = e.pass_begin([host.make_spec(parent=s, save=s, root_len=1, leaves=leaves, commit_chain=3)])
+    assert ps["M"] == 4
+    assert ps["desc"].tolist() == [[0, 0, 0, 0], [1, 0, 1, 0], [1, 0, 1, 0], [1, 0, 1, 0]]
+    assert ps["pos"][:, 0].tolist() == [100, 101, 102, 103]
+    # root row and the chain rows are all saved at the positions they take if committed
+    assert [(int(x["src_row"]), int(x["pos"])) for x in ps["saves"]] == [(0, 4), (1, 5), (2, 6), (3, 7)]
+    e.pass_commit()
+    assert e.slot_len(s) == 101
