@@ -1,0 +1,302 @@
+#!/usr/bin/env python3
+"""Paged-KV attention benchmark on one MI355X.
+
+A step is one pass of the hot path over one batch of synthetic input, through
+the C ABI, inputs resident in HBM when the clock starts. The default workload
+is the batched paged decode (16 sequences, contexts uniform in [512, 8192],
+32 Q / 4 KV heads, head_dim 128, fp16, page 16, pages scattered over a shared
+64K-page pool); --workload picks the other benchmark shapes.
+
+Prints ONE JSON line: whole-job throughput (`value`), the roofline of the
+dominant kernel measured with HIP events on the launch stream, and the CPU
+checker timed on a bounded sample of the same workload on the host cores.
+"""
+import argparse
+import json
+import os
+import sys
+import time
+
+import numpy as np
+
+ROOT = os.path.dirname(os.path.abspath(__file__))
+if ROOT not in sys.path:
+    sys.path.insert(0, ROOT)
+
+HBM_PEAK_GBS = 8000.0        # MI355X HBM3E
+MFMA_PEAK_TFLOPS = 2500.0    # dense fp16 / bf16
+N_CU = 256
+
+
+class Workload:
+    """Device-resident inputs of one benchmark shape plus the planned passes."""
+
+    def __init__(self, name, H, Hkv, HD, dtype, bt, seqs, window=0, rows_per_tile=1, desc_fn=None, pool_pages=65536,
+                 seed=0, workgroups=None, bound="hbm"):
+        import torch
+        from espetero_amd import abi, device, host, synth
+        self.torch, self.abi, self.device, self.host = torch, abi, device, host
+        self.name, self.bound, self.dtype = name, bound, dtype
+        self.H, self.Hkv, self.HD, self.bt, self.window = H, Hkv, HD, bt, window
+        self.seqs = list(seqs)
+        p = synth.make_params(H, Hkv, HD, dtype, bt, window=window, rows_per_tile=rows_per_tile)
+        self.params = p
+        tdt = torch.float16 if dtype == abi.ESP_F16 else torch.bfloat16
+        g = torch.Generator(device="cuda")
+        g.manual_seed(seed)
+        page_elems = 2 * bt * Hkv * HD
+        pages_per_set = sum((P + M + bt - 1) // bt for P, M in self.seqs)
+        self.n_sets = max(1, min(16, pool_pages // max(pages_per_set, 1)))
+        self.pool_pages = max(pool_pages, pages_per_set)
+        # The pool holds N(0, 1) * 0.5 everywhere: any page is a valid K / V page in the native layout.
+        self.pool = torch.empty(self.pool_pages * page_elems, dtype=tdt, device="cuda")
+        chunk = 1 << 26
+        for s in range(0, self.pool.numel(), chunk):
+            n = min(chunk, self.pool.numel() - s)
+            self.pool[s:s + n] = (torch.randn(n, generator=g, device="cuda", dtype=torch.float32) * 0.5).to(tdt)
+        n_rows = sum(M for _, M in self.seqs)
+        self.n_rows = n_rows
+        self.Q = (torch.randn(n_rows, H * HD, generator=g, device="cuda") * 0.5).to(tdt)
+        self.Kb = (torch.randn(n_rows, Hkv * HD, generator=g, device="cuda") * 0.5).to(tdt)
+        self.Vb = (torch.randn(n_rows, Hkv * HD, generator=g, device="cuda") * 0.5).to(tdt)
+        self.O = torch.zeros_like(self.Q)
+        # rows, trees, descriptors
+        trees = np.zeros(len(self.seqs), abi.TREE_DT)
+        desc = np.zeros((n_rows, 4), np.int32)
+        pos = np.zeros((n_rows, 4), np.int32)
+        base, tab = 0, 0
+        for i, (P, M) in enumerate(self.seqs):
+            trees[i] = (base, P, tab, M)
+            pos[base:base + M, :3] = (P + np.arange(M))[:, None]
+            if desc_fn is not None:
+                desc[base:base + M] = desc_fn(M)
+            base += M
+            tab += (P + M + bt - 1) // bt
+        self.trees, self.desc, self.pos = trees, desc, pos
+        wg = workgroups or 4 * N_CU
+        opts = host.options_mi355x(rows_per_tile, wg)
+        self.tiles, self.jobs, self.n_parts = host.plan_tiles(trees, Hkv, window, pos if window > 0 else None, opts)
+        # Block tables: disjoint slices of one seeded permutation of the pool, one slice per
+        # rotation set, so a step never finds the previous step's pages in a cache.
+        perm = np.random.default_rng(seed + 1).permutation(self.pool_pages).astype(np.int32)
+        self.tables = [perm[s * pages_per_set:(s + 1) * pages_per_set].copy() for s in range(self.n_sets)]
+        self.passes = [device.DevicePass(p, trees, self.tiles, self.jobs, self.n_parts, n_rows, t,
+                                         desc if desc_fn is not None else None, pos if window > 0 else None)
+                       for t in self.tables]
+        # algorithmic work: every visible K and V element once + Q + O + block-table entries; visible (q, k) pairs
+        es = 2
+        vis_keys, pairs = 0, 0
+        for P, M in self.seqs:
+            for r in range(M):
+                lo = max(0, P + r - window + 1) if window > 0 else 0
+                pairs += (P + r + 1) - lo
+            lo = max(0, P - window + 1) if window > 0 else 0
+            vis_keys += (P + M) - lo
+        self.alg_bytes = vis_keys * Hkv * HD * 2 * es + 2 * n_rows * H * HD * es + ((vis_keys + bt - 1) // bt) * 4
+        self.alg_flops = 4 * HD * H * pairs
+
+    def step(self, i, ev=None):
+        """Enqueue one pass. ev: (start, end) events bracketing the dominant kernel's call."""
+        dp = self.passes[i % self.n_sets]
+        if ev:
+            ev[0].record()
+        dp.run(self.Q, self.Kb, self.Vb, self.pool, self.O, merge=False)
+        if ev:
+            ev[1].record()
+        dp.merge(self.O)
+
+
+def make_workload(name, workgroups=None):
+    from espetero_amd import abi, synth
+    from functools import partial
+    F16, BF16 = abi.ESP_F16, abi.ESP_BF16
+    Workload_ = partial(Workload, workgroups=workgroups)
+    if name == "c1_single_decode":
+        return Workload_(name, 32, 4, 128, F16, 16, [(1024, 1)], pool_pages=64 * 16, seed=1)
+    if name == "c2_batched_decode":
+        lens = synth.c2_lengths()
+        return Workload_(name, 32, 4, 128, F16, 16, [(L, 1) for L in lens], pool_pages=65536, seed=2)
+    if name == "c4_decode_sliding":
+        return Workload_(name, 16, 8, 256, F16, 16, [(16384, 1)] * 8, window=1024, pool_pages=8 * 1025 * 4, seed=4)
+    if name == "c4_decode_global":
+        return Workload_(name, 16, 8, 256, F16, 16, [(16384, 1)] * 8, pool_pages=8 * 1025 * 4, seed=4)
+    if name == "c5_verify":
+        return Workload_(name, 32, 4, 128, F16, 16, [(32768, 4)] * 8, rows_per_tile=4,
+                        desc_fn=lambda M: synth.verify_desc(M, 1), pool_pages=65536 + 64, seed=5)
+    if name.startswith("c3_prefill_p"):
+        P = int(name[len("c3_prefill_p"):])
+        return Workload_(name, 40, 8, 128, BF16, 16, [(P, 2048)], rows_per_tile=128, pool_pages=1024, seed=3, bound="mfma")
+    if name == "c4_prefill_sliding":
+        return Workload_(name, 16, 8, 256, F16, 16, [(15360, 1024)] * 8, window=1024, rows_per_tile=128,
+                        pool_pages=8 * 1024 * 2, seed=4, bound="mfma")
+    if name == "c4_prefill_global":
+        return Workload_(name, 16, 8, 256, F16, 16, [(15360, 1024)] * 8, rows_per_tile=128, pool_pages=8 * 1024 * 2, seed=4,
+                        bound="mfma")
+    raise SystemExit(f"unknown workload {name}")
+
+
+WORKLOADS = ["c1_single_decode", "c2_batched_decode", "c3_prefill_p0", "c3_prefill_p2048", "c3_prefill_p4096",
+             "c3_prefill_p6144", "c4_decode_sliding", "c4_decode_global", "c4_prefill_sliding", "c4_prefill_global",
+             "c5_verify"]
+
+
+def cpu_baseline(w, budget_s=20.0):
+    """The CPU checker (scalar C restatement of the reference semantics) on a bounded sample of
+    the same workload: whole sequences, gathered from the device pool through esp_kv_gather into a
+    reference-layout pool. Timed single-threaded; the all-core time is reported beside it."""
+    import torch
+    from espetero_amd import abi, device, synth
+    from oracle import binding as ob
+    p = w.params
+    kvw = p.Hkv * p.head_dim
+    # ~0.35 GFLOP/s scalar with storage conversions: size the sample to the budget
+    flops_budget = 0.35e9 * budget_s
+    seqs, tot = [], 0.0
+    for i, (P, M) in enumerate(w.seqs):
+        rows = min(M, max(1, int(flops_budget // max(1.0, 4.0 * p.head_dim * p.H * (P + M)))))
+        f = 4.0 * p.head_dim * p.H * rows * (P + rows)
+        if seqs and tot + f > flops_budget:
+            break
+        seqs.append((i, P, rows))
+        tot += f
+    bt = p.bt
+    n_blocks = sum((P + bt - 1) // bt for _, P, _ in seqs) + 1
+    pool_ref = np.zeros(n_blocks * 2 * bt * kvw, np.uint16)
+    pv = pool_ref.reshape(n_blocks, 2, bt, kvw)
+    trees = np.zeros(len(seqs), abi.TREE_DT)
+    table, nb_used, base = [], 0, 0
+    table_dev = w.passes[0].blocks
+    rows_total = sum(r for _, _, r in seqs)
+    Q = np.zeros((rows_total, p.q_ld), np.uint16)
+    Kb = np.zeros((rows_total, p.kv_ld), np.uint16)
+    Vb = np.zeros((rows_total, p.kv_ld), np.uint16)
+    desc = np.zeros((rows_total, 4), np.int32)
+    pos = np.zeros((rows_total, 4), np.int32)
+    for (i, P, rows) in seqs:
+        t = w.trees[i]
+        nb = (P + bt - 1) // bt
+        if P:
+            K = torch.zeros(P * kvw, dtype=torch.int16, device="cuda")
+            V = torch.zeros_like(K)
+            device.kv_gather(p, w.pool, table_dev[int(t["table"]):], P, K, V)
+            torch.cuda.synchronize()
+            Kh = np.zeros((nb * bt, kvw), np.uint16)
+            Vh = np.zeros((nb * bt, kvw), np.uint16)
+            Kh[:P] = K.cpu().numpy().view(np.uint16).reshape(P, kvw)
+            Vh[:P] = V.cpu().numpy().view(np.uint16).reshape(P, kvw)
+            pv[nb_used:nb_used + nb, 0] = Kh.reshape(nb, bt, kvw)
+            pv[nb_used:nb_used + nb, 1] = Vh.reshape(nb, bt, kvw)
+        idx = [k for k, s in enumerate(seqs) if s[0] == i][0]
+        trees[idx] = (base, P, len(table), rows)
+        table.extend(range(nb_used, nb_used + nb))
+        nb_used += nb
+        b0 = int(t["base"])
+        Q[base:base + rows] = w.Q[b0:b0 + rows].view(torch.int16).cpu().numpy().view(np.uint16)
+        Kb[base:base + rows] = w.Kb[b0:b0 + rows].view(torch.int16).cpu().numpy().view(np.uint16)
+        Vb[base:base + rows] = w.Vb[b0:b0 + rows].view(torch.int16).cpu().numpy().view(np.uint16)
+        desc[base:base + rows] = w.desc[b0:b0 + rows]
+        pos[base:base + rows] = w.pos[b0:b0 + rows]
+        base += rows
+    blocks = np.asarray(table if table else [0], np.int32)
+    pr = synth.make_params(p.H, p.Hkv, p.head_dim, p.dtype, bt, window=p.window, rows_per_tile=p.rows_per_tile)
+    # work of the sample, counted as for the GPU
+    vis_keys, pairs = 0, 0
+    for _, P, rows in seqs:
+        for r in range(rows):
+            lo = max(0, P + r - p.window + 1) if p.window > 0 else 0
+            pairs += (P + r + 1) - lo
+        lo = max(0, P - p.window + 1) if p.window > 0 else 0
+        vis_keys += (P + rows) - lo
+    s_bytes = vis_keys * kvw * 2 * 2 + 2 * rows_total * p.H * p.head_dim * 2 + ((vis_keys + bt - 1) // bt) * 4
+    s_flops = 4 * p.head_dim * p.H * pairs
+    t0 = time.perf_counter()
+    o1 = ob.attn_direct(pr, Q, Kb, Vb, pool_ref, blocks, desc, pos, trees, n_threads=1)
+    t1 = time.perf_counter() - t0
+    ncores = min(16, os.cpu_count() or 1)
+    t0 = time.perf_counter()
+    ob.attn_direct(pr, Q, Kb, Vb, pool_ref, blocks, desc, pos, trees, n_threads=ncores)
+    tn = time.perf_counter() - t0
+    # the sample doubles as a parity spot check of the benchmarked device path
+    max_err = None
+    if all(rows == M for (_, _, rows), (_, M) in zip(seqs, [w.seqs[i] for i, _, _ in seqs])):
+        got = w.O.view(torch.int16).cpu().numpy().view(np.uint16)
+        errs = []
+        base = 0
+        for (i, P, rows) in seqs:
+            b0 = int(w.trees[i]["base"])
+            errs.append(np.abs(ob.to_f32(got[b0:b0 + rows], p.dtype) - ob.to_f32(o1[base:base + rows], p.dtype)).max())
+            base += rows
+        max_err = float(max(errs))
+    unit = "GB/s" if w.bound == "hbm" else "TFLOP/s"
+    val1 = s_bytes / t1 / 1e9 if w.bound == "hbm" else s_flops / t1 / 1e12
+    valn = s_bytes / tn / 1e9 if w.bound == "hbm" else s_flops / tn / 1e12
+    return {"value": round(val1, 6), "unit": unit, "cores": 1, "kind": "port",
+            "sample": f"{len(seqs)} of {len(w.seqs)} sequences ({rows_total} rows, {vis_keys} visible keys), "
+                      f"{t1:.2f} s single-threaded",
+            "all_cores": {"value": round(valn, 6), "cores": ncores, "seconds": round(tn, 3)},
+            "host_cpus": os.cpu_count(), "max_abs_err_vs_gpu": max_err}
+
+
+def main():
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=200)
+    ap.add_argument("--warmup", type=int, default=20)
+    ap.add_argument("--workload", default="c2_batched_decode", help="one of: " + ", ".join(WORKLOADS))
+    ap.add_argument("--workgroups", type=int, default=0, help="planner split target (0: 4 per CU)")
+    ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
+    args = ap.parse_args()
+    if args.gpus != 1:
+        raise SystemExit("bench.py measures one GPU: this path has no multi-GPU leg (run with --gpus 1)")
+
+    import torch
+    from espetero_amd import abi, device
+    assert torch.cuda.is_available(), "bench.py needs a GPU"
+    device.init(0)
+    w = make_workload(args.workload, args.workgroups or None)
+    K, W = args.steps, args.warmup
+    for i in range(W):
+        w.step(i)
+    torch.cuda.synchronize()
+    evs = [(torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)) for _ in range(K)]
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    for i in range(K):
+        w.step(W + i, evs[i])
+    torch.cuda.synchronize()
+    wall = (time.perf_counter() - t0) / K
+    kern_ms = float(np.mean([a.elapsed_time(b) for a, b in evs]))
+    kern_min_ms = float(np.min([a.elapsed_time(b) for a, b in evs]))
+
+    if w.bound == "hbm":
+        metric, unit = "decode-attn HBM GB/s", "GB/s"
+        value = w.alg_bytes / wall / 1e9
+        achieved, peak = w.alg_bytes / (kern_ms * 1e-3) / 1e9, HBM_PEAK_GBS
+    else:
+        metric, unit = "prefill-attn TFLOPS", "TFLOP/s"
+        value = w.alg_flops / wall / 1e12
+        achieved, peak = w.alg_flops / (kern_ms * 1e-3) / 1e12, MFMA_PEAK_TFLOPS
+    out = {
+        "metric": metric, "value": round(value, 3), "unit": unit, "n_gpus": 1, "steps": K, "warmup": W,
+        "ms_per_step": round(wall * 1e3, 6), "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
+        "dtype": "f16" if w.dtype == abi.ESP_F16 else "bf16", "data": "synthetic",
+        "config": {"workload": w.name, "sequences": len(w.seqs), "rows": w.n_rows, "H": w.H, "Hkv": w.Hkv,
+                   "head_dim": w.HD, "page": w.bt, "window": w.window, "context_tokens": int(sum(P for P, _ in w.seqs)),
+                   "tiles": int(len(w.tiles)), "parts": int(w.n_parts), "rotation_sets": w.n_sets,
+                   "pool_pages": w.pool_pages},
+        "roofline": {"bound": w.bound, "achieved": round(achieved, 3), "peak": peak, "unit": unit,
+                     "frac": round(achieved / peak, 4), "traffic": None,
+                     "kernel": "attn_stream_kernel" if w.bound == "hbm" and w.params.rows_per_tile * (w.H // w.Hkv) <= 32
+                     else "attn_tiled_kernel",
+                     "kernel_us_avg": round(kern_ms * 1e3, 3), "kernel_us_min": round(kern_min_ms * 1e3, 3),
+                     "alg_bytes": int(w.alg_bytes), "alg_flops": int(w.alg_flops)},
+    }
+    if not args.no_cpu:
+        w.step(0)   # leave rotation set 0's output in O: the CPU sample is checked against it
+        torch.cuda.synchronize()
+        out["cpu_baseline"] = cpu_baseline(w)
+    print(json.dumps(out), flush=True)
+
+
+if __name__ == "__main__":
+    main()

@@ -77,6 +77,33 @@ Carve carve(const esp_attn_params* p, int n_rows, int n_parts) {
   return c;
 }
 
+esp::KArgs make_args(const esp_attn_params* p, const Carve& c, void* workspace, int n_rows) {
+  char* ws = static_cast<char*>(workspace);
+  esp::KArgs a{};
+  a.parts_o = reinterpret_cast<float*>(ws + c.parts_o);
+  a.parts_ml = reinterpret_cast<float*>(ws + c.parts_ml);
+  a.vt_stage = reinterpret_cast<uint16_t*>(ws + c.vt_stage);
+  a.gate = p->gate;
+  a.gate_ld = p->gate_ld;
+  a.gate_hs = p->gate_hs;
+  a.gate_off = p->gate_off;
+  a.H = p->H;
+  a.Hkv = p->Hkv;
+  a.G = p->H / p->Hkv;
+  a.q_ld = p->q_ld;
+  a.kv_ld = p->kv_ld;
+  a.bt = p->bt;
+  a.window = p->window;
+  a.ring = p->ring;
+  a.bidi = p->bidi;
+  a.R = p->rows_per_tile;
+  a.cols = a.R * a.G;
+  a.n_rows = n_rows;
+  a.scale_log2 = p->scale * esp::kLog2e;
+  a.kv_base = p->kv_base;
+  return a;
+}
+
 }  // namespace
 
 extern "C" {
@@ -111,7 +138,7 @@ int esp_attn_forward(const esp_attn_params* p, const void* Q, const void* Kb, co
   if (p->window > 0 && !pos) return fail(err, errlen, ESP_EINVAL, "pos is NULL on a sliding-window layer");
   if (p->rows_per_tile <= 0) return fail(err, errlen, ESP_EINVAL, "rows_per_tile %d", p->rows_per_tile);
   if (n_jobs > 0 && !jobs) return fail(err, errlen, ESP_EINVAL, "jobs is NULL");
-  if ((n_jobs > 0) != (n_parts > 0)) return fail(err, errlen, ESP_EINVAL, "n_jobs %d and n_parts %d disagree", n_jobs, n_parts);
+  if (n_jobs > 0 && n_parts == 0) return fail(err, errlen, ESP_EINVAL, "n_jobs %d without partial records", n_jobs);
   if (!(p->scale > 0.0f)) return fail(err, errlen, ESP_EINVAL, "scale must be positive");
   const int fam = family(p);
   if (fam < 0 && p->rows_per_tile > 128)
@@ -122,8 +149,7 @@ int esp_attn_forward(const esp_attn_params* p, const void* Q, const void* Kb, co
   if (reinterpret_cast<uintptr_t>(workspace) % 16) return fail(err, errlen, ESP_EINVAL, "workspace must be 16-byte aligned");
 
   hipStream_t st = static_cast<hipStream_t>(stream);
-  char* ws = static_cast<char*>(workspace);
-  esp::KArgs a{};
+  esp::KArgs a = make_args(p, c, workspace, n_rows);
   a.Q = static_cast<const uint16_t*>(Q);
   a.Kb = static_cast<const uint16_t*>(Kb);
   a.Vb = static_cast<const uint16_t*>(Vb);
@@ -134,27 +160,6 @@ int esp_attn_forward(const esp_attn_params* p, const void* Q, const void* Kb, co
   a.O = static_cast<uint16_t*>(O);
   a.tiles = tiles;
   a.trees = trees;
-  a.parts_o = reinterpret_cast<float*>(ws + c.parts_o);
-  a.parts_ml = reinterpret_cast<float*>(ws + c.parts_ml);
-  a.vt_stage = reinterpret_cast<uint16_t*>(ws + c.vt_stage);
-  a.gate = p->gate;
-  a.gate_ld = p->gate_ld;
-  a.gate_hs = p->gate_hs;
-  a.gate_off = p->gate_off;
-  a.H = p->H;
-  a.Hkv = p->Hkv;
-  a.G = p->H / p->Hkv;
-  a.q_ld = p->q_ld;
-  a.kv_ld = p->kv_ld;
-  a.bt = p->bt;
-  a.window = p->window;
-  a.ring = p->ring;
-  a.bidi = p->bidi;
-  a.R = p->rows_per_tile;
-  a.cols = a.R * a.G;
-  a.n_rows = n_rows;
-  a.scale_log2 = p->scale * esp::kLog2e;
-  a.kv_base = p->kv_base;
 
   hipError_t e;
   if (fam > 0) {
@@ -173,6 +178,23 @@ int esp_attn_forward(const esp_attn_params* p, const void* Q, const void* Kb, co
     if (e != hipSuccess) return hip_fail(err, errlen, "attn_combine launch", e);
   }
   return ESP_OK;
+}
+
+int esp_attn_combine(const esp_attn_params* p, void* O, const esp_combine* jobs, int32_t n_jobs, int32_t n_parts,
+                     int32_t n_rows, void* workspace, size_t workspace_bytes, void* stream, char* err, size_t errlen) {
+  if (int rc = check_params(p, err, errlen)) return rc;
+  if (n_jobs < 0 || n_parts < 0 || n_rows < 0) return fail(err, errlen, ESP_EINVAL, "negative count");
+  if (n_jobs == 0) return ESP_OK;
+  if (!O || !jobs) return fail(err, errlen, ESP_EINVAL, "O and jobs must not be NULL");
+  if (n_parts == 0) return fail(err, errlen, ESP_EINVAL, "n_jobs %d without partial records", n_jobs);
+  if (p->rows_per_tile <= 0) return fail(err, errlen, ESP_EINVAL, "rows_per_tile %d", p->rows_per_tile);
+  const Carve c = carve(p, n_rows, n_parts);
+  if (!workspace || workspace_bytes < c.total)
+    return fail(err, errlen, ESP_EWORKSPACE, "workspace %zu bytes, %zu needed", workspace_bytes, c.total);
+  esp::KArgs a = make_args(p, c, workspace, n_rows);
+  a.O = static_cast<uint16_t*>(O);
+  hipError_t e = esp::launch_combine(p->dtype, p->head_dim, a, jobs, n_jobs, static_cast<hipStream_t>(stream));
+  return e == hipSuccess ? ESP_OK : hip_fail(err, errlen, "attn_combine launch", e);
 }
 
 int esp_kv_save(const esp_attn_params* p, const void* Kb, const void* Vb, void* kv_pool, const esp_kvsave* entries,

@@ -53,6 +53,12 @@ def forward(params, Q, Kb, Vb, pool, blocks, desc, pos, O, tiles, n_tiles, trees
     abi.check(rc, err)
 
 
+def combine(params, O, jobs, n_jobs, n_parts, n_rows, workspace, stream=None):
+    err = C.create_string_buffer(_ERRLEN)
+    abi.check(abi.attn_lib().esp_attn_combine(C.byref(params), _ptr(O), _ptr(jobs), n_jobs, n_parts, n_rows, _ptr(workspace),
+                                              workspace.numel() * workspace.element_size(), _stream(stream), err, _ERRLEN), err)
+
+
 def kv_save(params, Kb, Vb, pool, entries, n_entries, stream=None):
     err = C.create_string_buffer(_ERRLEN)
     abi.check(abi.attn_lib().esp_kv_save(C.byref(params), _ptr(Kb), _ptr(Vb), _ptr(pool), _ptr(entries), n_entries,
@@ -94,6 +100,11 @@ class DevicePass:
         nbytes = workspace_bytes(params, n_rows, n_parts)
         self.workspace = torch.empty(nbytes, dtype=torch.uint8, device=device)
 
-    def run(self, Q, Kb, Vb, pool, O, stream=None):
+    def run(self, Q, Kb, Vb, pool, O, stream=None, merge=True):
         forward(self.params, Q, Kb, Vb, pool, self.blocks, self.desc, self.pos, O, self.tiles, self.n_tiles, self.trees,
-                self.n_trees, self.jobs, self.n_jobs, self.n_parts, self.n_rows, self.workspace, stream)
+                self.n_trees, self.jobs if merge else None, self.n_jobs if merge else 0, self.n_parts, self.n_rows,
+                self.workspace, stream)
+
+    def merge(self, O, stream=None):
+        if self.n_jobs:
+            combine(self.params, O, self.jobs, self.n_jobs, self.n_parts, self.n_rows, self.workspace, stream)

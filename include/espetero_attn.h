@@ -128,13 +128,21 @@ size_t esp_attn_workspace_bytes(const esp_attn_params* p, int32_t n_rows, int32_
  * desc/pos: int32[4] per row (desc = seg_start, 0, anc_len, img_end; pos.x =
  * position); desc may be NULL (plain causal rows), pos may be NULL when
  * window == 0. O [n_rows][q_ld]. The kernel family is chosen from
- * rows_per_tile * G (streaming split-K kernel up to 64 packed rows, tiled
- * MFMA kernel above), as the reference chooses from its plan (forest.h:2863-2868). */
+ * rows_per_tile * G (streaming split-K kernel up to 32 packed rows, tiled
+ * MFMA kernel above), as the reference chooses from its plan (forest.h:2863-2868).
+ * n_jobs = 0 with n_parts > 0 skips the merge (see esp_attn_combine). */
 int esp_attn_forward(const esp_attn_params* p, const void* Q, const void* Kb, const void* Vb, const void* kv_pool,
                      const int32_t* blocks, const int32_t* desc, const int32_t* pos, void* O, const esp_tile* tiles,
                      int32_t n_tiles, const esp_tree* trees, int32_t n_trees, const esp_combine* jobs, int32_t n_jobs,
                      int32_t n_parts, int32_t n_rows, void* workspace, size_t workspace_bytes, void* stream, char* err,
                      size_t errlen);
+
+/* The split-K merge alone: attention_combine (40_:811-864, 80_:568-597) as its
+ * own dispatch, for callers that passed n_jobs = 0 to esp_attn_forward (a
+ * plan with n_parts > 0 then leaves its partial records in `workspace`). Same
+ * params, O, workspace and counts as that call. */
+int esp_attn_combine(const esp_attn_params* p, void* O, const esp_combine* jobs, int32_t n_jobs, int32_t n_parts,
+                     int32_t n_rows, void* workspace, size_t workspace_bytes, void* stream, char* err, size_t errlen);
 
 /* Append batch rows to the pool: replaces kv_save (40_:875-889; forest.h:2935-2947). */
 int esp_kv_save(const esp_attn_params* p, const void* Kb, const void* Vb, void* kv_pool, const esp_kvsave* entries,
@@ -153,7 +161,8 @@ int esp_kv_gather(const esp_attn_params* p, const void* kv_pool, const int32_t* 
                   void* V_out, void* stream, char* err, size_t errlen);
 
 /* Convert n_blocks whole blocks of one layer region between the reference's
- * block layout and the native one (src and dst regions must not overlap).
+ * block layout and the native one. src_pool / dst_pool point at the first
+ * block of the region (kv_base is not applied); they must not overlap.
  * src_layout / dst_layout: ESP_LAYOUT_*. Bit copy. */
 int esp_kv_relayout(const esp_attn_params* p, const void* src_pool, int32_t src_layout, void* dst_pool, int32_t dst_layout,
                     int32_t n_blocks, void* stream, char* err, size_t errlen);
