@@ -32,7 +32,7 @@ class Workload:
     """Device-resident inputs of one benchmark shape plus the planned passes."""
 
     def __init__(self, name, H, Hkv, HD, dtype, bt, seqs, window=0, rows_per_tile=1, desc_fn=None, pool_pages=65536,
-                 seed=0, workgroups=None, bound="hbm"):
+                 seed=0, workgroups=None, bound="hbm", contiguous=False):
         import torch
         from espetero_amd import abi, device, host, synth
         self.torch, self.abi, self.device, self.host = torch, abi, device, host
@@ -73,12 +73,14 @@ class Workload:
             base += M
             tab += (P + M + bt - 1) // bt
         self.trees, self.desc, self.pos = trees, desc, pos
-        wg = workgroups or 4 * N_CU
+        wg = workgroups or device.plan_hint(p)
         opts = host.options_mi355x(rows_per_tile, wg)
         self.tiles, self.jobs, self.n_parts = host.plan_tiles(trees, Hkv, window, pos if window > 0 else None, opts)
         # Block tables: disjoint slices of one seeded permutation of the pool, one slice per
         # rotation set, so a step never finds the previous step's pages in a cache.
         perm = np.random.default_rng(seed + 1).permutation(self.pool_pages).astype(np.int32)
+        if contiguous:  # experiment: pages in address order
+            perm = np.arange(self.pool_pages, dtype=np.int32)
         self.tables = [perm[s * pages_per_set:(s + 1) * pages_per_set].copy() for s in range(self.n_sets)]
         self.passes = [device.DevicePass(p, trees, self.tiles, self.jobs, self.n_parts, n_rows, t,
                                          desc if desc_fn is not None else None, pos if window > 0 else None)
@@ -106,31 +108,31 @@ class Workload:
         dp.merge(self.O)
 
 
-def make_workload(name, workgroups=None):
+def make_workload(name, workgroups=None, contiguous=False, page=16):
     from espetero_amd import abi, synth
     from functools import partial
     F16, BF16 = abi.ESP_F16, abi.ESP_BF16
-    Workload_ = partial(Workload, workgroups=workgroups)
+    Workload_ = partial(Workload, workgroups=workgroups, contiguous=contiguous)
     if name == "c1_single_decode":
-        return Workload_(name, 32, 4, 128, F16, 16, [(1024, 1)], pool_pages=64 * 16, seed=1)
+        return Workload_(name, 32, 4, 128, F16, page, [(1024, 1)], pool_pages=(64 * 16) * 16 // page, seed=1)
     if name == "c2_batched_decode":
         lens = synth.c2_lengths()
-        return Workload_(name, 32, 4, 128, F16, 16, [(L, 1) for L in lens], pool_pages=65536, seed=2)
+        return Workload_(name, 32, 4, 128, F16, page, [(L, 1) for L in lens], pool_pages=(65536) * 16 // page, seed=2)
     if name == "c4_decode_sliding":
-        return Workload_(name, 16, 8, 256, F16, 16, [(16384, 1)] * 8, window=1024, pool_pages=8 * 1025 * 4, seed=4)
+        return Workload_(name, 16, 8, 256, F16, page, [(16384, 1)] * 8, window=1024, pool_pages=(8 * 1025 * 4) * 16 // page, seed=4)
     if name == "c4_decode_global":
-        return Workload_(name, 16, 8, 256, F16, 16, [(16384, 1)] * 8, pool_pages=8 * 1025 * 4, seed=4)
+        return Workload_(name, 16, 8, 256, F16, page, [(16384, 1)] * 8, pool_pages=(8 * 1025 * 4) * 16 // page, seed=4)
     if name == "c5_verify":
-        return Workload_(name, 32, 4, 128, F16, 16, [(32768, 4)] * 8, rows_per_tile=4,
-                        desc_fn=lambda M: synth.verify_desc(M, 1), pool_pages=65536 + 64, seed=5)
+        return Workload_(name, 32, 4, 128, F16, page, [(32768, 4)] * 8, rows_per_tile=4,
+                        desc_fn=lambda M: synth.verify_desc(M, 1), pool_pages=(65536 + 64) * 16 // page, seed=5)
     if name.startswith("c3_prefill_p"):
         P = int(name[len("c3_prefill_p"):])
-        return Workload_(name, 40, 8, 128, BF16, 16, [(P, 2048)], rows_per_tile=128, pool_pages=1024, seed=3, bound="mfma")
+        return Workload_(name, 40, 8, 128, BF16, page, [(P, 2048)], rows_per_tile=128, pool_pages=(1024) * 16 // page, seed=3, bound="mfma")
     if name == "c4_prefill_sliding":
-        return Workload_(name, 16, 8, 256, F16, 16, [(15360, 1024)] * 8, window=1024, rows_per_tile=128,
-                        pool_pages=8 * 1024 * 2, seed=4, bound="mfma")
+        return Workload_(name, 16, 8, 256, F16, page, [(15360, 1024)] * 8, window=1024, rows_per_tile=128,
+                        pool_pages=(8 * 1024 * 2) * 16 // page, seed=4, bound="mfma")
     if name == "c4_prefill_global":
-        return Workload_(name, 16, 8, 256, F16, 16, [(15360, 1024)] * 8, rows_per_tile=128, pool_pages=8 * 1024 * 2, seed=4,
+        return Workload_(name, 16, 8, 256, F16, page, [(15360, 1024)] * 8, rows_per_tile=128, pool_pages=(8 * 1024 * 2) * 16 // page, seed=4,
                         bound="mfma")
     raise SystemExit(f"unknown workload {name}")
 
@@ -243,7 +245,10 @@ def main():
     ap.add_argument("--steps", type=int, default=200)
     ap.add_argument("--warmup", type=int, default=20)
     ap.add_argument("--workload", default="c2_batched_decode", help="one of: " + ", ".join(WORKLOADS))
-    ap.add_argument("--workgroups", type=int, default=0, help="planner split target (0: 4 per CU)")
+    ap.add_argument("--workgroups", type=int, default=0, help="planner split target (0: ask esp_attn_plan_hint)")
+    ap.add_argument("--tables", default="scattered", choices=["scattered", "contiguous"],
+                    help="block tables: a seeded permutation of the pool (the benchmark's definition) or address order")
+    ap.add_argument("--page", type=int, default=16, help="tokens per KV block (the benchmark's definition: 16)")
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
     args = ap.parse_args()
     if args.gpus != 1:
@@ -253,7 +258,7 @@ def main():
     from espetero_amd import abi, device
     assert torch.cuda.is_available(), "bench.py needs a GPU"
     device.init(0)
-    w = make_workload(args.workload, args.workgroups or None)
+    w = make_workload(args.workload, args.workgroups or None, args.tables == "contiguous", args.page)
     K, W = args.steps, args.warmup
     for i in range(W):
         w.step(i)

@@ -19,6 +19,8 @@ hipError_t launch_kv_gather(const esp_attn_params* p, const void* pool, const in
 hipError_t launch_kv_relayout(const esp_attn_params* p, const void* src, void* dst, int to_native, int n_blocks,
                               hipStream_t st);
 hipError_t launch_vt_stage(const esp_attn_params* p, const void* Vb, void* vt, int n_rows, hipStream_t st);
+int stream_workgroups_per_cu(int HD, int NC);
+int tiled_workgroups_per_cu(int HD);
 }  // namespace esp
 
 namespace {
@@ -116,6 +118,17 @@ int esp_attn_init(int device, char* err, size_t errlen) {
   if (e != hipSuccess) return hip_fail(err, errlen, "hipGetDeviceProperties", e);
   if (strncmp(prop.gcnArchName, "gfx950", 6) != 0)
     return fail(err, errlen, ESP_EUNSUPPORTED, "device %d is %s; this library is built for gfx950 only", device, prop.gcnArchName);
+  return ESP_OK;
+}
+
+int esp_attn_plan_hint(const esp_attn_params* p, int device, int32_t* workgroups, char* err, size_t errlen) {
+  if (int rc = check_params(p, err, errlen)) return rc;
+  if (!workgroups || p->rows_per_tile <= 0) return fail(err, errlen, ESP_EINVAL, "workgroups is NULL or rows_per_tile <= 0");
+  int cus = 0;
+  hipError_t e = hipDeviceGetAttribute(&cus, hipDeviceAttributeMultiprocessorCount, device);
+  if (e != hipSuccess) return hip_fail(err, errlen, "hipDeviceGetAttribute", e);
+  const int fam = family(p);
+  *workgroups = cus * (fam > 0 ? esp::stream_workgroups_per_cu(p->head_dim, fam) : esp::tiled_workgroups_per_cu(p->head_dim));
   return ESP_OK;
 }
 

@@ -17,8 +17,9 @@
 //   P^T = exp2(S^T - m) rounded to fp16 / bf16    (D layout of S^T == B layout of P^T: no shuffles)
 //   O^T[HD][cols]      += V^T[HD][32] . P^T        v_mfma_f32_16x16x32 (A = V^T straight from HBM: the pool keeps V transposed)
 // with no LDS on the way. The 4 wavefronts take 32-key units round robin and
-// merge their (m, l, O) through LDS in wave order at the end. Loads for the
-// next unit are issued before the current unit's math (two register sets).
+// merge their (m, l, O) through LDS in wave order at the end. Each wavefront
+// keeps a ring of register sets: the loads of the next units are in flight
+// while the current unit is in the matrix cores.
 #include "common.hpp"
 
 namespace esp {
@@ -30,18 +31,23 @@ struct Unit {  // operands of one unit of SBU 16-key sub-blocks
 };
 
 // SBU: 16-key sub-blocks per unit (2: P.V on 16x16x32 tiles; 1: on 16x16x16 tiles, for
-// head dims whose operands would not fit two register sets otherwise).
-template <int DT, int HD, int NC, int SBU, int OCC>
+// head dims whose operands would not fit the register ring otherwise).
+// BT: tokens per block when known at compile time (0: read from the arguments).
+template <int DT, int HD, int NC, int SBU, int NBUF, int BT, int OCC>
 __global__ __launch_bounds__(256, OCC) void attn_stream_kernel(const KArgs a) {
   constexpr int KK = HD / 32, MT = HD / 16, LDO = HD + 4, UK = 16 * SBU, USH = SBU == 2 ? 5 : 4;
   extern __shared__ float smem[];  // [4 waves][NC * 16 cols][LDO] O, then [4][NC * 16][2] m, l
 
+  const int bt = BT ? BT : a.bt;
   const int kvh = blockIdx.x;
   const int lane = threadIdx.x & 63;
   const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
   const int c16 = lane & 15, q4 = lane >> 4;
   const esp_tile tile = a.tiles[blockIdx.y];
   const esp_tree tree = a.trees[tile.tree];
+  // The planner may carry the tree's block-list offset in the tile (pad = table + 1): one
+  // dependent load less before the first KV page can be requested.
+  const int table = tile.pad > 0 ? tile.pad - 1 : tree.table;
   const int end = tree.base + tree.M;
   const int rows_live = min(a.R, end - tile.r0);
   const int rr0 = tile.r0 - tree.base;
@@ -66,27 +72,29 @@ __global__ __launch_bounds__(256, OCC) void attn_stream_kernel(const KArgs a) {
       qf[c][kk] = ok[c] ? *reinterpret_cast<const u32x4*>(qp + 32 * kk) : u32x4{0, 0, 0, 0};
   }
 
-  // ---- units of UK keys: the cached range, then the tree's batch rows
+  // ---- the cached range in units of UK keys. Interior units lie wholly inside
+  // [k0, k1) on a layer without a window: they need no masks and go through the
+  // pipelined loop. The (at most two) partial units at the ends of the range, every
+  // unit of a windowed layer, and the tree's batch rows take the general path.
   const int cp0 = tile.k0 >> USH;
-  const int n_cached = tile.k1 > tile.k0 ? ((tile.k1 + UK - 1) >> USH) - cp0 : 0;
-  int k_last = -1, bp0 = 0, n_batch = 0;
-  if (tile.last) {
-    // Last batch key any row of the tile sees: its last row, a root it sees whole
-    // (anc_len), the end of its image (bidi).
-    int kl = -1;
-#pragma unroll
-    for (int c = 0; c < NC; ++c)
-      if (ok[c]) kl = max(kl, max(rr[c], max(dsc[c].z - 1, a.bidi ? dsc[c].w - 1 : -1)));
-#pragma unroll
-    for (int o = 32; o >= 1; o >>= 1) kl = max(kl, __shfl_xor(kl, o));
-    k_last = __builtin_amdgcn_readfirstlane(min(kl, tree.M - 1));
-    bp0 = tile.b0 >> USH;
-    n_batch = max(0, ((k_last + UK) >> USH) - bp0);
+  const bool has_cached = tile.k1 > tile.k0;
+  const int ulast = has_cached ? (tile.k1 - 1) >> USH : cp0 - 1;
+  const int n_cached = ulast - cp0 + 1;
+  int ui0, ui1, n_edge;  // interior units [ui0, ui1)
+  bool first_edge = false, last_edge = false;
+  if (a.window > 0 || !has_cached) {
+    ui0 = ui1 = cp0;
+    n_edge = n_cached;
+  } else {
+    first_edge = (tile.k0 & (UK - 1)) != 0 || ((cp0 + 1) << USH) > tile.k1;
+    last_edge = (ulast != cp0 || !first_edge) && ((ulast + 1) << USH) > tile.k1;
+    ui0 = cp0 + (first_edge ? 1 : 0);
+    ui1 = ulast + 1 - (last_edge ? 1 : 0);
+    n_edge = (first_edge ? 1 : 0) + (last_edge ? 1 : 0);
   }
-  const int n_units = n_cached + n_batch;
-
+  int k_last = -1, bp0 = 0, n_batch = 0;  // batch range: set once the cached range has been streamed
   f32x4 acc[NC][MT];
-  float m_run[NC], l_run[NC];
+  float m_run[NC], l_run[NC];  // running max in log2 units of the scaled score; this lane's share of the sum
 #pragma unroll
   for (int c = 0; c < NC; ++c) {
     m_run[c] = -INFINITY;
@@ -95,36 +103,35 @@ __global__ __launch_bounds__(256, OCC) void attn_stream_kernel(const KArgs a) {
     for (int mt = 0; mt < MT; ++mt) acc[c][mt] = f32x4{0, 0, 0, 0};
   }
 
-  // Cached units: K rows and V^T rows straight from the pool.
-  auto load_cached = [&](int u, Unit<HD, SBU>& U) {
-    const int j0 = (cp0 + u) << USH;
+  // K rows and V^T rows of cached unit u (absolute unit index) straight from the pool.
+  // Straight-line code: a unit past the wavefront's last one (valid == false) reads one
+  // 16-byte line of Q with every load instead of being skipped, so the number of loads
+  // in flight is the same on every path and the hardware load counter can be waited
+  // on exactly. A sub-block past the range's last page re-reads that page.
+  const int last_js = (max(tile.k1, tile.k0 + 1) - 1) & ~15;
+  const int lane_k = (c16 * HD + 8 * q4), lane_v = c16 * bt + 4 * q4;
+  auto load_cached = [&](int u, Unit<HD, SBU>& U, const bool valid) {
+    const int j0 = (valid ? u : cp0) << USH;
 #pragma unroll
     for (int sb = 0; sb < SBU; ++sb) {
-      const int js = j0 + 16 * sb;  // first key of the sub-block
-      // A sub-block wholly outside the range is not read (its page may not exist).
-      const bool live = js < tile.k1 && js + 16 > tile.k0;
-      if (live) {
-        const int b = block_of(a, tree.table, js);
-        const uint16_t* hb = a.pool + head_base(a, HD, b, kvh);
-        const int t0 = js % a.bt;
-        const uint16_t* kp = hb + size_t(t0 + c16) * HD + 8 * q4;
-        const uint16_t* vp = hb + size_t(a.bt) * HD + size_t(c16) * a.bt + t0 + 4 * q4;
+      const int js = min(j0 + 16 * sb, last_js);  // first key of the sub-block
+      const int b = block_of(a, table, js);
+      const int t0 = js % bt;
+      const uint16_t* hb = a.pool + head_base(a, HD, b, kvh);
+      const uint16_t* kp = valid ? hb + t0 * HD + lane_k : a.Q;
+      const uint16_t* vp = valid ? hb + bt * HD + t0 + lane_v : a.Q;
+      const int ks = valid ? 32 : 0;
+      const int vs = valid ? 16 * bt : 0;
 #pragma unroll
-        for (int kk = 0; kk < KK; ++kk) U.k[sb][kk] = *reinterpret_cast<const u32x4*>(kp + 32 * kk);
+      for (int kk = 0; kk < KK; ++kk) U.k[sb][kk] = *reinterpret_cast<const u32x4*>(kp + ks * kk);
 #pragma unroll
-        for (int mt = 0; mt < MT; ++mt) U.v[sb][mt] = *reinterpret_cast<const u32x2*>(vp + size_t(16 * mt) * a.bt);
-      } else {
-#pragma unroll
-        for (int kk = 0; kk < KK; ++kk) U.k[sb][kk] = u32x4{0, 0, 0, 0};
-#pragma unroll
-        for (int mt = 0; mt < MT; ++mt) U.v[sb][mt] = u32x2{0, 0};
-      }
+      for (int mt = 0; mt < MT; ++mt) U.v[sb][mt] = *reinterpret_cast<const u32x2*>(vp + vs * mt);
     }
   };
 
   // Batch units: rows of the pass (row major Kb / Vb); V gathered element by element.
   auto load_batch = [&](int u, Unit<HD, SBU>& U) {
-    const int j0 = (bp0 + (u - n_cached)) << USH;
+    const int j0 = u << USH;
 #pragma unroll
     for (int sb = 0; sb < SBU; ++sb) {
       const int js = j0 + 16 * sb;
@@ -151,27 +158,8 @@ __global__ __launch_bounds__(256, OCC) void attn_stream_kernel(const KArgs a) {
     }
   };
 
-  // edge: the unit needs per-key visibility (range ends, window, batch rows).
-  auto compute_unit = [&](int u, Unit<HD, SBU>& U, const bool edge) {
-    const bool cached = u < n_cached;
-    const int j0 = cached ? (cp0 + u) << USH : (bp0 + (u - n_cached)) << USH;
-    if (edge && cached) {
-      // Keys outside [k0, k1) may be memory never written: their V must not reach the products.
-#pragma unroll
-      for (int sb = 0; sb < SBU; ++sb) {
-        const int jv = j0 + 16 * sb + 4 * q4;
-        const uint32_t m0 = (jv >= tile.k0 && jv < tile.k1) ? 0xffffu : 0u;
-        const uint32_t m1 = (jv + 1 >= tile.k0 && jv + 1 < tile.k1) ? 0xffff0000u : 0u;
-        const uint32_t m2 = (jv + 2 >= tile.k0 && jv + 2 < tile.k1) ? 0xffffu : 0u;
-        const uint32_t m3 = (jv + 3 >= tile.k0 && jv + 3 < tile.k1) ? 0xffff0000u : 0u;
-#pragma unroll
-        for (int mt = 0; mt < MT; ++mt) {
-          U.v[sb][mt].x &= (m0 | m1);
-          U.v[sb][mt].y &= (m2 | m3);
-        }
-      }
-    }
-    f32x4 s[NC][SBU];
+  // S^T = K . Q^T of one unit.
+  auto scores = [&](const Unit<HD, SBU>& U, f32x4 (&s)[NC][SBU]) {
 #pragma unroll
     for (int c = 0; c < NC; ++c)
 #pragma unroll
@@ -180,42 +168,15 @@ __global__ __launch_bounds__(256, OCC) void attn_stream_kernel(const KArgs a) {
 #pragma unroll
         for (int kk = 0; kk < KK; ++kk) s[c][sb] = mfma16x32<DT>(U.k[sb][kk], qf[c][kk], s[c][sb]);
       }
-    int kpos[SBU][4];
-    if (edge && !cached && a.window > 0) {
-#pragma unroll
-      for (int sb = 0; sb < SBU; ++sb)
-#pragma unroll
-        for (int e = 0; e < 4; ++e) {
-          const int j = j0 + 16 * sb + 4 * q4 + e;
-          kpos[sb][e] = a.pos[tree.base + min(j, tree.M - 1)].x;
-        }
-    }
+  };
+  // Online softmax over a unit's scores x (log2 units, -inf where masked), then O^T += V^T . P^T.
+  auto softmax_pv = [&](const Unit<HD, SBU>& U, f32x4 (&x)[NC][SBU], const float (&mx_in)[NC]) {
     bool any_change = false;
     u32x2 pb[NC][SBU];
     float corr[NC];
 #pragma unroll
     for (int c = 0; c < NC; ++c) {
-      float mx = -INFINITY;
-#pragma unroll
-      for (int sb = 0; sb < SBU; ++sb)
-#pragma unroll
-        for (int e = 0; e < 4; ++e) {
-          float x = s[c][sb][e] * a.scale_log2;
-          if (edge) {
-            const int j = j0 + 16 * sb + 4 * q4 + e;
-            bool vis;
-            if (cached) {
-              vis = j >= tile.k0 && j < tile.k1;
-              if (a.window > 0) vis = vis && (qpos[c] - j < a.window);
-            } else {
-              vis = j <= k_last && ((j < dsc[c].z) || (j >= dsc[c].x && (j <= rr[c] || (a.bidi && j < dsc[c].w))));
-              if (a.window > 0) vis = vis && (qpos[c] - kpos[sb][e] < a.window);
-            }
-            x = vis ? x : -INFINITY;
-          }
-          s[c][sb][e] = x;
-          mx = fmaxf(mx, x);
-        }
+      float mx = mx_in[c];
       mx = fmaxf(mx, __shfl_xor(mx, 16));
       mx = fmaxf(mx, __shfl_xor(mx, 32));
       const float m_new = fmaxf(m_run[c], mx);
@@ -229,7 +190,7 @@ __global__ __launch_bounds__(256, OCC) void attn_stream_kernel(const KArgs a) {
         float p[4];
 #pragma unroll
         for (int e = 0; e < 4; ++e) {
-          p[e] = fast_exp2(s[c][sb][e] - m_safe);
+          p[e] = fast_exp2(x[c][sb][e] - m_safe);
           ps += p[e];
         }
         pb[c][sb] = u32x2{pack2<DT>(p[0], p[1]), pack2<DT>(p[2], p[3])};
@@ -255,32 +216,127 @@ __global__ __launch_bounds__(256, OCC) void attn_stream_kernel(const KArgs a) {
       }
     }
   };
-  // Interior cached units of an unwindowed layer see every key.
-  auto is_edge = [&](int u) {
-    const int j0 = (cp0 + u) << USH;
-    return a.window > 0 || j0 < tile.k0 || j0 + UK > tile.k1;
+
+  // Interior unit: every key visible to every row.
+  auto compute_interior = [&](const Unit<HD, SBU>& U) {
+    f32x4 s[NC][SBU];
+    scores(U, s);
+    float mx[NC];
+#pragma unroll
+    for (int c = 0; c < NC; ++c) {
+      mx[c] = -INFINITY;
+#pragma unroll
+      for (int sb = 0; sb < SBU; ++sb)
+#pragma unroll
+        for (int e = 0; e < 4; ++e) {
+          s[c][sb][e] *= a.scale_log2;
+          mx[c] = fmaxf(mx[c], s[c][sb][e]);
+        }
+    }
+    softmax_pv(U, s, mx);
   };
 
-  // ---- stream the cached range: two register sets, the next unit's loads in
-  // flight during the math. Wavefront w takes units w, w + 4, ...
-  {
-    Unit<HD, SBU> A, B;
-    int u = wave;
-    if (u < n_cached) load_cached(u, A);
-    for (; u < n_cached; u += 8) {
-      if (u + 4 < n_cached) load_cached(u + 4, B);
-      if (is_edge(u)) compute_unit(u, A, true);
-      else compute_unit(u, A, false);
-      if (u + 4 < n_cached) {
-        if (u + 8 < n_cached) load_cached(u + 8, A);
-        if (is_edge(u + 4)) compute_unit(u + 4, B, true);
-        else compute_unit(u + 4, B, false);
+  // General unit: per-key visibility. BATCH: the keys are the tree's batch rows j0 .. (tree
+  // mask and window), else cached keys j0 .. (range ends and window).
+  auto compute_general = [&]<bool BATCH>(int j0, Unit<HD, SBU>& U) {
+    if constexpr (!BATCH) {
+      // Cached keys outside [k0, k1) may be memory never written: their V must not reach the products.
+#pragma unroll
+      for (int sb = 0; sb < SBU; ++sb) {
+        const int jv = j0 + 16 * sb + 4 * q4;
+        const uint32_t m0 = (jv >= tile.k0 && jv < tile.k1) ? 0xffffu : 0u;
+        const uint32_t m1 = (jv + 1 >= tile.k0 && jv + 1 < tile.k1) ? 0xffff0000u : 0u;
+        const uint32_t m2 = (jv + 2 >= tile.k0 && jv + 2 < tile.k1) ? 0xffffu : 0u;
+        const uint32_t m3 = (jv + 3 >= tile.k0 && jv + 3 < tile.k1) ? 0xffff0000u : 0u;
+#pragma unroll
+        for (int mt = 0; mt < MT; ++mt) {
+          U.v[sb][mt].x &= (m0 | m1);
+          U.v[sb][mt].y &= (m2 | m3);
+        }
       }
     }
-    // ---- then the batch rows (few: this kernel serves short trees)
-    for (u = n_cached + ((wave + 4 - (n_cached & 3)) & 3); u < n_units; u += 4) {
-      load_batch(u, A);
-      compute_unit(u, A, true);
+    f32x4 s[NC][SBU];
+    scores(U, s);
+    int kpos[SBU][4];
+    if (BATCH && a.window > 0) {
+#pragma unroll
+      for (int sb = 0; sb < SBU; ++sb)
+#pragma unroll
+        for (int e = 0; e < 4; ++e) {
+          const int j = j0 + 16 * sb + 4 * q4 + e;
+          kpos[sb][e] = a.pos[tree.base + min(j, tree.M - 1)].x;
+        }
+    }
+    float mx[NC];
+#pragma unroll
+    for (int c = 0; c < NC; ++c) {
+      mx[c] = -INFINITY;
+#pragma unroll
+      for (int sb = 0; sb < SBU; ++sb)
+#pragma unroll
+        for (int e = 0; e < 4; ++e) {
+          const int j = j0 + 16 * sb + 4 * q4 + e;
+          bool vis;
+          if constexpr (!BATCH) {
+            vis = j >= tile.k0 && j < tile.k1;
+            if (a.window > 0) vis = vis && (qpos[c] - j < a.window);
+          } else {
+            vis = j <= k_last && ((j < dsc[c].z) || (j >= dsc[c].x && (j <= rr[c] || (a.bidi && j < dsc[c].w))));
+            if (a.window > 0) vis = vis && (qpos[c] - kpos[sb][e] < a.window);
+          }
+          const float x = vis ? s[c][sb][e] * a.scale_log2 : -INFINITY;
+          s[c][sb][e] = x;
+          mx[c] = fmaxf(mx[c], x);
+        }
+    }
+    softmax_pv(U, s, mx);
+  };
+
+  {
+    Unit<HD, SBU> U[NBUF];
+    // ---- interior units through a ring of NBUF register sets: while one unit is in the
+    // matrix cores, the loads of the next NBUF - 1 are in flight. Wavefront w takes
+    // interior units w, w + 4, ...: n_mine of them.
+    const int n_int = ui1 - ui0;
+    const int n_mine = n_int > wave ? (n_int - wave + 3) >> 2 : 0;
+    if (n_mine > 0) {
+      const int u0 = ui0 + wave;
+#pragma unroll
+      for (int s = 0; s < NBUF; ++s) load_cached(u0 + 4 * s, U[s], s < n_mine);
+      for (int i = 0; i < n_mine; i += NBUF) {
+#pragma unroll
+        for (int s = 0; s < NBUF; ++s) {
+          if (i + s < n_mine) compute_interior(U[s]);
+          load_cached(u0 + 4 * (i + s + NBUF), U[s], i + s + NBUF < n_mine);
+        }
+      }
+    }
+    // ---- then the units that need masks: partial or windowed cached units, batch rows.
+    // They continue the round robin after the interior units.
+    if (tile.last) {
+      // Last batch key any row of the tile sees: its last row, a root it sees whole
+      // (anc_len), the end of its image (bidi).
+      int kl = -1;
+#pragma unroll
+      for (int c = 0; c < NC; ++c)
+        if (ok[c]) kl = max(kl, max(rr[c], max(dsc[c].z - 1, a.bidi ? dsc[c].w - 1 : -1)));
+#pragma unroll
+      for (int o = 32; o >= 1; o >>= 1) kl = max(kl, __shfl_xor(kl, o));
+      k_last = __builtin_amdgcn_readfirstlane(min(kl, tree.M - 1));
+      bp0 = tile.b0 >> USH;
+      n_batch = max(0, ((k_last + UK) >> USH) - bp0);
+    }
+    const int n_slow = n_edge + n_batch;
+    for (int i = (wave + 4 - (n_int & 3)) & 3; i < n_slow; i += 4) {
+      if (i < n_edge) {
+        const int u = (a.window > 0 || !has_cached) ? cp0 + i : ((i == 0 && first_edge) ? cp0 : ulast);
+        load_cached(u, U[0], true);
+        compute_general.template operator()<false>(u << USH, U[0]);
+      } else {
+        const int u = bp0 + (i - n_edge);
+        load_batch(u, U[0]);
+        compute_general.template operator()<true>(u << USH, U[0]);
+      }
     }
   }
 
@@ -412,12 +468,19 @@ __global__ __launch_bounds__(256) void attn_combine_kernel(const KArgs a, const 
 
 size_t stream_smem_bytes(int HD, int NC) { return size_t(4 * NC * 16) * (HD + 4 + 2) * sizeof(float); }
 
+// Resident workgroups per CU and ring depth of each variant: the single-column-tile
+// head_dim-128 kernel fits two workgroups per CU with a two-deep ring; the wider ones
+// run one workgroup per CU with a deeper ring.
+constexpr int stream_occ(int HD, int NC) { return (HD == 128 && NC == 1) ? 2 : 1; }
+constexpr int stream_nbuf(int HD, int NC) { return (HD == 128 && NC == 1) ? 2 : 3; }
+int stream_workgroups_per_cu(int HD, int NC) { return stream_occ(HD, NC); }
+
 template <int DT, int HD, int NC>
 static hipError_t launch_stream_t(const KArgs& a, int n_tiles, hipStream_t st) {
   constexpr int SBU = HD == 128 ? 2 : 1;
-  constexpr int OCC = (HD == 128 && NC == 1) ? 2 : 1;
+  constexpr int NBUF = stream_nbuf(HD, NC), OCC = stream_occ(HD, NC);
   const size_t smem = stream_smem_bytes(HD, NC);
-  auto k = attn_stream_kernel<DT, HD, NC, SBU, OCC>;
+  auto k = a.bt == 16 ? attn_stream_kernel<DT, HD, NC, SBU, NBUF, 16, OCC> : attn_stream_kernel<DT, HD, NC, SBU, NBUF, 0, OCC>;
   if (smem > 48 * 1024) {
     hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(k), hipFuncAttributeMaxDynamicSharedMemorySize, int(smem));
     if (e != hipSuccess) return e;

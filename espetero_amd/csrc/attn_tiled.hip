@@ -346,6 +346,8 @@ __global__ __launch_bounds__(256, (HD == 128 ? 2 : 1)) void attn_tiled_kernel(co
     }
 }
 
+int tiled_workgroups_per_cu(int HD) { return HD == 128 ? 2 : 1; }
+
 size_t tiled_smem_bytes(int HD) { return size_t(64 * (HD + 8) + HD * (64 + 8)) * sizeof(uint16_t); }
 
 template <int DT, int HD>

@@ -38,6 +38,14 @@ def to_dev(a, device="cuda"):
     return torch.from_numpy(a.copy()).to(device)
 
 
+def plan_hint(params, device=0):
+    """Workgroups of the kernel serving `params` that are resident at once: the planner's split target."""
+    err = C.create_string_buffer(_ERRLEN)
+    n = C.c_int32(0)
+    abi.check(abi.attn_lib().esp_attn_plan_hint(C.byref(params), device, C.byref(n), err, _ERRLEN), err)
+    return n.value
+
+
 def workspace_bytes(params, n_rows, n_parts):
     return abi.attn_lib().esp_attn_workspace_bytes(C.byref(params), n_rows, n_parts)
 

@@ -93,8 +93,22 @@ inline void plan_tiles(AttnPlan& A, int groups, int window, const int32_t* pos, 
   const int budget = std::max(1, o.groups_target / std::max(1, groups * n_tiles));
   int chunk_all = 0;  // balanced rule: keys per workgroup
   if (o.balanced && budget > 1) {
-    const long long want = (total_span * groups + o.groups_target - 1) / o.groups_target;
-    chunk_all = int(std::max<long long>(o.min_chunk, (want + o.granule - 1) / o.granule * o.granule));
+    // The smallest chunk (a granule multiple) whose tile count fits the target: a pass
+    // that overshoots the resident workgroup count by a few tiles pays a whole extra round.
+    const long long cap = std::max(1, o.groups_target / std::max(1, groups));
+    auto tiles_at = [&](long long chunk) {
+      long long n = 0;
+      for (const RowTile& rt : rts)
+        n += rt.span >= o.min_span ? std::min<long long>((rt.span + chunk - 1) / chunk, o.max_splits) : 1;
+      return n;
+    };
+    long long lo = std::max(1, o.min_chunk / o.granule), hi = std::max<long long>(lo, (total_span + o.granule - 1) / o.granule + 1);
+    while (lo < hi) {
+      const long long mid = (lo + hi) / 2;
+      if (tiles_at(mid * o.granule) <= cap) hi = mid;
+      else lo = mid + 1;
+    }
+    chunk_all = int(lo * o.granule);
   }
   for (const RowTile& rt : rts) {
     const esp_tree& t = A.trees[size_t(rt.tree)];
@@ -110,8 +124,11 @@ inline void plan_tiles(AttnPlan& A, int groups, int window, const int32_t* pos, 
         ns = std::min({(span + chunk - 1) / chunk, budget, o.max_splits});
       }
     }
+    // Balanced rule: the tile carries its tree's block-list offset (pad = table + 1), which
+    // saves the kernels a dependent load; the reference rule leaves pad 0 as the reference does.
+    const int pad = o.balanced ? t.table + 1 : 0;
     if (ns <= 1) {
-      A.tiles.push_back({rt.tree, t.base + rt.r, rt.k0, t.P, -1, 1, rt.b0, 0});
+      A.tiles.push_back({rt.tree, t.base + rt.r, rt.k0, t.P, -1, 1, rt.b0, pad});
       continue;
     }
     const int per = (span + ns - 1) / ns;
@@ -123,7 +140,7 @@ inline void plan_tiles(AttnPlan& A, int groups, int window, const int32_t* pos, 
       // Balanced rule: a windowed range starts anywhere, its inner boundaries still fall on page multiples.
       if (o.balanced && k1 < t.P) k1 = std::max(k + o.granule, k1 / o.granule * o.granule);
       k1 = std::min(t.P, k1);
-      A.tiles.push_back({rt.tree, t.base + rt.r, k, k1, A.parts++, k1 >= t.P ? 1 : 0, rt.b0, 0});
+      A.tiles.push_back({rt.tree, t.base + rt.r, k, k1, A.parts++, k1 >= t.P ? 1 : 0, rt.b0, pad});
       k = k1;
     }
     A.combine.push_back({t.base + rt.r, std::min(R, t.M - rt.r), part0, used});

@@ -69,7 +69,7 @@ typedef struct esp_tile {
   int32_t part; /* -1: write O; else index of the partial record this tile writes */
   int32_t last; /* also scan the tree's batch keys (this pass's own rows) */
   int32_t b0;   /* first batch key (relative row) any row of the tile may see */
-  int32_t pad;
+  int32_t pad;  /* 0 (the reference's value), or 1 + the tree's `table`: lets a kernel skip the tree lookup */
 } esp_tile;
 
 /* Merge job of one split tile group. Field for field AttnCombine (40_:804-809). */
@@ -115,6 +115,13 @@ typedef struct esp_attn_params {
 /* Library / device check. Safe to call more than once. */
 int esp_attn_init(int device, char* err, size_t errlen);
 int esp_attn_abi_version(void);
+
+/* Split target for the planner: how many workgroups of the kernel that serves
+ * these params (rows_per_tile x G packed rows, head_dim, dtype) are resident on
+ * the device at once. A pass split into more workgroups than this runs in
+ * rounds and pays the per-workgroup set-up again (the reference aims at a
+ * fixed 256 threadgroups, forest.h:1385). */
+int esp_attn_plan_hint(const esp_attn_params* p, int device, int32_t* workgroups, char* err, size_t errlen);
 
 /* Bytes of `workspace` esp_attn_forward needs for a pass of n_rows batch rows
  * whose plan holds n_parts partial records (replaces the reference's `parts`

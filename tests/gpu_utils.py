@@ -22,8 +22,8 @@ def native_pool(case, nan_fill=False):
     return nat
 
 
-def default_options(case, workgroups=1024):
-    return host.options_mi355x(case.params.rows_per_tile, workgroups)
+def default_options(case, workgroups=None):
+    return host.options_mi355x(case.params.rows_per_tile, workgroups or device.plan_hint(case.params))
 
 
 def plan(case, options):
