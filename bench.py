@@ -73,9 +73,9 @@ class Workload:
             base += M
             tab += (P + M + bt - 1) // bt
         self.trees, self.desc, self.pos = trees, desc, pos
-        wg = workgroups or device.plan_hint(p)
-        opts = host.options_mi355x(rows_per_tile, wg)
-        self.tiles, self.jobs, self.n_parts = host.plan_tiles(trees, Hkv, window, pos if window > 0 else None, opts)
+        resident, groups = device.plan_hint(p)
+        opts = host.options_mi355x(rows_per_tile, workgroups or resident)
+        self.tiles, self.jobs, self.n_parts = host.plan_tiles(trees, groups, window, pos if window > 0 else None, opts)
         # Block tables: disjoint slices of one seeded permutation of the pool, one slice per
         # rotation set, so a step never finds the previous step's pages in a cache.
         perm = np.random.default_rng(seed + 1).permutation(self.pool_pages).astype(np.int32)

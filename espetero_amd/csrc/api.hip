@@ -121,14 +121,17 @@ int esp_attn_init(int device, char* err, size_t errlen) {
   return ESP_OK;
 }
 
-int esp_attn_plan_hint(const esp_attn_params* p, int device, int32_t* workgroups, char* err, size_t errlen) {
+int esp_attn_plan_hint(const esp_attn_params* p, int device, int32_t* workgroups, int32_t* groups_per_tile, char* err,
+                       size_t errlen) {
   if (int rc = check_params(p, err, errlen)) return rc;
-  if (!workgroups || p->rows_per_tile <= 0) return fail(err, errlen, ESP_EINVAL, "workgroups is NULL or rows_per_tile <= 0");
+  if (!workgroups || !groups_per_tile || p->rows_per_tile <= 0)
+    return fail(err, errlen, ESP_EINVAL, "NULL output or rows_per_tile <= 0");
   int cus = 0;
   hipError_t e = hipDeviceGetAttribute(&cus, hipDeviceAttributeMultiprocessorCount, device);
   if (e != hipSuccess) return hip_fail(err, errlen, "hipDeviceGetAttribute", e);
   const int fam = family(p);
   *workgroups = cus * (fam > 0 ? esp::stream_workgroups_per_cu(p->head_dim, fam) : esp::tiled_workgroups_per_cu(p->head_dim));
+  *groups_per_tile = fam > 0 ? p->Hkv : p->H;
   return ESP_OK;
 }
 

@@ -20,16 +20,17 @@
 //   P^T = exp2(S^T - m)                 registers; the D layout of S^T is the B layout of P^T
 //   O^T[HD][32 rows]     += V^T . P^T   A = V^T from LDS
 // so the softmax runs along registers of one lane plus one cross-lane step, and
-// nothing is transposed on the way. MFMA row r of a 32-key group reads key
-// kappa(r) so that the 8 P values a lane packs for one P.V step are 8
-// consecutive keys, i.e. one 16-byte LDS read of V^T.
-// The next step's global loads are issued before the current step's math.
+// nothing is transposed on the way. The 8 P values a lane packs for one P.V
+// step are keys {8 a + 4 hb + j}: the staging writes V^T with key bits 2 and 3
+// swapped (kappa), which makes them one 16-byte LDS read.
+// Two LDS stages: while a step is in the matrix cores the next step's tile is
+// written to the other stage and the loads of the step after are in flight.
 #include "common.hpp"
 
 namespace esp {
 
-__device__ __forceinline__ int kappa(int r) {  // MFMA row -> key within a 32-key group
-  return (r & 16) | ((r & 4) << 1) | ((r & 8) >> 1) | (r & 3);
+__device__ __forceinline__ int kappa(int r) {  // swap bits 2 and 3: key <-> LDS column within a 16-key group
+  return (r & ~12) | ((r & 4) << 1) | ((r & 8) >> 1);
 }
 
 struct SubBlock {  // one 16-key sub-block of a step: where its K rows and V^T rows lie
@@ -46,9 +47,8 @@ __global__ __launch_bounds__(256, (HD == 128 ? 2 : 1)) void attn_tiled_kernel(co
   constexpr int CH = HD / 8;      // 16-byte chunks per K row
   constexpr int KP = CH / 4;      // K fill passes of a wavefront (64 / CH keys each)
   constexpr int VP = HD / 32;     // V^T fill passes (32 dims each)
+  constexpr int STAGE = 64 * LDK + HD * LDV;  // elements of one LDS stage: K [64 keys][LDK], V^T [HD dims][LDV]
   extern __shared__ uint16_t lds[];
-  uint16_t* Ks = lds;              // [64 keys][LDK]
-  uint16_t* Vs = lds + 64 * LDK;   // [HD dims][LDV]
   __shared__ int red[4][6];
 
   // Workgroup -> (KV head, head in group, tile): consecutive ids differ in KV
@@ -193,14 +193,20 @@ __global__ __launch_bounds__(256, (HD == 128 ? 2 : 1)) void attn_tiled_kernel(co
       }
     }
   };
-  auto fill_store = [&]() {
+  auto fill_store = [&](int stage) {
+    uint16_t* Ks = lds + stage * STAGE;
+    uint16_t* Vs = Ks + 64 * LDK;
     const int kpp = 64 / CH;
 #pragma unroll
     for (int p = 0; p < KP; ++p)
       *reinterpret_cast<u32x4*>(Ks + (16 * wave + kpp * p + lane / CH) * LDK + 8 * (lane % CH)) = fk[p];
+    // This lane holds keys 8 a .. 8 a + 7 of one dim (a = lane & 1): keys 8 a + 4 b + j go to column 8 b + 4 a + j.
 #pragma unroll
-    for (int p = 0; p < VP; ++p)
-      *reinterpret_cast<u32x4*>(Vs + (32 * p + (lane >> 1)) * LDV + 16 * wave + 8 * (lane & 1)) = fv[p];
+    for (int p = 0; p < VP; ++p) {
+      uint16_t* vrow = Vs + (32 * p + (lane >> 1)) * LDV + 16 * wave + 4 * (lane & 1);
+      *reinterpret_cast<u32x2*>(vrow) = u32x2{fv[p].x, fv[p].y};
+      *reinterpret_cast<u32x2*>(vrow + 8) = u32x2{fv[p].z, fv[p].w};
+    }
   };
 
   f32x16 acc[NT];
@@ -209,105 +215,138 @@ __global__ __launch_bounds__(256, (HD == 128 ? 2 : 1)) void attn_tiled_kernel(co
 #pragma unroll
     for (int i = 0; i < 16; ++i) acc[nt][i] = 0.0f;
   float m_run = -INFINITY, l_run = 0.0f;
-  const int krow = kappa(l32);
+  // Batch steps past this wavefront's last row hold nothing it can see (plain causal rows).
+  const int wave_last = rr0 + min(32 * wave + 31, rows_live - 1);
 
-  if (n_steps > 0) fill_load(0);
+  if (n_steps > 0) {
+    fill_load(0);
+    fill_store(0);
+    if (n_steps > 1) fill_load(1);
+  }
+  __syncthreads();
   for (int step = 0; step < n_steps; ++step) {
-    __syncthreads();  // the previous step's LDS reads are done
-    fill_store();
-    __syncthreads();
-    if (step + 1 < n_steps) fill_load(step + 1);
+    const int cur = step & 1;
+    if (step + 1 < n_steps) fill_store(cur ^ 1);   // the tile loaded during the previous step
+    if (step + 2 < n_steps) fill_load(step + 2);
+    const uint16_t* Ks = lds + cur * STAGE;
+    const uint16_t* Vs = Ks + 64 * LDK;
 
-    // ---- S^T = K . Q^T
-    f32x16 s[2];
-#pragma unroll
-    for (int kt = 0; kt < 2; ++kt) {
-#pragma unroll
-      for (int i = 0; i < 16; ++i) s[kt][i] = 0.0f;
-      const uint16_t* kp = Ks + (32 * kt + krow) * LDK + 8 * hb;
-#pragma unroll
-      for (int ks = 0; ks < KS; ++ks)
-        s[kt] = mfma32x16<DT>(*reinterpret_cast<const u32x4*>(kp + 16 * ks), qf[ks], s[kt]);
+    // Sub-block kinds of this step; a step whose keys are all batch rows after this
+    // wavefront's rows is skipped (its rows see none of them).
+    bool skip = false;
+    {
+      const int s0 = 4 * step;
+      if (s0 >= n_c && seg_max != INT32_MAX) {
+        const int jfirst = ((a0 + s0 - n_c) << 4) - tree.base;
+        skip = jfirst > wave_last;
+      }
     }
+    if (!skip) {
+      // ---- S^T = K . Q^T
+      f32x16 s[2];
+#pragma unroll
+      for (int kt = 0; kt < 2; ++kt) {
+#pragma unroll
+        for (int i = 0; i < 16; ++i) s[kt][i] = 0.0f;
+        const uint16_t* kp = Ks + (32 * kt + l32) * LDK + 8 * hb;
+#pragma unroll
+        for (int ks = 0; ks < KS; ++ks)
+          s[kt] = mfma32x16<DT>(*reinterpret_cast<const u32x4*>(kp + 16 * ks), qf[ks], s[kt]);
+      }
 
-    // ---- mask, online softmax. s[kt][8 t + e] is key 32 kt + 16 t + 8 hb + e of the step.
-    float mx = -INFINITY;
-#pragma unroll
-    for (int kt = 0; kt < 2; ++kt)
-#pragma unroll
-      for (int t = 0; t < 2; ++t) {
-        const int sidx = 4 * step + 2 * kt + t;  // sub-block of the range
-        int kind, j0;
-        if (sidx < n_c) {
-          kind = 0;
-          j0 = (c0 + sidx) << 4;
-        } else if (sidx < n_sb) {
-          kind = 1;
-          j0 = ((a0 + sidx - n_c) << 4) - tree.base;
+      // ---- mask, online softmax. s[kt][4 i + j] is key 32 kt + 8 i + 4 hb + j of the step.
+      // One uniform test per step: are all 64 keys visible to every row of this wavefront?
+      bool step_full;
+      {
+        const int s0 = 4 * step;
+        if (s0 + 4 <= n_c) {
+          const int j0 = (c0 + s0) << 4;
+          step_full = j0 >= tile.k0 && j0 + 64 <= tile.k1 && (a.window == 0 || qpos_max - j0 < a.window);
+        } else if (s0 >= n_c && s0 + 4 <= n_sb) {
+          const int j0 = ((a0 + s0 - n_c) << 4) - tree.base;
+          step_full = a.window == 0 && j0 >= seg_max && j0 + 63 <= rr0 + 32 * wave && j0 >= 0;
         } else {
-          kind = 2;
-          j0 = 0;
+          step_full = false;
         }
-        bool full;  // every row of this wavefront sees every key of the sub-block
-        if (kind == 0) full = j0 >= tile.k0 && j0 + 16 <= tile.k1 && (a.window == 0 || qpos_max - j0 < a.window);
-        else if (kind == 1) full = a.window == 0 && j0 >= seg_max && j0 + 15 <= rr0 + 32 * wave && j0 >= 0;
-        else full = false;
+      }
+      if (!step_full) {
 #pragma unroll
-        for (int e = 0; e < 8; ++e) {
-          float x = s[kt][8 * t + e] * a.scale_log2;
-          if (!full) {
-            const int j = j0 + 8 * hb + e;
-            bool vis;
-            if (kind == 0) {
-              vis = j >= tile.k0 && j < tile.k1 && (a.window == 0 || qpos - j < a.window);
-            } else if (kind == 1) {
-              vis = j >= 0 && j <= k_last && ((j < d.z) || (j >= d.x && (j <= rr || (a.bidi && j < d.w))));
-              if (a.window > 0 && vis) vis = qpos - a.pos[tree.base + j].x < a.window;
+        for (int kt = 0; kt < 2; ++kt)
+#pragma unroll
+          for (int t = 0; t < 2; ++t) {
+            const int sidx = 4 * step + 2 * kt + t;  // sub-block of the range
+            // Visible keys of the sub-block for this lane's row: j in [lo, hi], plus j < anc.
+            int j0, lo, hi, anc = 0;
+            if (sidx < n_c) {
+              j0 = (c0 + sidx) << 4;
+              lo = tile.k0;
+              hi = tile.k1 - 1;
+              if (a.window > 0) lo = max(lo, qpos - a.window + 1);
+            } else if (sidx < n_sb) {
+              j0 = ((a0 + sidx - n_c) << 4) - tree.base;
+              lo = max(d.x, 0);
+              hi = min(k_last, (a.bidi && d.w > 0) ? max(rr, d.w - 1) : rr);
+              anc = min(d.z, k_last + 1);
             } else {
-              vis = false;
+              j0 = 0;
+              lo = 1;
+              hi = 0;
             }
-            x = vis ? x : -INFINITY;
+            const bool batch_window = sidx >= n_c && sidx < n_sb && a.window > 0;
+#pragma unroll
+            for (int e = 0; e < 8; ++e) {
+              const int idx = 8 * t + e;  // = 4 i + j with i = 2 t + e / 4, j = e % 4
+              const int j = j0 + 8 * (e >> 2) + 4 * hb + (e & 3);
+              bool vis = (j >= lo && j <= hi) || (j >= 0 && j < anc);
+              if (batch_window && vis) vis = qpos - a.pos[tree.base + j].x < a.window;
+              s[kt][idx] = vis ? s[kt][idx] : -INFINITY;
+            }
           }
-          s[kt][8 * t + e] = x;
-          mx = fmaxf(mx, x);
-        }
       }
-    mx = fmaxf(mx, __shfl_xor(mx, 32));
-    const float m_new = fmaxf(m_run, mx);
-    const float m_safe = (m_new == -INFINITY) ? 0.0f : m_new;
-    const float corr = fast_exp2(m_run - m_safe);
-    const bool changed = m_new > m_run;
-    m_run = m_new;
-    float ps = 0.0f;
-    u32x4 pb[2][2];
-#pragma unroll
-    for (int kt = 0; kt < 2; ++kt)
-#pragma unroll
-      for (int t = 0; t < 2; ++t) {
-        float p[8];
-#pragma unroll
-        for (int e = 0; e < 8; ++e) {
-          p[e] = fast_exp2(s[kt][8 * t + e] - m_safe);
-          ps += p[e];
-        }
-        pb[kt][t] = u32x4{pack2<DT>(p[0], p[1]), pack2<DT>(p[2], p[3]), pack2<DT>(p[4], p[5]), pack2<DT>(p[6], p[7])};
-      }
-    l_run = l_run * corr + ps;
-    if (__any(changed)) {
-#pragma unroll
-      for (int nt = 0; nt < NT; ++nt) acc[nt] *= corr;
-    }
-
-    // ---- O^T += V^T . P^T
-#pragma unroll
-    for (int nt = 0; nt < NT; ++nt) {
-      const uint16_t* vp = Vs + (32 * nt + l32) * LDV + 8 * hb;
+      float mx = -INFINITY;
 #pragma unroll
       for (int kt = 0; kt < 2; ++kt)
 #pragma unroll
-        for (int t = 0; t < 2; ++t)
-          acc[nt] = mfma32x16<DT>(*reinterpret_cast<const u32x4*>(vp + 32 * kt + 16 * t), pb[kt][t], acc[nt]);
+        for (int i = 0; i < 16; ++i) mx = fmaxf(mx, s[kt][i]);
+      mx *= a.scale_log2;  // scale > 0: the max commutes with it
+      mx = fmaxf(mx, __shfl_xor(mx, 32));
+      const float m_new = fmaxf(m_run, mx);
+      const float m_safe = (m_new == -INFINITY) ? 0.0f : m_new;
+      const float corr = fast_exp2(m_run - m_safe);
+      const bool changed = m_new > m_run;
+      m_run = m_new;
+      float ps = 0.0f;
+      u32x4 pb[2][2];
+#pragma unroll
+      for (int kt = 0; kt < 2; ++kt)
+#pragma unroll
+        for (int t = 0; t < 2; ++t) {
+          float p[8];
+#pragma unroll
+          for (int e = 0; e < 8; ++e) {
+            p[e] = fast_exp2(__builtin_fmaf(s[kt][8 * t + e], a.scale_log2, -m_safe));
+            ps += p[e];
+          }
+          pb[kt][t] = u32x4{pack2<DT>(p[0], p[1]), pack2<DT>(p[2], p[3]), pack2<DT>(p[4], p[5]), pack2<DT>(p[6], p[7])};
+        }
+      l_run = l_run * corr + ps;
+      if (__any(changed)) {
+#pragma unroll
+        for (int nt = 0; nt < NT; ++nt) acc[nt] *= corr;
+      }
+
+      // ---- O^T += V^T . P^T. pb[kt][t] holds keys 32 kt + 16 t + {8 a + 4 hb + j}: LDS columns 32 kt + 16 t + 8 hb ..
+#pragma unroll
+      for (int nt = 0; nt < NT; ++nt) {
+        const uint16_t* vp = Vs + (32 * nt + l32) * LDV + 8 * hb;
+#pragma unroll
+        for (int kt = 0; kt < 2; ++kt)
+#pragma unroll
+          for (int t = 0; t < 2; ++t)
+            acc[nt] = mfma32x16<DT>(*reinterpret_cast<const u32x4*>(vp + 32 * kt + 16 * t), pb[kt][t], acc[nt]);
+      }
     }
+    __syncthreads();
   }
 
   // ---- output: lane (row l32, half hb) holds dims 32 nt + 8 i + 4 hb + j at acc[nt][4 i + j]
@@ -348,7 +387,7 @@ __global__ __launch_bounds__(256, (HD == 128 ? 2 : 1)) void attn_tiled_kernel(co
 
 int tiled_workgroups_per_cu(int HD) { return HD == 128 ? 2 : 1; }
 
-size_t tiled_smem_bytes(int HD) { return size_t(64 * (HD + 8) + HD * (64 + 8)) * sizeof(uint16_t); }
+size_t tiled_smem_bytes(int HD) { return size_t(2) * size_t(64 * (HD + 8) + HD * (64 + 8)) * sizeof(uint16_t); }
 
 template <int DT, int HD>
 static hipError_t launch_tiled_t(const KArgs& a, int n_tiles, hipStream_t st) {

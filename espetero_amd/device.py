@@ -39,11 +39,12 @@ def to_dev(a, device="cuda"):
 
 
 def plan_hint(params, device=0):
-    """Workgroups of the kernel serving `params` that are resident at once: the planner's split target."""
+    """(workgroups resident at once, workgroups per tile) of the kernel serving `params`:
+    the planner's split target and its `groups` argument."""
     err = C.create_string_buffer(_ERRLEN)
-    n = C.c_int32(0)
-    abi.check(abi.attn_lib().esp_attn_plan_hint(C.byref(params), device, C.byref(n), err, _ERRLEN), err)
-    return n.value
+    n, g = C.c_int32(0), C.c_int32(0)
+    abi.check(abi.attn_lib().esp_attn_plan_hint(C.byref(params), device, C.byref(n), C.byref(g), err, _ERRLEN), err)
+    return n.value, g.value
 
 
 def workspace_bytes(params, n_rows, n_parts):

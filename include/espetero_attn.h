@@ -116,12 +116,18 @@ typedef struct esp_attn_params {
 int esp_attn_init(int device, char* err, size_t errlen);
 int esp_attn_abi_version(void);
 
-/* Split target for the planner: how many workgroups of the kernel that serves
- * these params (rows_per_tile x G packed rows, head_dim, dtype) are resident on
- * the device at once. A pass split into more workgroups than this runs in
- * rounds and pays the per-workgroup set-up again (the reference aims at a
- * fixed 256 threadgroups, forest.h:1385). */
-int esp_attn_plan_hint(const esp_attn_params* p, int device, int32_t* workgroups, char* err, size_t errlen);
+/* What the planner needs to know about the kernel that serves these params
+ * (rows_per_tile x G packed rows, head_dim, dtype):
+ *   workgroups      how many of its workgroups are resident on the device at
+ *                   once. A pass split into more runs in rounds and pays the
+ *                   per-workgroup set-up again (the reference aims at a fixed
+ *                   256 threadgroups, forest.h:1385);
+ *   groups_per_tile workgroups one tile becomes: KV heads for the streaming
+ *                   kernel (the G heads of a KV head share a workgroup), query
+ *                   heads for the tiled kernel (the reference: KV heads x SPLIT,
+ *                   forest.h:2920, gemma.h:231). */
+int esp_attn_plan_hint(const esp_attn_params* p, int device, int32_t* workgroups, int32_t* groups_per_tile, char* err,
+                       size_t errlen);
 
 /* Bytes of `workspace` esp_attn_forward needs for a pass of n_rows batch rows
  * whose plan holds n_parts partial records (replaces the reference's `parts`

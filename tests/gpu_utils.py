@@ -23,13 +23,13 @@ def native_pool(case, nan_fill=False):
 
 
 def default_options(case, workgroups=None):
-    return host.options_mi355x(case.params.rows_per_tile, workgroups or device.plan_hint(case.params))
+    return host.options_mi355x(case.params.rows_per_tile, workgroups or device.plan_hint(case.params)[0])
 
 
 def plan(case, options):
     p = case.params
     p.rows_per_tile = options.rows_per_tile
-    return host.plan_tiles(case.trees, p.Hkv, p.window, case.pos if p.window > 0 else None, options)
+    return host.plan_tiles(case.trees, device.plan_hint(p)[1], p.window, case.pos if p.window > 0 else None, options)
 
 
 def run_case(case, options=None, pool=None, with_desc=True):

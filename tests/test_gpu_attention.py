@@ -128,8 +128,9 @@ def test_chunked_prefill_then_decode_through_kv_save():
     for n in (128, 100, 71, 1):     # three prefill chunks, then one decode step
         p.rows_per_tile = 128 if n > 1 else 1
         trees = np.array([(s, s, 0, n)], abi.TREE_DT)
-        opts = host.options_mi355x(p.rows_per_tile, 512)
-        tiles, jobs, n_parts = host.plan_tiles(trees, p.Hkv, 0, None, opts)
+        resident, groups = device.plan_hint(p)
+        opts = host.options_mi355x(p.rows_per_tile, resident)
+        tiles, jobs, n_parts = host.plan_tiles(trees, groups, 0, None, opts)
         dp = device.DevicePass(p, trees, tiles, jobs, n_parts, 300, blocks, None, None)
         dp.run(Q, Kb, Vb, pool, O)
         saves = np.array(ho.kv_saves(s, s, n, [int(b) for b in blocks], p.bt), abi.KVSAVE_DT)
