@@ -249,6 +249,8 @@ def main():
     ap.add_argument("--tables", default="scattered", choices=["scattered", "contiguous"],
                     help="block tables: a seeded permutation of the pool (the benchmark's definition) or address order")
     ap.add_argument("--page", type=int, default=16, help="tokens per KV block (the benchmark's definition: 16)")
+    ap.add_argument("--copy-calibration", action="store_true",
+                    help="also run a plain 256 MiB device copy (for scaling rocprofv3 FETCH_SIZE / WRITE_SIZE readings)")
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
     args = ap.parse_args()
     if args.gpus != 1:
@@ -259,6 +261,13 @@ def main():
     assert torch.cuda.is_available(), "bench.py needs a GPU"
     device.init(0)
     w = make_workload(args.workload, args.workgroups or None, args.tables == "contiguous", args.page)
+    if args.copy_calibration:
+        src = torch.ones(256 << 20, dtype=torch.uint8, device="cuda")
+        dst = torch.empty_like(src)
+        for _ in range(3):
+            dst.copy_(src)   # a plain copy kernel of known size: reads 256 MiB, writes 256 MiB
+        torch.cuda.synchronize()
+        del src, dst
     K, W = args.steps, args.warmup
     for i in range(W):
         w.step(i)

@@ -425,34 +425,35 @@ __global__ __launch_bounds__(256) void attn_combine_kernel(const KArgs a, const 
   const int col = r * a.G + hg;
   const size_t stride = size_t(a.Hkv) * a.cols;  // records from one part to the next
   const size_t rec0 = (size_t(job.part0) * a.Hkv + kvh) * a.cols + col;
-  float M = -INFINITY;
-  for (int s = 0; s < job.nparts; ++s) M = fmaxf(M, a.parts_ml[(rec0 + s * stride) * 2]);
-  float L = 0.0f;
+  // One pass, 8 records in flight at a time, merged in part order with a running maximum
+  // (a loop that waits for each record's loads in turn is latency bound: the reference
+  // measured 39 us against 11 us for the same change, 40_attention.metal:801-803).
+  float M = -INFINITY, L = 0.0f;
   f32x4 o = {0, 0, 0, 0};
-  int s = 0;
-  for (; s + 4 <= job.nparts; s += 4) {  // 4 records in flight, summed in order
-    float m4[4], l4[4];
-    f32x4 o4[4];
+  for (int s = 0; s < job.nparts; s += 8) {
+    float m8[8], l8[8];
+    f32x4 o8[8];
 #pragma unroll
-    for (int i = 0; i < 4; ++i) {
-      const size_t rec = rec0 + size_t(s + i) * stride;
-      m4[i] = a.parts_ml[rec * 2];
-      l4[i] = a.parts_ml[rec * 2 + 1];
-      o4[i] = *reinterpret_cast<const f32x4*>(a.parts_o + rec * HD + d);
+    for (int i = 0; i < 8; ++i) {
+      const bool in = s + i < job.nparts;
+      const size_t rec = rec0 + size_t(in ? s + i : s) * stride;
+      m8[i] = in ? a.parts_ml[rec * 2] : -INFINITY;
+      l8[i] = a.parts_ml[rec * 2 + 1];
+      o8[i] = *reinterpret_cast<const f32x4*>(a.parts_o + rec * HD + d);
     }
+    float Mn = M;
 #pragma unroll
-    for (int i = 0; i < 4; ++i) {
-      const float w = (m4[i] == -INFINITY) ? 0.0f : fast_exp2(m4[i] - M);
-      L += w * l4[i];
-      o += o4[i] * w;
+    for (int i = 0; i < 8; ++i) Mn = fmaxf(Mn, m8[i]);
+    const float c = (M == -INFINITY) ? 0.0f : fast_exp2(M - Mn);
+    L *= c;
+    o *= c;
+    M = Mn;
+#pragma unroll
+    for (int i = 0; i < 8; ++i) {
+      const float w = (m8[i] == -INFINITY) ? 0.0f : fast_exp2(m8[i] - M);
+      L += w * l8[i];
+      o += o8[i] * w;
     }
-  }
-  for (; s < job.nparts; ++s) {
-    const size_t rec = rec0 + size_t(s) * stride;
-    const float ms = a.parts_ml[rec * 2];
-    const float w = (ms == -INFINITY) ? 0.0f : fast_exp2(ms - M);
-    L += w * a.parts_ml[rec * 2 + 1];
-    o += *reinterpret_cast<const f32x4*>(a.parts_o + rec * HD + d) * w;
   }
   const int row = job.r0 + r;
   const float inv = L > 0.0f ? 1.0f / L : 0.0f;
