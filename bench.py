@@ -40,6 +40,9 @@ class Workload:
         self.H, self.Hkv, self.HD, self.bt, self.window = H, Hkv, HD, bt, window
         self.seqs = list(seqs)
         p = synth.make_params(H, Hkv, HD, dtype, bt, window=window, rows_per_tile=rows_per_tile)
+        if rows_per_tile > 32:  # a prefill pass: plan with the largest tile the tiled kernel takes
+            rows_per_tile = device.plan_hint3(p)[2]
+            p.rows_per_tile = rows_per_tile
         self.params = p
         tdt = torch.float16 if dtype == abi.ESP_F16 else torch.bfloat16
         g = torch.Generator(device="cuda")

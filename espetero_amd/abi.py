@@ -62,7 +62,7 @@ _ERR = (C.c_char_p, C.c_size_t)
 ATTN_SYMBOLS = {
     "esp_attn_init": (C.c_int, (C.c_int,) + _ERR),
     "esp_attn_abi_version": (C.c_int, ()),
-    "esp_attn_plan_hint": (C.c_int, (_P, C.c_int, C.POINTER(C.c_int32), C.POINTER(C.c_int32)) + _ERR),
+    "esp_attn_plan_hint": (C.c_int, (_P, C.c_int, C.POINTER(C.c_int32), C.POINTER(C.c_int32), C.POINTER(C.c_int32)) + _ERR),
     "esp_attn_workspace_bytes": (C.c_size_t, (_P, C.c_int32, C.c_int32)),
     "esp_attn_forward": (C.c_int, (_P, _V, _V, _V, _V, _V, _V, _V, _V, _V, C.c_int32, _V, C.c_int32, _V, C.c_int32,
                                    C.c_int32, C.c_int32, _V, C.c_size_t, _V) + _ERR),

@@ -21,6 +21,7 @@ hipError_t launch_kv_relayout(const esp_attn_params* p, const void* src, void* d
 hipError_t launch_vt_stage(const esp_attn_params* p, const void* Vb, void* vt, int n_rows, hipStream_t st);
 int stream_workgroups_per_cu(int HD, int NC);
 int tiled_workgroups_per_cu(int HD);
+int tiled_max_rows(int HD);
 }  // namespace esp
 
 namespace {
@@ -121,10 +122,10 @@ int esp_attn_init(int device, char* err, size_t errlen) {
   return ESP_OK;
 }
 
-int esp_attn_plan_hint(const esp_attn_params* p, int device, int32_t* workgroups, int32_t* groups_per_tile, char* err,
-                       size_t errlen) {
+int esp_attn_plan_hint(const esp_attn_params* p, int device, int32_t* workgroups, int32_t* groups_per_tile,
+                       int32_t* max_rows, char* err, size_t errlen) {
   if (int rc = check_params(p, err, errlen)) return rc;
-  if (!workgroups || !groups_per_tile || p->rows_per_tile <= 0)
+  if (!workgroups || !groups_per_tile || !max_rows || p->rows_per_tile <= 0)
     return fail(err, errlen, ESP_EINVAL, "NULL output or rows_per_tile <= 0");
   int cus = 0;
   hipError_t e = hipDeviceGetAttribute(&cus, hipDeviceAttributeMultiprocessorCount, device);
@@ -132,6 +133,7 @@ int esp_attn_plan_hint(const esp_attn_params* p, int device, int32_t* workgroups
   const int fam = family(p);
   *workgroups = cus * (fam > 0 ? esp::stream_workgroups_per_cu(p->head_dim, fam) : esp::tiled_workgroups_per_cu(p->head_dim));
   *groups_per_tile = fam > 0 ? p->Hkv : p->H;
+  *max_rows = esp::tiled_max_rows(p->head_dim);
   return ESP_OK;
 }
 
@@ -157,8 +159,9 @@ int esp_attn_forward(const esp_attn_params* p, const void* Q, const void* Kb, co
   if (n_jobs > 0 && n_parts == 0) return fail(err, errlen, ESP_EINVAL, "n_jobs %d without partial records", n_jobs);
   if (!(p->scale > 0.0f)) return fail(err, errlen, ESP_EINVAL, "scale must be positive");
   const int fam = family(p);
-  if (fam < 0 && p->rows_per_tile > 128)
-    return fail(err, errlen, ESP_EUNSUPPORTED, "rows_per_tile %d: the tiled kernel takes at most 128 rows per tile", p->rows_per_tile);
+  if (fam < 0 && p->rows_per_tile > esp::tiled_max_rows(p->head_dim))
+    return fail(err, errlen, ESP_EUNSUPPORTED, "rows_per_tile %d: the tiled kernel takes at most %d rows per tile at head_dim %d",
+                p->rows_per_tile, esp::tiled_max_rows(p->head_dim), p->head_dim);
   const Carve c = carve(p, n_rows, n_parts);
   if (!workspace || workspace_bytes < c.total)
     return fail(err, errlen, ESP_EWORKSPACE, "workspace %zu bytes, %zu needed", workspace_bytes, c.total);

@@ -41,10 +41,15 @@ def to_dev(a, device="cuda"):
 def plan_hint(params, device=0):
     """(workgroups resident at once, workgroups per tile) of the kernel serving `params`:
     the planner's split target and its `groups` argument."""
+    return plan_hint3(params, device)[:2]
+
+
+def plan_hint3(params, device=0):
+    """plan_hint plus the largest rows_per_tile the tiled kernel takes at this head_dim."""
     err = C.create_string_buffer(_ERRLEN)
-    n, g = C.c_int32(0), C.c_int32(0)
-    abi.check(abi.attn_lib().esp_attn_plan_hint(C.byref(params), device, C.byref(n), C.byref(g), err, _ERRLEN), err)
-    return n.value, g.value
+    n, g, r = C.c_int32(0), C.c_int32(0), C.c_int32(0)
+    abi.check(abi.attn_lib().esp_attn_plan_hint(C.byref(params), device, C.byref(n), C.byref(g), C.byref(r), err, _ERRLEN), err)
+    return n.value, g.value, r.value
 
 
 def workspace_bytes(params, n_rows, n_parts):

@@ -125,9 +125,12 @@ int esp_attn_abi_version(void);
  *   groups_per_tile workgroups one tile becomes: KV heads for the streaming
  *                   kernel (the G heads of a KV head share a workgroup), query
  *                   heads for the tiled kernel (the reference: KV heads x SPLIT,
- *                   forest.h:2920, gemma.h:231). */
-int esp_attn_plan_hint(const esp_attn_params* p, int device, int32_t* workgroups, int32_t* groups_per_tile, char* err,
-                       size_t errlen);
+ *                   forest.h:2920, gemma.h:231);
+ *   max_rows        the largest rows_per_tile the tiled kernel takes at this
+ *                   head_dim: what a prefill pass should plan with (the
+ *                   reference: 8, or 16 on Spark prompt passes, gemma.h:137-142). */
+int esp_attn_plan_hint(const esp_attn_params* p, int device, int32_t* workgroups, int32_t* groups_per_tile,
+                       int32_t* max_rows, char* err, size_t errlen);
 
 /* Bytes of `workspace` esp_attn_forward needs for a pass of n_rows batch rows
  * whose plan holds n_parts partial records (replaces the reference's `parts`
