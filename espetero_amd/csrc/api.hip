@@ -131,7 +131,9 @@ int esp_attn_plan_hint(const esp_attn_params* p, int device, int32_t* workgroups
   hipError_t e = hipDeviceGetAttribute(&cus, hipDeviceAttributeMultiprocessorCount, device);
   if (e != hipSuccess) return hip_fail(err, errlen, "hipDeviceGetAttribute", e);
   const int fam = family(p);
-  *workgroups = cus * (fam > 0 ? esp::stream_workgroups_per_cu(p->head_dim, fam) : esp::tiled_workgroups_per_cu(p->head_dim));
+  // Streaming kernel: one resident round (its per-workgroup set-up is what a second round would
+  // pay again). Tiled kernel: four rounds, so that tiles of unequal length pack the CUs evenly.
+  *workgroups = cus * (fam > 0 ? esp::stream_workgroups_per_cu(p->head_dim, fam) : 4 * esp::tiled_workgroups_per_cu(p->head_dim));
   *groups_per_tile = fam > 0 ? p->Hkv : p->H;
   *max_rows = esp::tiled_max_rows(p->head_dim);
   return ESP_OK;

@@ -3,7 +3,7 @@
 // bound: Q K^T and P V run on v_mfma_f32_32x32x16 with K and V^T staged in LDS.
 //
 // Semantics: the reference's 8-row tile kernels (kernels/40_attention.metal:155-343,
-// kernels/80_gemma.metal:157-342) with the tile enlarged to up to 256 rows:
+// kernels/80_gemma.metal:157-342) with the tile enlarged to up to 128 rows:
 // cached keys [k0, k1) through the block table or ring, then the tree's batch
 // keys (`last` tiles) under the tree mask (80_:284) and the window (80_:285),
 // online softmax in fp32, P rounded to the storage type before P.V, output
@@ -11,9 +11,11 @@
 // partial record for attention_combine.
 //
 // Mapping to gfx950. One workgroup = one tile of query rows x one query head,
-// 4 wavefronts; a wavefront owns CT column tiles of 32 rows (CT = 2 at head
-// dim 128: 256-row tiles; CT = 1 at head dim 256: 128-row tiles), so every K /
-// V^T operand read from LDS feeds CT matrix instructions. Keys advance in steps
+// 4 wavefronts; a wavefront owns CT column tiles of 32 rows. CT = 1 (128-row
+// tiles) is what is built: at CT = 2 the accumulators of two column tiles no
+// longer fit the 256 architectural registers next to the operands and the
+// compiler's copies through the accumulation registers cost more than the
+// halved LDS reads gain. Keys advance in steps
 // of 64 (four 16-key sub-blocks: one page each at page size 16); wavefront w
 // stages sub-block w of a step: K rows as they lie in the pool, V already
 // transposed in the pool (batch rows: K from the pass's row-major Kb, V from the
@@ -40,7 +42,7 @@ struct SubBlock {  // one 16-key sub-block of a step: where its K rows and V^T r
   int kind;        // 0 cached, 1 batch, 2 none
 };
 
-// KST: LDS stages of K (3: one barrier per step; 2: a second barrier frees K(i) before K(i + 2) lands).
+// KST: LDS stages of K and V^T (2: step i + 1 is written while step i is in the matrix cores).
 template <int DT, int HD, int CT, int KST, int OCC>
 __global__ __launch_bounds__(256, OCC) void attn_tiled_kernel(const KArgs a, int n_tiles) {
   constexpr int KS = HD / 16, NT = HD / 32, LDK = HD + 8, LDV = 64 + 8;

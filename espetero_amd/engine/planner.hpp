@@ -48,6 +48,11 @@ struct PlanOptions {
     o.max_splits = 256;
     o.min_span = 128;
     o.balanced = true;
+    if (rows > 32) {  // tiled kernel: 64-key steps, and a split part must amortise its partial record
+      o.granule = 64;
+      o.min_chunk = 512;
+      o.min_span = 1024;
+    }
     return o;
   }
 };
@@ -70,6 +75,7 @@ inline void plan_tiles(AttnPlan& A, int groups, int window, const int32_t* pos, 
   const int R = o.rows_per_tile;
   struct RowTile {
     int tree, r, k0, b0, span;
+    int batch;  // batch keys the tile scans after its cached range (balanced rule: part of its work)
   };
   std::vector<RowTile> rts;
   long long total_span = 0;
@@ -85,8 +91,10 @@ inline void plan_tiles(AttnPlan& A, int groups, int window, const int32_t* pos, 
         k0 = std::clamp(minpos - window + 1, 0, t.P);
         b0 = std::max(0, minpos - window + 1 - t.P);
       }
-      rts.push_back({ti, r, k0, b0, t.P - k0});
-      total_span += t.P - k0;
+      // A causal tile scans the batch rows up to its own last row; one split part takes them all.
+      const int batch = o.balanced ? std::max(0, std::min(t.M, r + R) - b0) : 0;
+      rts.push_back({ti, r, k0, b0, t.P - k0, batch});
+      total_span += t.P - k0 + batch;
     }
   }
   const int n_tiles = int(rts.size());
@@ -99,7 +107,7 @@ inline void plan_tiles(AttnPlan& A, int groups, int window, const int32_t* pos, 
     auto tiles_at = [&](long long chunk) {
       long long n = 0;
       for (const RowTile& rt : rts)
-        n += rt.span >= o.min_span ? std::min<long long>((rt.span + chunk - 1) / chunk, o.max_splits) : 1;
+        n += rt.span >= o.min_span ? std::min<long long>((rt.span + rt.batch + chunk - 1) / chunk, o.max_splits) : 1;
       return n;
     };
     long long lo = std::max(1, o.min_chunk / o.granule), hi = std::max<long long>(lo, (total_span + o.granule - 1) / o.granule + 1);
@@ -116,7 +124,7 @@ inline void plan_tiles(AttnPlan& A, int groups, int window, const int32_t* pos, 
     int ns = 1;
     if (budget > 1 && span >= o.min_span) {
       if (o.balanced) {
-        ns = std::min((span + chunk_all - 1) / chunk_all, o.max_splits);
+        ns = std::min((span + rt.batch + chunk_all - 1) / chunk_all, o.max_splits);
       } else if (o.split > 0) {
         const int chunk =
             std::max(std::max(32, o.min_chunk),
@@ -131,17 +139,33 @@ inline void plan_tiles(AttnPlan& A, int groups, int window, const int32_t* pos, 
       A.tiles.push_back({rt.tree, t.base + rt.r, rt.k0, t.P, -1, 1, rt.b0, pad});
       continue;
     }
-    const int per = (span + ns - 1) / ns;
+    // Balanced rule: the batch keys count as work of the last part, so the cached range is
+    // cut into parts of (cached + batch) / ns keys and the last part keeps what is left.
+    const int per = (span + rt.batch + ns - 1) / ns;
     const int step = (per + o.granule - 1) / o.granule * o.granule;
     const int part0 = A.parts;
     int used = 0;
-    for (int k = rt.k0; k < t.P; ++used) {
-      int k1 = std::min(t.P, k + step);
-      // Balanced rule: a windowed range starts anywhere, its inner boundaries still fall on page multiples.
-      if (o.balanced && k1 < t.P) k1 = std::max(k + o.granule, k1 / o.granule * o.granule);
-      k1 = std::min(t.P, k1);
-      A.tiles.push_back({rt.tree, t.base + rt.r, k, k1, A.parts++, k1 >= t.P ? 1 : 0, rt.b0, pad});
-      k = k1;
+    if (o.balanced) {
+      // ns parts: all but the last are `step` cached keys on page multiples; the last keeps the
+      // rest of the cached range (possibly nothing) and the batch keys.
+      int k = rt.k0;
+      for (int p = 0; p < ns; ++p) {
+        const bool is_last = p + 1 == ns;
+        int k1 = t.P;
+        if (!is_last) {
+          k1 = std::min(t.P, k + step);
+          if (k1 < t.P) k1 = std::min(t.P, std::max(k + o.granule, k1 / o.granule * o.granule));
+          if (k1 == k) continue;  // the cached range ran out: the batch keys alone fill the last part
+        }
+        A.tiles.push_back({rt.tree, t.base + rt.r, k, k1, A.parts++, is_last ? 1 : 0, rt.b0, pad});
+        k = k1;
+        ++used;
+      }
+    } else {
+      for (int k = rt.k0; k < t.P; k += step, ++used) {
+        const int k1 = std::min(t.P, k + step);
+        A.tiles.push_back({rt.tree, t.base + rt.r, k, k1, A.parts++, k1 >= t.P ? 1 : 0, rt.b0, pad});
+      }
     }
     A.combine.push_back({t.base + rt.r, std::min(R, t.M - rt.r), part0, used});
   }

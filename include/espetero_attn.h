@@ -118,10 +118,11 @@ int esp_attn_abi_version(void);
 
 /* What the planner needs to know about the kernel that serves these params
  * (rows_per_tile x G packed rows, head_dim, dtype):
- *   workgroups      how many of its workgroups are resident on the device at
- *                   once. A pass split into more runs in rounds and pays the
- *                   per-workgroup set-up again (the reference aims at a fixed
- *                   256 threadgroups, forest.h:1385);
+ *   workgroups      how many workgroups a pass should be split up to: what is
+ *                   resident at once for the streaming kernel (a second round
+ *                   pays its per-workgroup set-up again), four rounds of that
+ *                   for the tiled kernel (the reference aims at a fixed 256
+ *                   threadgroups, forest.h:1385);
  *   groups_per_tile workgroups one tile becomes: KV heads for the streaming
  *                   kernel (the G heads of a KV head share a workgroup), query
  *                   heads for the tiled kernel (the reference: KV heads x SPLIT,
