@@ -35,6 +35,8 @@
 // Keys a row must not see get S = -inf before the softmax; V of keys outside the
 // tile's range (cached memory possibly never written) is zeroed in LDS by the
 // wavefront that staged it, so 0 * garbage never reaches the accumulators.
+#include <utility>
+
 #include "common.hpp"
 
 namespace esp {
@@ -181,11 +183,12 @@ __global__ __launch_bounds__(256, OCC) void attn_tiled_kernel(const KArgs a, int
   const uint32_t voff_c = uint32_t(l32 * a.bt * 2 + hb * 16);
   const uint32_t voff_b = uint32_t(l32 * 32 + hb * 16);
 
-  auto fill = [&](int step, int stage) __attribute__((always_inline)) {
+  // interior: the caller knows that all four sub-blocks of the step are cached keys.
+  auto fill = [&](int step, int stage, auto interior) __attribute__((always_inline)) {
     const int s = 4 * step + wave;
     const uint32_t kdst = lds_base + stage * KBUF + wave * (16 * ROWB);
     const uint32_t vdst = lds_base + VOFF + stage * VBUF + wave * SUBV;
-    if (s < n_c) {
+    if (decltype(interior)::value || s < n_c) {
       const int js = (c0 + s) << 4;
       const int b = block_id(step);
       const int t0 = a.bt == 16 ? 0 : js % a.bt;
@@ -259,23 +262,60 @@ __global__ __launch_bounds__(256, OCC) void attn_tiled_kernel(const KArgs a, int
     return ((a0 + s0 - n_c) << 4) - tree.base > wave_last;
   };
 
-  // S^T of half step kt of the step in stage S: s[4 i + j] is S^T row 8 i + 4 hb + j, which is key
-  // 32 kt + pi(8 i + 4 hb + j) = 32 kt + 16 (i / 2) + 8 hb + 4 (i % 2) + j of the step.
-  auto qk = [&]<int S>(int kt, f32x16& s) __attribute__((always_inline)) {
-    const char* kp = lds + S * KBUF + kt * 32 * ROWB;
+  // A step's matrix work is 4 KS operand reads from LDS, each feeding one matrix instruction:
+  // Q K^T of keys 0..31 (KS reads of K), Q K^T of keys 32..63, P V of keys 0..31 (KS reads of
+  // V^T), P V of keys 32..63. They run in groups of GP operands through two register buffers:
+  // while the matrix cores consume one group, the reads of the next are in flight, and the
+  // softmax of a half step sits beside the matrix work of the following group.
+  constexpr int GP = 8;           // operands per group
+  constexpr int GK = KS / GP;     // groups per half step of Q K^T (and of P V)
+  constexpr int NG = 4 * GK;      // groups per step
+  f32x16 s[2];                    // S^T of the two half steps: s[kt][4 i + j] is S^T row 8 i + 4 hb + j, which is key
+                                  // 32 kt + pi(8 i + 4 hb + j) = 32 kt + 16 (i / 2) + 8 hb + 4 (i % 2) + j of the step
+  u32x4 pb[2][2];                 // P^T of the two half steps as matrix operands
+  u32x4 ring[2][GP];
+
+  auto read_group = [&]<int S, int G>(u32x4 (&buf)[GP]) __attribute__((always_inline)) {
+    if constexpr (G < 2 * GK) {
+      constexpr int kt = G / GK, ks0 = (G % GK) * GP;
+      const char* kp = lds + S * KBUF + kt * 32 * ROWB;
 #pragma unroll
-    for (int i = 0; i < 16; ++i) s[i] = 0.0f;
+      for (int j = 0; j < GP; ++j) buf[j] = *reinterpret_cast<const u32x4*>(kp + kaddr[ks0 + j]);
+    } else {
+      // Operand o = 2 nt + t of half step kt: keys 8 hb .. 8 hb + 7 of sub-block 2 kt + t, dims 32 nt .. : the
+      // lane's 16 bytes of that sub-block's dim group.
+      constexpr int kt = (G - 2 * GK) / GK, o0 = ((G - 2 * GK) % GK) * GP;
+      const char* vp = lds + VOFF + S * VBUF + 2 * kt * SUBV + lane * 16;
 #pragma unroll
-    for (int ks = 0; ks < KS; ++ks) {
-      const u32x4 kf = *reinterpret_cast<const u32x4*>(kp + kaddr[ks]);
-      s = mfma32x16<DT>(kf, qf[ks], s);
+      for (int j = 0; j < GP; ++j) buf[j] = *reinterpret_cast<const u32x4*>(vp + ((o0 + j) & 1) * SUBV + ((o0 + j) >> 1) * 1024);
+    }
+  };
+  auto mma_group = [&]<int G>(const u32x4 (&buf)[GP]) __attribute__((always_inline)) {
+    if constexpr (G < 2 * GK) {
+      constexpr int kt = G / GK, ks0 = (G % GK) * GP;
+      if constexpr (ks0 == 0) {
+#pragma unroll
+        for (int i = 0; i < 16; ++i) s[kt][i] = 0.0f;
+      }
+#pragma unroll
+      for (int j = 0; j < GP; ++j) s[kt] = mfma32x16<DT>(buf[j], qf[ks0 + j], s[kt]);
+    } else {
+      constexpr int kt = (G - 2 * GK) / GK, o0 = ((G - 2 * GK) % GK) * GP;
+#pragma unroll
+      for (int j = 0; j < GP; ++j) acc[(o0 + j) >> 1] = mfma32x16<DT>(buf[j], pb[kt][(o0 + j) & 1], acc[(o0 + j) >> 1]);
     }
   };
 
-  // Masks (cold path), online softmax, O^T += V^T . P^T of half step (step, kt) in stage S.
-  auto softmax_pv = [&]<int S>(int step, int kt, f32x16& s) __attribute__((always_inline)) {
-    bool half_full;  // all 32 keys visible to every row of this wavefront?
-    {
+  // Online softmax of half step (step, kt), first part: masks (cold path) and the running
+  // reference. Everything with a branch in it lives here, so that the second part is straight-line
+  // code the scheduler can lay between the matrix instructions of the next group.
+  float corr_late = 1.0f;
+  bool late = false;
+  auto softmax_pre = [&](int step, auto kt_c, auto interior) __attribute__((always_inline)) {
+    constexpr int kt = decltype(kt_c)::value;
+    f32x16& sv = s[kt];
+    bool half_full = true;  // all 32 keys visible to every row of this wavefront?
+    if constexpr (!decltype(interior)::value) {
       const int s0 = 4 * step + 2 * kt;
       if (s0 + 2 <= n_c) {
         const int j0 = (c0 + s0) << 4;
@@ -312,7 +352,7 @@ __global__ __launch_bounds__(256, OCC) void attn_tiled_kernel(const KArgs a, int
           const int j = j0 + 8 * hb + e;
           bool vis = (j >= lo && j <= hi) || (j >= 0 && j < anc);
           if (batch && a.window > 0 && vis) vis = qpos - a.pos[tree.base + j].x < a.window;
-          s[8 * t + e] = vis ? s[8 * t + e] : -INFINITY;
+          sv[8 * t + e] = vis ? sv[8 * t + e] : -INFINITY;
         }
       }
     }
@@ -322,7 +362,7 @@ __global__ __launch_bounds__(256, OCC) void attn_tiled_kernel(const KArgs a, int
     // m_run because both take the maximum over the pair whenever either wants to move.
     float x = -INFINITY;
 #pragma unroll
-    for (int i = 0; i < 16; ++i) x = fmaxf(x, s[i]);
+    for (int i = 0; i < 16; ++i) x = fmaxf(x, sv[i]);
     x *= a.scale_log2;  // scale > 0: the max commutes with it
     if (__any(x > m_run + 8.0f)) {
       asm volatile("s_nop 0");  // a real branch: this block must not be speculated into the loop body
@@ -330,33 +370,69 @@ __global__ __launch_bounds__(256, OCC) void attn_tiled_kernel(const KArgs a, int
       const float corr = (m_new == -INFINITY) ? 1.0f : fast_exp2(m_run - m_new);
       m_run = m_new;
       l_run *= corr;
+      if constexpr (kt == 0) {
 #pragma unroll
-      for (int nt = 0; nt < NT; ++nt) acc[nt] *= corr;
+        for (int nt = 0; nt < NT; ++nt) acc[nt] *= corr;
+      } else {
+        // P V of the first half step is still to be accumulated and its P is relative to the old
+        // reference: the accumulators take this factor once those products are in.
+        corr_late = corr;
+        late = true;
+      }
     }
+  };
+  // Second part: s[kt] -> pb[kt], the lane's share of the row sum.
+  auto softmax_exp = [&](auto kt_c) __attribute__((always_inline)) {
+    constexpr int kt = decltype(kt_c)::value;
     const float m_safe = (m_run == -INFINITY) ? 0.0f : m_run;
-    u32x4 pb[2];
     float ps = 0.0f;
 #pragma unroll
     for (int t = 0; t < 2; ++t) {
       float p[8];
 #pragma unroll
       for (int e = 0; e < 8; ++e) {
-        p[e] = fast_exp2(__builtin_fmaf(s[8 * t + e], a.scale_log2, -m_safe));
+        p[e] = fast_exp2(__builtin_fmaf(s[kt][8 * t + e], a.scale_log2, -m_safe));
         ps += p[e];
       }
-      pb[t] = u32x4{pack2<DT>(p[0], p[1]), pack2<DT>(p[2], p[3]), pack2<DT>(p[4], p[5]), pack2<DT>(p[6], p[7])};
+      // keys 8 hb .. 8 hb + 7 of sub-block 2 kt + t
+      pb[kt][t] = u32x4{pack2<DT>(p[0], p[1]), pack2<DT>(p[2], p[3]), pack2<DT>(p[4], p[5]), pack2<DT>(p[6], p[7])};
     }
     l_run += ps;
-    // pb[t] holds keys 8 hb .. 8 hb + 7 of sub-block 2 kt + t: the V^T operand of the same keys
-    // is the lane's 16 bytes of that sub-block's dim group.
-    const char* vp = lds + VOFF + S * VBUF + 2 * kt * SUBV + lane * 16;
+    // Pin the results here: without a use in this block the arithmetic above is sunk to the
+    // block of its first real use, away from the matrix instructions it should overlap with.
+    asm volatile("" : "+v"(pb[kt][0]), "+v"(pb[kt][1]), "+v"(l_run));
+  };
+
+  // Phase G of a step: reads of group G + 1, matrix work of group G, and the softmax whose
+  // Q K^T finished with the previous group.
+  auto phase = [&]<int S, int G>(int step, auto interior) __attribute__((always_inline)) {
+    if constexpr (G + 1 < NG) read_group.template operator()<S, G + 1>(ring[(G + 1) & 1]);
+    if constexpr (G == GK) softmax_pre(step, std::integral_constant<int, 0>{}, interior);
+    if constexpr (G == 2 * GK) softmax_pre(step, std::integral_constant<int, 1>{}, interior);
+    __builtin_amdgcn_sched_barrier(0);
+    mma_group.template operator()<G>(ring[G & 1]);
+    if constexpr (G == GK) softmax_exp(std::integral_constant<int, 0>{});
+    if constexpr (G == 2 * GK) softmax_exp(std::integral_constant<int, 1>{});
+    if constexpr (G == GK || G == 2 * GK) {
+      // one matrix instruction, then its share of the softmax arithmetic
 #pragma unroll
-    for (int nt = 0; nt < NT; ++nt)
-#pragma unroll
-      for (int t = 0; t < 2; ++t) {
-        const u32x4 vf = *reinterpret_cast<const u32x4*>(vp + t * SUBV + nt * 1024);
-        acc[nt] = mfma32x16<DT>(vf, pb[t], acc[nt]);
+      for (int j = 0; j < GP; ++j) {
+        __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
+        __builtin_amdgcn_sched_group_barrier(0x002, 8, 0);
       }
+    }
+    __builtin_amdgcn_sched_barrier(0);
+    if constexpr (G == 3 * GK - 1) {  // P V of the first half step is in: the deferred rescale
+      if (late) {
+        asm volatile("s_nop 0");
+#pragma unroll
+        for (int nt = 0; nt < NT; ++nt) acc[nt] *= corr_late;
+        late = false;
+      }
+    }
+  };
+  auto phases = [&]<int S, int... G>(int step, auto interior, std::integer_sequence<int, G...>) __attribute__((always_inline)) {
+    (phase.template operator()<S, G>(step, interior), ...);
   };
 
   // Steps this wavefront computes: batch steps past its last row hold nothing it can see.
@@ -364,38 +440,67 @@ __global__ __launch_bounds__(256, OCC) void attn_tiled_kernel(const KArgs a, int
   while (my_steps > 0 && skipped(my_steps - 1)) --my_steps;
 
   // Iteration i: request step i + 1 into the other stage (every wavefront left it at the
-  // previous barrier), do the math of step i in two halves of 32 keys so the second half's
-  // Q K^T sits next to the first half's softmax, wait for the own loads, barrier.
-  f32x16 sa, sb;
-  auto iter = [&]<int S>(int i) __attribute__((always_inline)) {
-    if (i + 1 < n_steps) fill(i + 1, S ^ 1);
-    qk.template operator()<S>(0, sa);
-    qk.template operator()<S>(1, sb);
-    softmax_pv.template operator()<S>(i, 0, sa);
-    softmax_pv.template operator()<S>(i, 1, sb);
+  // previous barrier), the matrix work and softmax of step i, wait for the own loads, barrier.
+  // interior: every key of steps i and i + 1 is a cached key inside [k0, k1) that every row of
+  // the tile sees: no masks, no edges, one kind of load.
+  auto iter = [&]<int S>(int i, auto interior) __attribute__((always_inline)) {
+    if (decltype(interior)::value || i + 1 < n_steps) fill(i + 1, S ^ 1, interior);
+    read_group.template operator()<S, 0>(ring[0]);
+    __builtin_amdgcn_sched_barrier(0);
+    phases.template operator()<S>(i, interior, std::make_integer_sequence<int, NG>{});
     wait_loads();
-    if (i + 1 < n_steps) fix(i + 1, S ^ 1);
+    if constexpr (!decltype(interior)::value) {
+      if (i + 1 < n_steps) fix(i + 1, S ^ 1);
+    }
     __syncthreads();
   };
+  // Steps [int_lo, int_hi) are interior.
+  int int_lo, int_hi;
+  {
+    const int first = c0 << 4;  // key of sub-block 0
+    int lo_key = tile.k0;
+    if (a.window > 0) lo_key = max(lo_key, qpos_max - a.window + 1);
+    int_lo = lo_key <= first ? 0 : (lo_key - first + 63) >> 6;
+    const int full_steps = ((tile.k1 >> 4) - c0) >> 2;  // steps wholly inside the cached range
+    int_hi = min(full_steps - 1, my_steps);
+  }
+  constexpr std::false_type general{};
+  constexpr std::true_type inner{};
 
   if (n_steps > 0) {
-    fill(0, 0);
+    fill(0, 0, general);
     wait_loads();
     fix(0, 0);
   }
   __syncthreads();
+  // Pairs of steps (one per stage): general ones up to the interior range, the interior
+  // range, general ones again. The two general stretches share one loop's code.
+  const int in0 = min((int_lo + 1) & ~1, my_steps & ~1);
+  const int in1 = int_hi > in0 ? in0 + ((int_hi - in0) & ~1) : in0;
   int i = 0;
-  for (; i + 2 <= my_steps; i += 2) {
-    iter.template operator()<0>(i);
-    iter.template operator()<1>(i + 1);
+#pragma nounroll
+  for (int seg = 0; seg < 2; ++seg) {
+    const int bound = seg == 0 ? in0 : my_steps;
+#pragma nounroll
+    for (; i + 2 <= bound; i += 2) {
+      iter.template operator()<0>(i, general);
+      iter.template operator()<1>(i + 1, general);
+    }
+    if (seg == 0) {
+#pragma nounroll
+      for (; i + 2 <= in1; i += 2) {
+        iter.template operator()<0>(i, inner);
+        iter.template operator()<1>(i + 1, inner);
+      }
+    }
   }
   if (i < my_steps) {
-    iter.template operator()<0>(i);
+    iter.template operator()<0>(i, general);
     ++i;
   }
   for (; i < n_steps; ++i) {  // keep staging for the wavefronts whose rows reach further
     if (i + 1 < n_steps) {
-      fill(i + 1, (i + 1) & 1);
+      fill(i + 1, (i + 1) & 1, general);
       wait_loads();
       fix(i + 1, (i + 1) & 1);
     }
