@@ -158,6 +158,21 @@ __global__ __launch_bounds__(256, OCC) void attn_tiled_kernel(const KArgs a, int
   const int n_steps = (n_sb + 3) >> 2;
   const int n_groups = (a.n_rows + 15) >> 4;
 
+  // Windowed layers: do this tile's batch keys need the per-key position test at all? Not when
+  // the oldest position among them is inside the window of the row with the largest position.
+  bool batch_window = false;
+  if (a.window > 0 && n_b > 0) {
+    int kp = INT32_MAX;
+    for (int j = tile.b0 + int(threadIdx.x); j <= k_last; j += 256) kp = min(kp, a.pos[tree.base + j].x);
+#pragma unroll
+    for (int o = 32; o >= 1; o >>= 1) kp = min(kp, __shfl_xor(kp, o));
+    __syncthreads();  // every wavefront has read the facts above
+    if (lane == 0) red[wave][0] = kp;
+    __syncthreads();
+    kp = min(min(red[0][0], red[1][0]), min(red[2][0], red[3][0]));
+    batch_window = qpos_max - __builtin_amdgcn_readfirstlane(kp) >= a.window;
+  }
+
   // Block ids of this wavefront's cached sub-blocks, 64 steps at a time: lane l holds the
   // block of sub-block 4 (ids_step0 + l) + wave, so the per-step lookup is a lane read
   // instead of a dependent memory access in front of every staging load.
@@ -290,19 +305,20 @@ __global__ __launch_bounds__(256, OCC) void attn_tiled_kernel(const KArgs a, int
       for (int j = 0; j < GP; ++j) buf[j] = *reinterpret_cast<const u32x4*>(vp + ((o0 + j) & 1) * SUBV + ((o0 + j) >> 1) * 1024);
     }
   };
-  auto mma_group = [&]<int G>(const u32x4 (&buf)[GP]) __attribute__((always_inline)) {
+  // Operands [J0, J1) of group G.
+  auto mma_group = [&]<int G, int J0, int J1>(const u32x4 (&buf)[GP]) __attribute__((always_inline)) {
     if constexpr (G < 2 * GK) {
       constexpr int kt = G / GK, ks0 = (G % GK) * GP;
-      if constexpr (ks0 == 0) {
+      if constexpr (ks0 == 0 && J0 == 0) {
 #pragma unroll
         for (int i = 0; i < 16; ++i) s[kt][i] = 0.0f;
       }
 #pragma unroll
-      for (int j = 0; j < GP; ++j) s[kt] = mfma32x16<DT>(buf[j], qf[ks0 + j], s[kt]);
+      for (int j = J0; j < J1; ++j) s[kt] = mfma32x16<DT>(buf[j], qf[ks0 + j], s[kt]);
     } else {
       constexpr int kt = (G - 2 * GK) / GK, o0 = ((G - 2 * GK) % GK) * GP;
 #pragma unroll
-      for (int j = 0; j < GP; ++j) acc[(o0 + j) >> 1] = mfma32x16<DT>(buf[j], pb[kt][(o0 + j) & 1], acc[(o0 + j) >> 1]);
+      for (int j = J0; j < J1; ++j) acc[(o0 + j) >> 1] = mfma32x16<DT>(buf[j], pb[kt][(o0 + j) & 1], acc[(o0 + j) >> 1]);
     }
   };
 
@@ -322,7 +338,7 @@ __global__ __launch_bounds__(256, OCC) void attn_tiled_kernel(const KArgs a, int
         half_full = j0 >= tile.k0 && j0 + 32 <= tile.k1 && (a.window == 0 || qpos_max - j0 < a.window);
       } else if (s0 >= n_c && s0 + 2 <= n_sb) {
         const int j0 = ((a0 + s0 - n_c) << 4) - tree.base;
-        half_full = a.window == 0 && j0 >= seg_max && j0 + 31 <= rr0 + 32 * wave && j0 >= 0;
+        half_full = !batch_window && j0 >= seg_max && j0 + 31 <= rr0 + 32 * wave && j0 >= 0;
       } else {
         half_full = false;
       }
@@ -351,7 +367,7 @@ __global__ __launch_bounds__(256, OCC) void attn_tiled_kernel(const KArgs a, int
         for (int e = 0; e < 8; ++e) {
           const int j = j0 + 8 * hb + e;
           bool vis = (j >= lo && j <= hi) || (j >= 0 && j < anc);
-          if (batch && a.window > 0 && vis) vis = qpos - a.pos[tree.base + j].x < a.window;
+          if (batch && batch_window && vis) vis = qpos - a.pos[tree.base + j].x < a.window;
           sv[8 * t + e] = vis ? sv[8 * t + e] : -INFINITY;
         }
       }
@@ -407,19 +423,25 @@ __global__ __launch_bounds__(256, OCC) void attn_tiled_kernel(const KArgs a, int
   // Q K^T finished with the previous group.
   auto phase = [&]<int S, int G>(int step, auto interior) __attribute__((always_inline)) {
     if constexpr (G + 1 < NG) read_group.template operator()<S, G + 1>(ring[(G + 1) & 1]);
-    if constexpr (G == GK) softmax_pre(step, std::integral_constant<int, 0>{}, interior);
-    if constexpr (G == 2 * GK) softmax_pre(step, std::integral_constant<int, 1>{}, interior);
-    __builtin_amdgcn_sched_barrier(0);
-    mma_group.template operator()<G>(ring[G & 1]);
-    if constexpr (G == GK) softmax_exp(std::integral_constant<int, 0>{});
-    if constexpr (G == 2 * GK) softmax_exp(std::integral_constant<int, 1>{});
     if constexpr (G == GK || G == 2 * GK) {
-      // one matrix instruction, then its share of the softmax arithmetic
+      // The first matrix instructions of the group go out before the branchy part of the softmax,
+      // whose wait for the previous group's results they cover; the rest carry the arithmetic,
+      // one matrix instruction then its share.
+      constexpr int HEAD = 3;
+      mma_group.template operator()<G, 0, HEAD>(ring[G & 1]);
+      __builtin_amdgcn_sched_barrier(0);
+      softmax_pre(step, std::integral_constant<int, G == GK ? 0 : 1>{}, interior);
+      __builtin_amdgcn_sched_barrier(0);
+      mma_group.template operator()<G, HEAD, GP>(ring[G & 1]);
+      softmax_exp(std::integral_constant<int, G == GK ? 0 : 1>{});
 #pragma unroll
-      for (int j = 0; j < GP; ++j) {
+      for (int j = HEAD; j < GP; ++j) {
         __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
-        __builtin_amdgcn_sched_group_barrier(0x002, 8, 0);
+        __builtin_amdgcn_sched_group_barrier(0x002, 13, 0);
       }
+    } else {
+      __builtin_amdgcn_sched_barrier(0);
+      mma_group.template operator()<G, 0, GP>(ring[G & 1]);
     }
     __builtin_amdgcn_sched_barrier(0);
     if constexpr (G == 3 * GK - 1) {  // P V of the first half step is in: the deferred rescale
@@ -439,20 +461,26 @@ __global__ __launch_bounds__(256, OCC) void attn_tiled_kernel(const KArgs a, int
   int my_steps = n_steps;
   while (my_steps > 0 && skipped(my_steps - 1)) --my_steps;
 
-  // Iteration i: request step i + 1 into the other stage (every wavefront left it at the
-  // previous barrier), the matrix work and softmax of step i, wait for the own loads, barrier.
-  // interior: every key of steps i and i + 1 is a cached key inside [k0, k1) that every row of
+  // At the top of iteration i the barrier that publishes step i has been passed, step i + 1 is
+  // on its way into the other stage and the first operand group of step i is being read.
+  // The iteration: all groups but the last (reads one group ahead), then - every operand of the
+  // step now in registers - wait for the own loads of step i + 1, barrier, request step i + 2
+  // into the stage just left, start reading step i + 1, and only then the last group's matrix
+  // work: it covers the barrier, the address arithmetic of the loads and the first read latency.
+  // interior: every key of steps i .. i + 2 is a cached key inside [k0, k1) that every row of
   // the tile sees: no masks, no edges, one kind of load.
   auto iter = [&]<int S>(int i, auto interior) __attribute__((always_inline)) {
-    if (decltype(interior)::value || i + 1 < n_steps) fill(i + 1, S ^ 1, interior);
-    read_group.template operator()<S, 0>(ring[0]);
-    __builtin_amdgcn_sched_barrier(0);
-    phases.template operator()<S>(i, interior, std::make_integer_sequence<int, NG>{});
-    wait_loads();
+    phases.template operator()<S>(i, interior, std::make_integer_sequence<int, NG - 1>{});
+    asm volatile("s_waitcnt vmcnt(0) lgkmcnt(0)" ::: "memory");  // loads of step i + 1 landed, reads of stage S done
     if constexpr (!decltype(interior)::value) {
       if (i + 1 < n_steps) fix(i + 1, S ^ 1);
     }
     __syncthreads();
+    if (decltype(interior)::value || i + 2 < n_steps) fill(i + 2, S, interior);
+    read_group.template operator()<S ^ 1, 0>(ring[0]);
+    __builtin_amdgcn_sched_barrier(0);
+    mma_group.template operator()<NG - 1, 0, GP>(ring[(NG - 1) & 1]);
+    __builtin_amdgcn_sched_barrier(0);
   };
   // Steps [int_lo, int_hi) are interior.
   int int_lo, int_hi;
@@ -462,7 +490,7 @@ __global__ __launch_bounds__(256, OCC) void attn_tiled_kernel(const KArgs a, int
     if (a.window > 0) lo_key = max(lo_key, qpos_max - a.window + 1);
     int_lo = lo_key <= first ? 0 : (lo_key - first + 63) >> 6;
     const int full_steps = ((tile.k1 >> 4) - c0) >> 2;  // steps wholly inside the cached range
-    int_hi = min(full_steps - 1, my_steps);
+    int_hi = min(full_steps - 2, my_steps);
   }
   constexpr std::false_type general{};
   constexpr std::true_type inner{};
@@ -473,6 +501,9 @@ __global__ __launch_bounds__(256, OCC) void attn_tiled_kernel(const KArgs a, int
     fix(0, 0);
   }
   __syncthreads();
+  if (n_steps > 1) fill(1, 1, general);
+  read_group.template operator()<0, 0>(ring[0]);
+  __builtin_amdgcn_sched_barrier(0);
   // Pairs of steps (one per stage): general ones up to the interior range, the interior
   // range, general ones again. The two general stretches share one loop's code.
   const int in0 = min((int_lo + 1) & ~1, my_steps & ~1);
@@ -499,12 +530,10 @@ __global__ __launch_bounds__(256, OCC) void attn_tiled_kernel(const KArgs a, int
     ++i;
   }
   for (; i < n_steps; ++i) {  // keep staging for the wavefronts whose rows reach further
-    if (i + 1 < n_steps) {
-      fill(i + 1, (i + 1) & 1, general);
-      wait_loads();
-      fix(i + 1, (i + 1) & 1);
-    }
+    wait_loads();
+    if (i + 1 < n_steps) fix(i + 1, (i + 1) & 1);
     __syncthreads();
+    if (i + 2 < n_steps) fill(i + 2, i & 1, general);
   }
 
   // ---- output: lane (row l32, half hb) holds dims 32 nt + 8 i + 4 hb + j at acc[nt][4 i + j]
