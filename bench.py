@@ -140,6 +140,17 @@ def make_workload(name, workgroups=None, contiguous=False, page=16):
     raise SystemExit(f"unknown workload {name}")
 
 
+def measured_traffic(workload):
+    """HBM bytes one launch of the dominant kernel moves, as measured with the rocprofv3 FETCH_SIZE and
+    WRITE_SIZE counters (each scaled by what the same counter reads for a plain 256 MiB copy); the
+    summaries under profiles/ show the runs. None for a workload that has not been measured."""
+    try:
+        with open(os.path.join(ROOT, "profiles", "traffic.json")) as f:
+            return int(json.load(f)[workload]["hbm_bytes_per_launch"])
+    except (OSError, KeyError, ValueError):
+        return None
+
+
 WORKLOADS = ["c1_single_decode", "c2_batched_decode", "c3_prefill_p0", "c3_prefill_p2048", "c3_prefill_p4096",
              "c3_prefill_p6144", "c4_decode_sliding", "c4_decode_global", "c4_prefill_sliding", "c4_prefill_global",
              "c5_verify"]
@@ -302,7 +313,7 @@ def main():
                    "tiles": int(len(w.tiles)), "parts": int(w.n_parts), "rotation_sets": w.n_sets,
                    "pool_pages": w.pool_pages},
         "roofline": {"bound": w.bound, "achieved": round(achieved, 3), "peak": peak, "unit": unit,
-                     "frac": round(achieved / peak, 4), "traffic": None,
+                     "frac": round(achieved / peak, 4), "traffic": measured_traffic(w.name),
                      "kernel": "attn_stream_kernel" if w.bound == "hbm" and w.params.rows_per_tile * (w.H // w.Hkv) <= 32
                      else "attn_tiled_kernel",
                      "kernel_us_avg": round(kern_ms * 1e3, 3), "kernel_us_min": round(kern_min_ms * 1e3, 3),
