@@ -66,6 +66,7 @@ ATTN_SYMBOLS = {
     "esp_attn_workspace_bytes": (C.c_size_t, (_P, C.c_int32, C.c_int32)),
     "esp_attn_forward": (C.c_int, (_P, _V, _V, _V, _V, _V, _V, _V, _V, _V, C.c_int32, _V, C.c_int32, _V, C.c_int32,
                                    C.c_int32, C.c_int32, _V, C.c_size_t, _V) + _ERR),
+    "esp_attn_time_next": (C.c_int, (_V, _V)),
     "esp_attn_combine": (C.c_int, (_P, _V, _V, C.c_int32, C.c_int32, C.c_int32, _V, C.c_size_t, _V) + _ERR),
     "esp_kv_save": (C.c_int, (_P, _V, _V, _V, _V, C.c_int32, _V) + _ERR),
     "esp_kv_copy_blocks": (C.c_int, (_P, _V, _V, C.c_int32, C.c_int32, C.c_uint64, _V) + _ERR),

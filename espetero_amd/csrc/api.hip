@@ -109,6 +109,15 @@ esp::KArgs make_args(const esp_attn_params* p, const Carve& c, void* workspace, 
 
 }  // namespace
 
+namespace esp {
+static TimeNext g_time_next;
+TimeNext take_time_next() {
+  const TimeNext t = g_time_next;
+  g_time_next = TimeNext{};
+  return t;
+}
+}  // namespace esp
+
 extern "C" {
 
 int esp_attn_abi_version(void) { return ESP_ABI_VERSION; }
@@ -198,6 +207,13 @@ int esp_attn_forward(const esp_attn_params* p, const void* Q, const void* Kb, co
     e = esp::launch_combine(p->dtype, p->head_dim, a, jobs, n_jobs, st);
     if (e != hipSuccess) return hip_fail(err, errlen, "attn_combine launch", e);
   }
+  return ESP_OK;
+}
+
+int esp_attn_time_next(void* start_event, void* stop_event) {
+  if ((start_event == nullptr) != (stop_event == nullptr)) return ESP_EINVAL;
+  esp::g_time_next.start = static_cast<hipEvent_t>(start_event);
+  esp::g_time_next.stop = static_cast<hipEvent_t>(stop_event);
   return ESP_OK;
 }
 

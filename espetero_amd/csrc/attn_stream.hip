@@ -486,7 +486,7 @@ static hipError_t launch_stream_t(const KArgs& a, int n_tiles, hipStream_t st) {
     hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(k), hipFuncAttributeMaxDynamicSharedMemorySize, int(smem));
     if (e != hipSuccess) return e;
   }
-  hipLaunchKernelGGL(k, dim3(a.Hkv, n_tiles), dim3(256), smem, st, a);
+  launch_timed(k, dim3(a.Hkv, n_tiles), dim3(256), smem, st, a);
   return hipGetLastError();
 }
 

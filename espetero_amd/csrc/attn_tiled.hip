@@ -586,7 +586,7 @@ static hipError_t launch_tiled_t(const KArgs& a, int n_tiles, hipStream_t st) {
     hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(k), hipFuncAttributeMaxDynamicSharedMemorySize, int(smem));
     if (e != hipSuccess) return e;
   }
-  hipLaunchKernelGGL(k, dim3(unsigned(n_tiles) * a.H), dim3(256), smem, st, a, n_tiles);
+  launch_timed(k, dim3(unsigned(n_tiles) * a.H), dim3(256), smem, st, a, n_tiles);
   return hipGetLastError();
 }
 

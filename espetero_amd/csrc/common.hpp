@@ -4,6 +4,7 @@
 #pragma once
 
 #include <hip/hip_runtime.h>
+#include <hip/hip_ext.h>
 #include <stdint.h>
 
 #include "../../include/espetero_attn.h"
@@ -112,6 +113,23 @@ __device__ __forceinline__ size_t head_base(const KArgs& a, int HD, int b, int k
 __device__ __forceinline__ int block_of(const KArgs& a, int table, int j) {
   const int bi = j / a.bt;
   return a.ring ? table + bi % a.ring : a.blocks[table + bi];
+}
+
+// Events the next attention kernel launch records its own begin and end into (esp_attn_time_next);
+// both null otherwise. One caller thread drives the library, so a plain pair is enough.
+struct TimeNext {
+  hipEvent_t start = nullptr, stop = nullptr;
+};
+TimeNext take_time_next();  // returns the pair and clears it
+
+// Launches k; with a pending event pair the launch itself timestamps the kernel's begin and end.
+template <typename K, typename... Args>
+inline void launch_timed(K k, dim3 grid, dim3 block, size_t smem, hipStream_t st, Args... args) {
+  const TimeNext t = take_time_next();
+  if (t.start && t.stop)
+    hipExtLaunchKernelGGL(k, grid, block, smem, st, t.start, t.stop, 0, args...);
+  else
+    hipLaunchKernelGGL(k, grid, block, smem, st, args...);
 }
 
 }  // namespace esp

@@ -67,6 +67,14 @@ def forward(params, Q, Kb, Vb, pool, blocks, desc, pos, O, tiles, n_tiles, trees
     abi.check(rc, err)
 
 
+def time_next(start, stop):
+    """The next forward() records its attention kernel's begin and end into these two torch events
+    (created with enable_timing=True and recorded once before, so that their handles exist)."""
+    rc = abi.attn_lib().esp_attn_time_next(C.c_void_p(start.cuda_event), C.c_void_p(stop.cuda_event))
+    if rc != 0:
+        raise abi.EspError(f"esp_attn_time_next: error {rc}")
+
+
 def combine(params, O, jobs, n_jobs, n_parts, n_rows, workspace, stream=None):
     err = C.create_string_buffer(_ERRLEN)
     abi.check(abi.attn_lib().esp_attn_combine(C.byref(params), _ptr(O), _ptr(jobs), n_jobs, n_parts, n_rows, _ptr(workspace),

@@ -154,6 +154,16 @@ int esp_attn_forward(const esp_attn_params* p, const void* Q, const void* Kb, co
                      int32_t n_parts, int32_t n_rows, void* workspace, size_t workspace_bytes, void* stream, char* err,
                      size_t errlen);
 
+/* Measurement hook; no counterpart in the reference (its bench times command
+ * buffers, src/model/impl/bench.h:697-722). The next esp_attn_forward on this
+ * thread hands the two HIP events (hipEvent_t, created with timing enabled) to
+ * the launch of its attention kernel - the streaming or the tiled kernel, not
+ * the staging copy or the merge - which records the kernel's own begin and end
+ * into them: hipEventElapsedTime(start, stop) is then that kernel's duration,
+ * without marker packets between the kernels of the stream. The pair is used
+ * once. Both NULL clears a pending pair. */
+int esp_attn_time_next(void* start_event, void* stop_event);
+
 /* The split-K merge alone: attention_combine (40_:811-864, 80_:568-597) as its
  * own dispatch, for callers that passed n_jobs = 0 to esp_attn_forward (a
  * plan with n_parts > 0 then leaves its partial records in `workspace`). Same
