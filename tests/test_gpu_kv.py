@@ -58,3 +58,30 @@ def test_relayout_gather_save_copy_are_bit_exact(HD, Hkv, bt, dtype):
         device.kv_relayout(p, nat[l * region:], abi.ESP_LAYOUT_NATIVE, back[l * region:], abi.ESP_LAYOUT_REFERENCE, n_blocks)
     torch.cuda.synchronize()
     assert (to_host_u16(back) == ref).all()
+
+
+def test_time_next_brackets_the_attention_kernel_only():
+    """esp_attn_time_next: the two events take the attention kernel's own begin and end; the pair is used once."""
+    import torch
+    from espetero_amd import device, host, synth
+    from gpu_utils import dev_u16, native_pool
+    device.init(0)
+    c = synth.c1_single_decode()
+    p = c.params
+    tiles, jobs, n_parts = host.plan_tiles(c.trees, device.plan_hint(p)[1], 0, None,
+                                           host.options_mi355x(p.rows_per_tile, device.plan_hint(p)[0]))
+    dp = device.DevicePass(p, c.trees, tiles, jobs, n_parts, c.n_rows, c.blocks, None, None)
+    Q, Kb, Vb, pool = dev_u16(c.Q), dev_u16(c.Kb), dev_u16(c.Vb), native_pool(c)
+    O = torch.zeros_like(Q)
+    a, b = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+    a.record()
+    b.record()
+    torch.cuda.synchronize()
+    for _ in range(3):
+        dp.run(Q, Kb, Vb, pool, O)
+    device.time_next(a, b)
+    dp.run(Q, Kb, Vb, pool, O)
+    dp.run(Q, Kb, Vb, pool, O)      # no pending pair any more: must not touch the events
+    torch.cuda.synchronize()
+    us = a.elapsed_time(b) * 1e3
+    assert 1.0 < us < 200.0, us
