@@ -50,6 +50,14 @@ def make_params(H, Hkv, HD, dtype, bt, window=0, ring=0, scale=None, rows_per_ti
     return p
 
 
+def image_desc(M, a, b):
+    """Plain causal rows with one bidirectional span [a, b) (image tokens on a layer with bidi set):
+    rows inside the span also see the span's later rows (80_gemma.metal:284, img_end)."""
+    d = np.zeros((M, 4), np.int32)
+    d[a:b, 3] = b
+    return d
+
+
 def verify_desc(M, root=1):
     """Rows of one verify tree: `root` pending tokens, then one hosted draft chain
     (src/model/impl/forest.h:2400-2404, 2439-2442): chain rows see the whole root and
@@ -61,7 +69,7 @@ def verify_desc(M, root=1):
 
 
 def make_case(name, seed, H, Hkv, HD, dtype, bt, seqs, n_blocks=None, window=0, ring_layer=False, scale=None,
-              rows_per_tile=8, desc_fn=None, fill_unused=False, sigma=0.5):
+              rows_per_tile=8, desc_fn=None, fill_unused=False, sigma=0.5, bidi=0):
     """seqs: list of (P cached keys, M rows this pass). Block tables: slices of one
     seeded permutation of the pool's pages (tools/qsa_check.mm:120-123 shuffles its table
     for the same reason: contiguous pages would hide addressing mistakes)."""
@@ -75,7 +83,7 @@ def make_case(name, seed, H, Hkv, HD, dtype, bt, seqs, n_blocks=None, window=0, 
     elif n_blocks is None:
         n_blocks = max(need + 3, 4)
     assert ring_layer or need <= n_blocks
-    p = make_params(H, Hkv, HD, dtype, bt, window=window, ring=ring, scale=scale, rows_per_tile=rows_per_tile)
+    p = make_params(H, Hkv, HD, dtype, bt, window=window, ring=ring, scale=scale, rows_per_tile=rows_per_tile, bidi=bidi)
     blk = bt * kvw
     if fill_unused:  # unwritten pages hold NaN patterns: nothing outside [0, P) may reach a result
         pool = np.full(n_blocks * 2 * blk, 0x7E00 if dtype == abi.ESP_F16 else 0x7FC0, np.uint16)

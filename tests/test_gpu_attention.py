@@ -41,6 +41,7 @@ def _check(case, options=None, **kw):
     dict(seqs=((900, 1), (40, 1)), window=128, rows_per_tile=1),        # sliding window over block lists
     dict(seqs=((900, 1), (2000, 1)), window=256, ring_layer=True, rows_per_tile=1),  # sliding window over rings
     dict(seqs=((300, 5),), window=64, rows_per_tile=8, H=4, Hkv=2),     # window on multi-row tiles
+    dict(seqs=((200, 8),), rows_per_tile=8, H=4, Hkv=2, bidi=1, desc_fn=lambda M: synth.image_desc(M, 2, 6)),  # bidirectional span
 ])
 def test_stream_kernel_matches_checker(kw):
     _check(small_case(seed=31, fill_unused=not kw.get("ring_layer", False), **kw))
@@ -98,6 +99,9 @@ def test_gate():
     dict(seqs=((700, 150),), window=256, ring_layer=True, H=4, Hkv=2),  # sliding window, rings
     dict(seqs=((90, 40),), desc_fn=lambda M: synth.verify_desc(M, 30), H=4, Hkv=2),  # wide verify tree
     dict(seqs=((128, 128),), bt=64, H=4, Hkv=2),
+    dict(seqs=((100, 140),), H=4, Hkv=2, bidi=1, desc_fn=lambda M: synth.image_desc(M, 10, 90)),   # bidirectional span
+    dict(seqs=((1500, 130),), H=4, Hkv=2, HD=256),                      # long cached range: the mask-free loop, head_dim 256
+    dict(seqs=((1203, 128), (700, 40)), bt=64, H=4, Hkv=2, fill_unused=True),  # the same at the reference's block size, ragged end
 ])
 def test_tiled_kernel_matches_checker(kw):
     _check(small_case(seed=41, rows_per_tile=128, **kw))

@@ -67,6 +67,7 @@ CASES = [
     dict(seqs=((41, 7),), H=10, Hkv=2, dtype=abi.ESP_BF16),          # GQA 5, bf16
     dict(seqs=((33, 2),), H=4, Hkv=2, HD=256),                       # head_dim 256
     dict(seqs=((64, 9),), bt=64),                                    # the reference's default block size
+    dict(seqs=((20, 8),), H=4, Hkv=2, bidi=1, desc_fn=lambda M: synth.image_desc(M, 2, 6)),  # bidirectional span
 ]
 
 
@@ -124,6 +125,22 @@ def test_tree_mask_truth_table():
     for r in range(6):
         # P = 1/n is rounded to fp16 before P.V and the output again: both < 2^-10 relative.
         assert got[r] == pytest.approx(vals[want[r]].mean(), rel=2e-3)
+
+
+def test_bidirectional_span_truth_table():
+    """Rows 2..5 form a span with img_end = 6 on a layer with bidi set: inside the span every row sees
+    the whole span, outside it the rule stays causal (kernels/80_gemma.metal:284); without bidi the
+    same descriptors are plain causal."""
+    c = small_case(seed=4, H=2, Hkv=1, seqs=((1, 8),), bidi=1, desc_fn=lambda M: synth.image_desc(M, 2, 6))
+    want = np.zeros((8, 9), bool)
+    want[:, 0] = True                                   # the cached key
+    for r in range(8):
+        want[r, 1:r + 2] = True                         # causal over the batch keys
+    want[2:6, 1 + 2:1 + 6] = True                       # the span sees itself whole
+    assert (ob.visible_mask(c.params, c.trees[0], c.desc, c.pos) == want).all()
+    c.params.bidi = 0
+    causal = np.tril(np.ones((8, 8), bool))
+    assert (ob.visible_mask(c.params, c.trees[0], c.desc, c.pos)[:, 1:] == causal).all()
 
 
 # ---------------------------------------------------------------- closed forms
