@@ -108,11 +108,62 @@ class Workload:
         dp.run(self.Q, self.Kb, self.Vb, self.pool, self.O)  # attention + split-K merge, one call
 
 
+class PrepWorkload:
+    """esp_attn_prep over one chunk of rows: fp32 fused projection in, Q / K / V in the storage type out,
+    the rows' K / V appended to a paged pool by the same kernel."""
+
+    kernel = "attn_prep_kernel"
+
+    def __init__(self, name, kind, H, Hkv, HD, dtype, n_rows, bt=16, seed=7):
+        import torch
+        from espetero_amd import abi, device, synth
+        self.torch, self.device = torch, device
+        self.name, self.bound, self.dtype = name, "hbm", dtype
+        self.H, self.Hkv, self.HD, self.bt, self.window = H, Hkv, HD, bt, 0
+        self.seqs, self.n_rows, self.tiles, self.n_parts = [(0, n_rows)], n_rows, [], 0
+        self.kind = kind
+        p, a = synth.make_prep(kind, H, Hkv, HD, dtype, n_rows, seed=seed, bt=bt)
+        self.params, self.host = p, a
+        tdt = torch.float16 if dtype == abi.ESP_F16 else torch.bfloat16
+        dev = lambda x: None if x is None else torch.from_numpy(np.ascontiguousarray(x)).cuda()  # noqa: E731
+        # rotation sets of X so that a step never finds its input in a cache
+        self.n_sets = 4
+        g = torch.Generator(device="cuda")
+        g.manual_seed(seed)
+        self.X = [dev(a["X"])] + [torch.randn(n_rows, p.x_ld, generator=g, device="cuda") * 1.5 for _ in range(self.n_sets - 1)]
+        self.qn_w, self.kn_w, self.pos = dev(a["qn_w"]), dev(a["kn_w"]), dev(a["pos"])
+        self.inv_freq, self.rope_sel = dev(a["inv_freq"]), dev(a["rope_sel"])
+        self.Q = torch.zeros(n_rows, p.q_ld, dtype=tdt, device="cuda")
+        self.Kb = torch.zeros(n_rows, p.kv_ld, dtype=tdt, device="cuda")
+        self.Vb = torch.zeros_like(self.Kb)
+        n_blocks = (n_rows + bt - 1) // bt
+        self.pool_pages = n_blocks
+        self.pool = torch.zeros(n_blocks * 2 * bt * p.kv_ld, dtype=tdt, device="cuda")
+        perm = np.random.default_rng(seed).permutation(n_blocks).astype(np.int32)
+        table = np.full((n_rows, 4), -1, np.int32)
+        table[:, 0] = perm[np.arange(n_rows) // bt]
+        table[:, 1] = np.arange(n_rows) % bt
+        self.table_host, self.table = table, dev(table)
+        elems = (H + 2 * Hkv) * HD
+        self.alg_bytes = n_rows * (elems * 4 + elems * 2 + 2 * Hkv * HD * 2 + 16 + 16)  # X, Q K V, pool entries, pos, table
+        self.alg_flops = 0
+
+    def step(self, i, ev=None):
+        if ev:
+            self.device.time_next(ev[0], ev[1])
+        self.device.attn_prep(self.params, self.X[i % self.n_sets], self.qn_w, self.kn_w, self.pos, self.inv_freq, self.rope_sel,
+                              self.Q, self.Kb, self.Vb, self.table, self.pool, self.n_rows)
+
+
 def make_workload(name, workgroups=None, contiguous=False, page=16):
     from espetero_amd import abi, synth
     from functools import partial
     F16, BF16 = abi.ESP_F16, abi.ESP_BF16
     Workload_ = partial(Workload, workgroups=workgroups, contiguous=contiguous)
+    if name == "c3_attn_prep":   # the rows of one C3 prefill chunk, Qwen3-Omni arrangement (82_qwen3_omni.metal:30-88)
+        return PrepWorkload(name, "omni", 40, 8, 128, BF16, 2048, bt=page)
+    if name == "c4_attn_prep":   # the rows of one C4 prefill pass, Qwen3.5 arrangement (40_attention.metal:9-102)
+        return PrepWorkload(name, "qwen35", 16, 8, 256, F16, 8 * 1024, bt=page)
     if name == "c1_single_decode":
         return Workload_(name, 32, 4, 128, F16, page, [(1024, 1)], pool_pages=(64 * 16) * 16 // page, seed=1)
     if name == "c2_batched_decode":
@@ -150,7 +201,7 @@ def measured_traffic(workload):
 
 WORKLOADS = ["c1_single_decode", "c2_batched_decode", "c3_prefill_p0", "c3_prefill_p2048", "c3_prefill_p4096",
              "c3_prefill_p6144", "c4_decode_sliding", "c4_decode_global", "c4_prefill_sliding", "c4_prefill_global",
-             "c5_verify"]
+             "c5_verify", "c3_attn_prep", "c4_attn_prep"]
 
 
 def cpu_baseline(w, budget_s=20.0):
@@ -250,6 +301,22 @@ def cpu_baseline(w, budget_s=20.0):
             "host_cpus": os.cpu_count(), "max_abs_err_vs_gpu": max_err}
 
 
+def prep_cpu_baseline(w):
+    """The CPU checker's attn_prep on the workload's own rows (rotation set 0), single-threaded."""
+    from oracle import binding as ob
+    a, p = w.host, w.params
+    rows = min(w.n_rows, 2048)
+    t0 = time.perf_counter()
+    Q, K, V = ob.attn_prep(p, a["X"][:rows], a["qn_w"], a["kn_w"], a["pos"][:rows], a["inv_freq"], a["rope_sel"], rows)
+    dt = time.perf_counter() - t0
+    bits = lambda t: t.view(w.torch.int16).cpu().numpy().view(np.uint16)  # noqa: E731
+    f = lambda b: ob.to_f32(b, p.dtype).astype(np.float64)  # noqa: E731
+    err = max(float(np.abs(f(bits(g)[:rows]) - f(c)).max()) for g, c in ((w.Q, Q), (w.Kb, K), (w.Vb, V)))
+    return {"value": round(w.alg_bytes * rows / w.n_rows / dt / 1e9, 6), "unit": "GB/s", "cores": 1, "kind": "port",
+            "sample": f"{rows} of {w.n_rows} rows, {dt:.2f} s single-threaded", "host_cpus": os.cpu_count(),
+            "max_abs_err_vs_gpu": err}
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
@@ -301,7 +368,7 @@ def main():
     kern_min_ms = float(np.min([a.elapsed_time(b) for a, b in evs]))
 
     if w.bound == "hbm":
-        metric, unit = "decode-attn HBM GB/s", "GB/s"
+        metric, unit = ("attn-prep HBM GB/s" if isinstance(w, PrepWorkload) else "decode-attn HBM GB/s"), "GB/s"
         value = w.alg_bytes / wall / 1e9
         achieved, peak = w.alg_bytes / (kern_ms * 1e-3) / 1e9, HBM_PEAK_GBS
     else:
@@ -318,15 +385,16 @@ def main():
                    "pool_pages": w.pool_pages},
         "roofline": {"bound": w.bound, "achieved": round(achieved, 3), "peak": peak, "unit": unit,
                      "frac": round(achieved / peak, 4), "traffic": measured_traffic(w.name),
-                     "kernel": "attn_stream_kernel" if w.bound == "hbm" and w.params.rows_per_tile * (w.H // w.Hkv) <= 32
-                     else "attn_tiled_kernel",
+                     "kernel": getattr(w, "kernel", None) or (
+                         "attn_stream_kernel" if w.bound == "hbm" and w.params.rows_per_tile * (w.H // w.Hkv) <= 32
+                         else "attn_tiled_kernel"),
                      "kernel_us_avg": round(kern_ms * 1e3, 3), "kernel_us_min": round(kern_min_ms * 1e3, 3),
                      "alg_bytes": int(w.alg_bytes), "alg_flops": int(w.alg_flops)},
     }
     if not args.no_cpu:
         w.step(0)   # leave rotation set 0's output in O: the CPU sample is checked against it
         torch.cuda.synchronize()
-        out["cpu_baseline"] = cpu_baseline(w)
+        out["cpu_baseline"] = prep_cpu_baseline(w) if isinstance(w, PrepWorkload) else cpu_baseline(w)
     print(json.dumps(out), flush=True)
 
 

@@ -43,6 +43,14 @@ class AttnParams(C.Structure):
                 ("gate_off", C.c_int32), ("reserved", C.c_int32)]
 
 
+class PrepParams(C.Structure):
+    _fields_ = [("H", C.c_int32), ("Hkv", C.c_int32), ("head_dim", C.c_int32), ("dtype", C.c_int32),
+                ("x_ld", C.c_int32), ("q_off", C.c_int32), ("q_hs", C.c_int32), ("k_off", C.c_int32),
+                ("v_off", C.c_int32), ("q_ld", C.c_int32), ("kv_ld", C.c_int32), ("rope_dims", C.c_int32),
+                ("v_norm", C.c_int32), ("bt", C.c_int32), ("eps", C.c_float), ("q_scale", C.c_float),
+                ("kv_base", C.c_uint64)]
+
+
 TREE_DT = np.dtype([("base", "<i4"), ("P", "<i4"), ("table", "<i4"), ("M", "<i4")])
 TILE_DT = np.dtype([("tree", "<i4"), ("r0", "<i4"), ("k0", "<i4"), ("k1", "<i4"),
                     ("part", "<i4"), ("last", "<i4"), ("b0", "<i4"), ("pad", "<i4")])
@@ -54,6 +62,7 @@ assert C.sizeof(Tile) == TILE_DT.itemsize == 32
 assert C.sizeof(Combine) == COMBINE_DT.itemsize == 16
 assert C.sizeof(KVSave) == KVSAVE_DT.itemsize == 16
 assert C.sizeof(AttnParams) == 80
+assert C.sizeof(PrepParams) == 72
 
 # name -> (restype, argtypes); every symbol the header declares.
 _P = C.POINTER(AttnParams)
@@ -72,6 +81,7 @@ ATTN_SYMBOLS = {
     "esp_kv_copy_blocks": (C.c_int, (_P, _V, _V, C.c_int32, C.c_int32, C.c_uint64, _V) + _ERR),
     "esp_kv_gather": (C.c_int, (_P, _V, _V, C.c_int32, _V, _V, _V) + _ERR),
     "esp_kv_relayout": (C.c_int, (_P, _V, C.c_int32, _V, C.c_int32, C.c_int32, _V) + _ERR),
+    "esp_attn_prep": (C.c_int, (C.POINTER(PrepParams), _V, _V, _V, _V, _V, _V, _V, _V, _V, _V, _V, C.c_int32, _V) + _ERR),
 }
 
 

@@ -19,6 +19,7 @@ hipError_t launch_kv_gather(const esp_attn_params* p, const void* pool, const in
 hipError_t launch_kv_relayout(const esp_attn_params* p, const void* src, void* dst, int to_native, int n_blocks,
                               hipStream_t st);
 hipError_t launch_vt_stage(const esp_attn_params* p, const void* Vb, void* vt, int n_rows, hipStream_t st);
+hipError_t launch_attn_prep(const PrepArgs& a, int n_rows, hipStream_t st);
 int stream_workgroups_per_cu(int HD, int NC);
 int tiled_workgroups_per_cu(int HD);
 int tiled_max_rows(int HD);
@@ -276,6 +277,41 @@ int esp_kv_relayout(const esp_attn_params* p, const void* src_pool, int32_t src_
   if (!src_pool || !dst_pool) return fail(err, errlen, ESP_EINVAL, "NULL argument");
   hipError_t e = esp::launch_kv_relayout(p, src_pool, dst_pool, dst_layout == ESP_LAYOUT_NATIVE, n_blocks, static_cast<hipStream_t>(stream));
   return e == hipSuccess ? ESP_OK : hip_fail(err, errlen, "kv_relayout launch", e);
+}
+
+int esp_attn_prep(const esp_prep_params* p, const float* X, const float* qn_w, const float* kn_w, const int32_t* pos,
+                  const float* inv_freq, const int32_t* rope_sel, void* Q, void* Kb, void* Vb, const int32_t* row_table,
+                  void* kv_pool, int32_t n_rows, void* stream, char* err, size_t errlen) {
+  if (!p) return fail(err, errlen, ESP_EINVAL, "params is NULL");
+  if (p->H <= 0 || p->Hkv <= 0) return fail(err, errlen, ESP_EINVAL, "H=%d Hkv=%d", p->H, p->Hkv);
+  if (p->head_dim != 128 && p->head_dim != 256) return fail(err, errlen, ESP_EUNSUPPORTED, "head_dim %d (128 or 256)", p->head_dim);
+  if (p->dtype != ESP_F16 && p->dtype != ESP_BF16) return fail(err, errlen, ESP_EINVAL, "dtype %d", p->dtype);
+  const int HD = p->head_dim;
+  if (p->x_ld % 4 || p->q_off % 4 || p->q_hs % 4 || p->k_off % 4 || p->v_off % 4 || p->q_off < 0 || p->k_off < 0 || p->v_off < 0)
+    return fail(err, errlen, ESP_EINVAL, "x_ld, q_off, q_hs, k_off, v_off must be non-negative multiples of 4 floats");
+  if (p->q_hs < HD) return fail(err, errlen, ESP_EINVAL, "q_hs %d < head_dim", p->q_hs);
+  if (p->x_ld < p->q_off + (p->H - 1) * p->q_hs + HD || p->x_ld < p->k_off + p->Hkv * HD || p->x_ld < p->v_off + p->Hkv * HD)
+    return fail(err, errlen, ESP_EINVAL, "x_ld %d does not hold the q / k / v columns", p->x_ld);
+  if (p->q_ld < p->H * HD || p->q_ld % 4 || p->kv_ld < p->Hkv * HD || p->kv_ld % 4)
+    return fail(err, errlen, ESP_EINVAL, "q_ld %d / kv_ld %d", p->q_ld, p->kv_ld);
+  const int rd = p->rope_dims;
+  if (rd < 0 || rd > HD || (rd != 0 && (rd < 8 || (rd & (rd - 1)))))
+    return fail(err, errlen, ESP_EINVAL, "rope_dims %d: 0 or a power of two in [8, head_dim]", rd);
+  if (n_rows < 0) return fail(err, errlen, ESP_EINVAL, "negative count");
+  if (n_rows == 0) return ESP_OK;
+  if (!X || !qn_w || !kn_w || !Q || !Kb || !Vb) return fail(err, errlen, ESP_EINVAL, "X, qn_w, kn_w, Q, Kb, Vb must not be NULL");
+  if (rd > 0 && (!pos || !inv_freq)) return fail(err, errlen, ESP_EINVAL, "pos and inv_freq must not be NULL when dims rotate");
+  if (row_table) {
+    if (!kv_pool) return fail(err, errlen, ESP_EINVAL, "row_table without kv_pool");
+    if (p->bt <= 0 || p->bt % 16) return fail(err, errlen, ESP_EINVAL, "bt %d: tokens per block must be a positive multiple of 16", p->bt);
+    if (p->kv_base % 8) return fail(err, errlen, ESP_EINVAL, "kv_base must be a multiple of 8 elements");
+  }
+  esp::PrepArgs a{X, qn_w, kn_w, reinterpret_cast<const int4*>(pos), inv_freq, rope_sel, static_cast<uint16_t*>(Q),
+                  static_cast<uint16_t*>(Kb), static_cast<uint16_t*>(Vb), reinterpret_cast<const int4*>(row_table),
+                  static_cast<uint16_t*>(kv_pool), *p};
+  const hipError_t e = esp::launch_attn_prep(a, n_rows, static_cast<hipStream_t>(stream));
+  if (e != hipSuccess) return hip_fail(err, errlen, "attn_prep launch", e);
+  return ESP_OK;
 }
 
 }  // extern "C"

@@ -1,0 +1,169 @@
+// attn_prep: what runs between the fused in-projection and the attention of a
+// layer. Per (row, head) of the fp32 projection: RMSNorm over the head with a
+// learned weight (queries and keys), rotary embedding of the leading
+// `rope_dims` dims in the half-split pairing (d, d + rope_dims / 2), cast to the
+// storage type; values are cast (or normalised without weight); the rows' K / V
+// also go straight into their pool entries, so no kv_save dispatch follows.
+//
+// One kernel for the reference's three: attn_prep (kernels/40_attention.metal:9-102:
+// head_dim 256, 64 rotating dims, the gate beside each query head, the folded
+// append), g4_attn_prep<HD> (kernels/80_gemma.metal:52-108: all dims rotate,
+// values normalised) and q3m_attn_prep<HD> (kernels/82_qwen3_omni.metal:30-88:
+// per-frequency position component, query scale).
+//
+// Mapping to gfx950: HBM bound (fp32 in, 16-bit out). One workgroup = 8 consecutive
+// rows x 1024 columns (8 heads of 128 dims, 4 of 256); a lane owns 4 consecutive dims (one 16-byte load, one 8-byte store), so a
+// head is 32 or 64 lanes and the norm's sum and the rotation's partner are lane
+// exchanges inside a wavefront. A thread works on the same (head, dims) of all 8
+// rows at once: 8 independent loads in flight. The rows' cos / sin tables
+// (rope_dims / 2 entries each) are computed once per workgroup into LDS and shared
+// by its heads: the reference computes them once per (row, head).
+// The folded append writes K rows as they are. V lies transposed in the pool
+// (tokens contiguous per dim): when the 8 rows go to 8 consecutive, 8-aligned
+// positions of one block - every full group of a prefill chunk - their V is
+// staged in LDS and leaves as one 16-byte store per (head, dim); any other
+// arrangement (decode rows of different sequences, a row saved into two slots)
+// takes element stores.
+#include "common.hpp"
+
+namespace esp {
+
+
+constexpr int kPrepRows = 8;
+
+template <int DT, int HD>
+__global__ __launch_bounds__(256) void attn_prep_kernel(const PrepArgs a, int n_rows) {
+  constexpr int R = kPrepRows;
+  constexpr int LPH = HD / 4;     // lanes per head
+  constexpr int HPP = 256 / LPH;  // heads of the workgroup
+  __shared__ float2 cs[R][128];   // (cos, sin) per row and frequency
+  __shared__ int run_ok;
+  __shared__ __attribute__((aligned(16))) uint16_t vstage[R][HPP * HD];  // the workgroup's V heads, for the transposed append
+  const esp_prep_params& p = a.p;
+  const int row0 = blockIdx.x * R;
+  const int rows = min(R, n_rows - row0);
+  const int tid = threadIdx.x;
+  const int half = p.rope_dims / 2;
+  for (int i = tid; i < rows * half; i += 256) {
+    const int r = i / half, f = i % half;
+    const int4 pr = a.pos[row0 + r];
+    const int sel = a.rope_sel ? a.rope_sel[f] : 0;
+    const float position = float(sel == 0 ? pr.x : (sel == 1 ? pr.y : pr.z));
+    float sn, c;
+    sincosf(position * a.inv_freq[f], &sn, &c);
+    cs[r][f] = make_float2(c, sn);
+  }
+  // Do the 8 rows go to positions ps0 .. ps0 + 7 (ps0 a multiple of 8) of one block, nowhere else?
+  int4 ent[R];
+#pragma unroll
+  for (int r = 0; r < R; ++r) ent[r] = (a.row_table && r < rows) ? a.row_table[row0 + r] : make_int4(-1, -1, -1, -1);
+  bool run = rows == R && ent[0].x >= 0 && (ent[0].y & (R - 1)) == 0;
+#pragma unroll
+  for (int r = 0; r < R; ++r) run = run && ent[r].x == ent[0].x && ent[r].y == ent[0].y + r && ent[r].z < 0;
+  if (tid == 0) run_ok = run;
+  __syncthreads();
+  run = run_ok != 0;  // the same value everywhere; through LDS so that the compiler treats it as uniform
+
+  const int li = tid % LPH, d0 = 4 * li;
+  const int n_slots = p.H + 2 * p.Hkv;
+  const int slot0 = blockIdx.y * HPP;  // the workgroup's first head: queries, then keys, then values
+  for (int slot = slot0 + tid / LPH; slot < n_slots; slot += n_slots) {  // at most one head per thread
+    const int kind = slot < p.H ? 0 : (slot < p.H + p.Hkv ? 1 : 2);  // q, k, v
+    const int h = kind == 0 ? slot : (kind == 1 ? slot - p.H : slot - p.H - p.Hkv);
+    const size_t col = size_t(kind == 0 ? p.q_off + h * p.q_hs : (kind == 1 ? p.k_off : p.v_off) + h * HD) + d0;
+    f32x4 xv[R];
+#pragma unroll
+    for (int r = 0; r < R; ++r)
+      xv[r] = r < rows ? *reinterpret_cast<const f32x4*>(a.X + size_t(row0 + r) * p.x_ld + col) : f32x4{0, 0, 0, 0};
+    f32x4 w = {1, 1, 1, 1};
+    if (kind != 2) w = *reinterpret_cast<const f32x4*>((kind == 0 ? a.qn_w : a.kn_w) + d0);
+#pragma unroll
+    for (int r = 0; r < R; ++r) {
+      if (r >= rows) break;
+      const size_t row = size_t(row0 + r);
+      float x[4] = {xv[r][0], xv[r][1], xv[r][2], xv[r][3]};
+      if (kind != 2 || p.v_norm) {
+        float ss = x[0] * x[0] + x[1] * x[1] + x[2] * x[2] + x[3] * x[3];
+#pragma unroll
+        for (int o = LPH / 2; o >= 1; o >>= 1) ss += __shfl_xor(ss, o);
+        const float inv = rsqrtf(ss / float(HD) + p.eps);
+#pragma unroll
+        for (int i = 0; i < 4; ++i) x[i] = kind == 2 ? x[i] * inv : x[i] * inv * w[i];
+      }
+      if (kind != 2 && half > 0) {
+        // The partner of dim d < half is d + half: half / 4 lanes away. Every lane of the head takes
+        // part in the exchange; only the rotating dims use it.
+        const bool lower = d0 < half;
+#pragma unroll
+        for (int i = 0; i < 4; ++i) {
+          const float partner = __shfl_xor(x[i], half / 4);
+          if (d0 < p.rope_dims) {
+            const float2 t = cs[r][(lower ? d0 : d0 - half) + i];
+            x[i] = lower ? x[i] * t.x - partner * t.y : x[i] * t.x + partner * t.y;
+          }
+        }
+      }
+      if (kind == 0) {
+#pragma unroll
+        for (int i = 0; i < 4; ++i) x[i] *= p.q_scale;
+      }
+      const u32x2 out = {pack2<DT>(x[0], x[1]), pack2<DT>(x[2], x[3])};
+      if (kind == 0) {
+        *reinterpret_cast<u32x2*>(a.Q + row * size_t(p.q_ld) + size_t(h) * HD + d0) = out;
+        continue;
+      }
+      *reinterpret_cast<u32x2*>((kind == 1 ? a.Kb : a.Vb) + row * size_t(p.kv_ld) + size_t(h) * HD + d0) = out;
+      // The folded append: the same bits into the row's pool entries (a row saved into two slots has two).
+      if (kind == 2 && run) {
+        *reinterpret_cast<u32x2*>(&vstage[r][(slot - slot0) * HD + d0]) = out;
+        continue;
+      }
+#pragma unroll
+      for (int e = 0; e < 2; ++e) {
+        const int b = e ? ent[r].z : ent[r].x, ps = e ? ent[r].w : ent[r].y;
+        if (b < 0) continue;
+        uint16_t* hb = a.pool + p.kv_base + (size_t(b) * p.Hkv + h) * size_t(2 * p.bt * HD);
+        if (kind == 1) {
+          *reinterpret_cast<u32x2*>(hb + size_t(ps) * HD + d0) = out;
+        } else {
+          uint16_t* vt = hb + size_t(p.bt) * HD + size_t(d0) * p.bt + ps;
+          vt[0] = uint16_t(out[0] & 0xffffu);
+          vt[p.bt] = uint16_t(out[0] >> 16);
+          vt[2 * p.bt] = uint16_t(out[1] & 0xffffu);
+          vt[3 * p.bt] = uint16_t(out[1] >> 16);
+        }
+      }
+    }
+  }
+  if (!run) return;
+  __syncthreads();
+  // 8 tokens of one (head, dim): 16 contiguous bytes of the transposed V plane.
+  for (int i = tid; i < HPP * HD; i += 256) {
+    const int slot = slot0 + i / HD, d = i % HD;
+    if (slot < p.H + p.Hkv || slot >= n_slots) continue;  // not a value head
+    const int h = slot - p.H - p.Hkv;
+    uint16_t* hb = a.pool + p.kv_base + (size_t(ent[0].x) * p.Hkv + h) * size_t(2 * p.bt * HD);
+    uint16_t* dst = hb + size_t(p.bt) * HD + size_t(d) * p.bt + ent[0].y;
+#pragma unroll
+    for (int g = 0; g < R / 8; ++g) {
+      u32x4 v;
+#pragma unroll
+      for (int e = 0; e < 4; ++e) v[e] = uint32_t(vstage[8 * g + 2 * e][i]) | (uint32_t(vstage[8 * g + 2 * e + 1][i]) << 16);
+      *reinterpret_cast<u32x4*>(dst + 8 * g) = v;
+    }
+  }
+}
+
+hipError_t launch_attn_prep(const PrepArgs& a, int n_rows, hipStream_t st) {
+  const int dt = a.p.dtype, HD = a.p.head_dim;
+  const int hpp = 256 / (HD / 4), n_slots = a.p.H + 2 * a.p.Hkv;
+  const dim3 grid((n_rows + kPrepRows - 1) / kPrepRows, (n_slots + hpp - 1) / hpp), block(256);
+  if (dt == ESP_F16 && HD == 128) launch_timed(attn_prep_kernel<ESP_F16, 128>, grid, block, 0, st, a, n_rows);
+  else if (dt == ESP_F16 && HD == 256) launch_timed(attn_prep_kernel<ESP_F16, 256>, grid, block, 0, st, a, n_rows);
+  else if (dt == ESP_BF16 && HD == 128) launch_timed(attn_prep_kernel<ESP_BF16, 128>, grid, block, 0, st, a, n_rows);
+  else if (dt == ESP_BF16 && HD == 256) launch_timed(attn_prep_kernel<ESP_BF16, 256>, grid, block, 0, st, a, n_rows);
+  else return hipErrorInvalidValue;
+  return hipGetLastError();
+}
+
+}  // namespace esp

@@ -115,6 +115,22 @@ __device__ __forceinline__ int block_of(const KArgs& a, int table, int j) {
   return a.ring ? table + bi % a.ring : a.blocks[table + bi];
 }
 
+// Everything the prep kernel reads (esp_attn_prep).
+struct PrepArgs {
+  const float* X;
+  const float* qn_w;
+  const float* kn_w;
+  const int4* pos;
+  const float* inv_freq;
+  const int32_t* rope_sel;
+  uint16_t* Q;
+  uint16_t* Kb;
+  uint16_t* Vb;
+  const int4* row_table;
+  uint16_t* pool;
+  esp_prep_params p;
+};
+
 // Events the next attention kernel launch records its own begin and end into (esp_attn_time_next);
 // both null otherwise. One caller thread drives the library, so a plain pair is enough.
 struct TimeNext {

@@ -105,6 +105,14 @@ def kv_relayout(params, src, src_layout, dst, dst_layout, n_blocks, stream=None)
                                              _stream(stream), err, _ERRLEN), err)
 
 
+def attn_prep(params, X, qn_w, kn_w, pos, inv_freq, rope_sel, Q, Kb, Vb, row_table, pool, n_rows, stream=None):
+    """All device tensors; rope_sel, row_table and pool may be None."""
+    err = C.create_string_buffer(_ERRLEN)
+    abi.check(abi.attn_lib().esp_attn_prep(C.byref(params), _ptr(X), _ptr(qn_w), _ptr(kn_w), _ptr(pos), _ptr(inv_freq),
+                                           _ptr(rope_sel), _ptr(Q), _ptr(Kb), _ptr(Vb), _ptr(row_table), _ptr(pool), n_rows,
+                                           _stream(stream), err, _ERRLEN), err)
+
+
 class DevicePass:
     """One planned pass resident on the device: uploads the records once and
     replays esp_attn_forward (what a decode chain does between host syncs)."""

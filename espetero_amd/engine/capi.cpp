@@ -167,6 +167,16 @@ int esp_engine_pass_cow(const esp_engine* e, int32_t* out) {
   if (!p.cow.empty()) memcpy(out, p.cow.data(), p.cow.size() * 8);
   return int(p.cow.size());
 }
+int esp_kv_row_table(const esp_kvsave* saves, int32_t n_saves, int32_t rows, int32_t* out, char* err, size_t errlen) {
+  try {
+    const std::vector<int32_t> t = espetero::engine::row_table(saves, n_saves, rows);
+    memcpy(out, t.data(), size_t(std::max(rows, 1)) * 16);
+    return 0;
+  } catch (const std::exception& ex) {
+    if (err && errlen) snprintf(err, errlen, "%s", ex.what());
+    return 1;
+  }
+}
 int esp_engine_pass_commit(esp_engine* e) { return guarded([&] { e->e.pass_commit(); }); }
 int esp_engine_pass_abort(esp_engine* e) { return guarded([&] { e->e.pass_abort(); }); }
 

@@ -75,6 +75,23 @@ struct TreePlan {
   std::vector<int> dst_blocks, work_blocks;
 };
 
+// Per pass row the pool entries its K / V go to, (block, position, block2, position2), -1 none: what
+// esp_attn_prep's folded append reads instead of a kv_save dispatch (kv_row_table,
+// src/model/impl/forest.h:1737-1749). A row saved into more than two slots is refused, as there.
+inline std::vector<int32_t> row_table(const esp_kvsave* saves, int n_saves, int rows) {
+  std::vector<int32_t> t(size_t(std::max(rows, 1)) * 4, -1);
+  for (int i = 0; i < n_saves; ++i) {
+    const esp_kvsave& r = saves[i];
+    if (r.src_row < 0 || r.src_row >= rows) throw EngineError("row_table: a save names a row outside the pass");
+    int32_t* e = t.data() + size_t(r.src_row) * 4;
+    const int j = e[0] < 0 ? 0 : 2;
+    if (j == 2 && e[2] >= 0) throw EngineError("row_table: a row saved into more than two slots");
+    e[j] = r.block;
+    e[j + 1] = r.pos;
+  }
+  return t;
+}
+
 class KvEngine {
  public:
   KvEngine(int n_blocks, int bt, int n_slots, int max_ctx) : max_ctx_(max_ctx) {

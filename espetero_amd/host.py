@@ -49,6 +49,7 @@ ENGINE_SYMBOLS = {
     "esp_engine_pass_table": (C.c_int, (_V, _V)),
     "esp_engine_pass_saves": (C.c_int, (_V, _V)),
     "esp_engine_pass_cow": (C.c_int, (_V, _V)),
+    "esp_kv_row_table": (C.c_int, (_V, C.c_int32, C.c_int32, _V, C.c_char_p, C.c_size_t)),
     "esp_engine_pass_commit": (C.c_int, (_V,)),
     "esp_engine_pass_abort": (C.c_int, (_V,)),
 }
@@ -100,6 +101,17 @@ def plan_tiles(trees, groups, window, pos, options):
                             C.byref(nj), C.byref(npart), err, 256)
     abi.check(rc, err)
     return tiles, jobs, npart.value
+
+
+def row_table(saves, rows):
+    """KVSAVE_DT records -> int32 [rows][4] = (block, position, block2, position2), -1 none."""
+    saves = np.ascontiguousarray(saves, dtype=abi.KVSAVE_DT)
+    out = np.zeros((max(rows, 1), 4), np.int32)
+    err = C.create_string_buffer(256)
+    rc = engine_lib().esp_kv_row_table(saves.ctypes.data if len(saves) else None, len(saves), rows, out.ctypes.data, err, 256)
+    if rc != 0:
+        raise abi.EspError(err.value.decode(errors="replace"))
+    return out[:rows]
 
 
 def make_spec(parent=-1, save=-1, work=-1, root_len=0, save_len=0, leaves=(), commit_chain=0, noncausal=0):

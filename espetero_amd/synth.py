@@ -134,6 +134,42 @@ def make_case(name, seed, H, Hkv, HD, dtype, bt, seqs, n_blocks=None, window=0, 
                 dict(seqs=list(seqs), seed=seed))
 
 
+def make_prep(kind, H, Hkv, HD, dtype, n_rows, seed=0, bt=16, max_pos=40000):
+    """Inputs of one esp_attn_prep call in the arrangement of one of the reference's three prep
+    kernels: "qwen35" (kernels/40_attention.metal:9-102: a gate beside each query head, 64 rotating
+    dims, position component per frequency), "gemma" (80_gemma.metal:52-108: all dims rotate by pos.x,
+    values normalised), "omni" (82_qwen3_omni.metal:30-88: all dims rotate, component per frequency,
+    queries scaled). Returns (params, dict of numpy arrays)."""
+    rng = np.random.default_rng(seed)
+    p = abi.PrepParams()
+    p.H, p.Hkv, p.head_dim, p.dtype = H, Hkv, HD, dtype
+    p.q_hs = 2 * HD if kind == "qwen35" else HD
+    p.q_off = 0
+    p.k_off = H * p.q_hs
+    p.v_off = p.k_off + Hkv * HD
+    p.x_ld = p.v_off + Hkv * HD
+    p.q_ld, p.kv_ld = H * HD, Hkv * HD
+    p.rope_dims = 64 if kind == "qwen35" else HD
+    p.v_norm = 1 if kind == "gemma" else 0
+    p.bt, p.eps = bt, 1e-6
+    p.q_scale = float(1.0 / np.sqrt(HD)) if kind == "omni" else 1.0
+    p.kv_base = 0
+    half = p.rope_dims // 2
+    a = dict(
+        X=(rng.standard_normal((n_rows, p.x_ld), dtype=np.float32) * 1.5),
+        qn_w=(1.0 + 0.25 * rng.standard_normal(HD, dtype=np.float32)),
+        kn_w=(1.0 + 0.25 * rng.standard_normal(HD, dtype=np.float32)),
+        inv_freq=(1.0e6 ** (-np.arange(half, dtype=np.float64) / half)).astype(np.float32),
+        rope_sel=None if kind == "gemma" else (np.arange(half) % 3).astype(np.int32),
+        pos=np.zeros((n_rows, 4), np.int32),
+    )
+    t = rng.integers(0, max_pos, n_rows)
+    a["pos"][:, 0] = t
+    a["pos"][:, 1] = t if kind == "gemma" else rng.integers(0, 64, n_rows)
+    a["pos"][:, 2] = t if kind == "gemma" else rng.integers(0, 64, n_rows)
+    return p, a
+
+
 # ---- the benchmark shapes (BASELINE configs), with a shrink factor for tests ----
 def c1_single_decode(ctx=1024):
     return make_case("c1_single_decode", 1, 32, 4, 128, abi.ESP_F16, 16, [(ctx, 1)], rows_per_tile=1)

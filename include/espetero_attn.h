@@ -155,10 +155,11 @@ int esp_attn_forward(const esp_attn_params* p, const void* Q, const void* Kb, co
                      size_t errlen);
 
 /* Measurement hook; no counterpart in the reference (its bench times command
- * buffers, src/model/impl/bench.h:697-722). The next esp_attn_forward on this
- * thread hands the two HIP events (hipEvent_t, created with timing enabled) to
- * the launch of its attention kernel - the streaming or the tiled kernel, not
- * the staging copy or the merge - which records the kernel's own begin and end
+ * buffers, src/model/impl/bench.h:697-722). The next esp_attn_forward (or
+ * esp_attn_prep) hands the two HIP events (hipEvent_t, created with timing
+ * enabled) to the launch of its main kernel - the streaming or the tiled
+ * attention kernel, not the staging copy or the merge; the prep kernel - which
+ * records the kernel's own begin and end
  * into them: hipEventElapsedTime(start, stop) is then that kernel's duration,
  * without marker packets between the kernels of the stream. The pair is used
  * once. Both NULL clears a pending pair. */
@@ -193,6 +194,47 @@ int esp_kv_gather(const esp_attn_params* p, const void* kv_pool, const int32_t* 
  * src_layout / dst_layout: ESP_LAYOUT_*. Bit copy. */
 int esp_kv_relayout(const esp_attn_params* p, const void* src_pool, int32_t src_layout, void* dst_pool, int32_t dst_layout,
                     int32_t n_blocks, void* stream, char* err, size_t errlen);
+
+/* ---- attn_prep: the step before the attention of a layer ----------------------
+ * One entry point for the reference's three prep kernels:
+ *   attn_prep        kernels/40_attention.metal:9-102   (AttnPrepParams; binding forest.h:2951-2977)
+ *   g4_attn_prep<HD> kernels/80_gemma.metal:52-108      (G4PrepParams;   binding gemma.h:455-475)
+ *   q3m_attn_prep<HD> kernels/82_qwen3_omni.metal:30-88 (Q3PrepParams;   binding qwen3_omni.h:286-302)
+ * Per row of the fp32 fused projection X: every query and key head gets
+ * x * rsqrt(mean(x^2) + eps) * weight, then the rotation of its first rope_dims
+ * dims in the half-split pairing (d, d + rope_dims/2) by angle
+ * position * inv_freq[d mod rope_dims/2], then the cast to the storage type;
+ * queries are multiplied by q_scale after the rotation. Values are cast, or
+ * normalised without weight first (v_norm). */
+typedef struct esp_prep_params {
+  int32_t H, Hkv, head_dim, dtype;
+  int32_t x_ld;      /* floats between rows of X */
+  int32_t q_off;     /* column of query head 0 */
+  int32_t q_hs;      /* floats between query heads: head_dim, or 2 * head_dim with a gate beside each query (40_:47) */
+  int32_t k_off;     /* column of key head 0 (key heads head_dim apart) */
+  int32_t v_off;     /* column of value head 0 */
+  int32_t q_ld;      /* Q output row stride, elements */
+  int32_t kv_ld;     /* Kb / Vb output row stride, elements */
+  int32_t rope_dims; /* 64 in 40_:58-71, head_dim in 80_:99-104 and 82_:75-82, 0: no rotation; a power of two >= 8 */
+  int32_t v_norm;    /* 1: 80_:92-96; 0: 40_:81-83, 82_:58-62 */
+  int32_t bt;        /* tokens per KV block, for the folded append */
+  float eps;
+  float q_scale;     /* 82_:84; 1 in the other two */
+  uint64_t kv_base;  /* element offset of the layer's pool region, for the folded append */
+} esp_prep_params;
+
+/* X [n_rows][x_ld] fp32; qn_w / kn_w [head_dim] fp32; pos int32[4] per row (x, y, z
+ * position components); inv_freq [rope_dims / 2]; rope_sel [rope_dims / 2]: which position
+ * component each frequency rotates by (40_:62-63, 82_:77-79), NULL: all by pos.x (80_:99).
+ * Q [n_rows][q_ld], Kb / Vb [n_rows][kv_ld]: storage type.
+ * row_table NULL, or int32[4] per row = (block, position, block2, position2), -1 none
+ * (kv_row_table, forest.h:1737-1749): the row's K and V also go to those entries of
+ * kv_pool in the native layout, which replaces the kv_save dispatch after the attention
+ * (40_:86-100). The reference launches one SIMD group per (row, head); here one workgroup
+ * takes a row and computes the row's cos / sin once. */
+int esp_attn_prep(const esp_prep_params* p, const float* X, const float* qn_w, const float* kn_w, const int32_t* pos,
+                  const float* inv_freq, const int32_t* rope_sel, void* Q, void* Kb, void* Vb, const int32_t* row_table,
+                  void* kv_pool, int32_t n_rows, void* stream, char* err, size_t errlen);
 
 #ifdef __cplusplus
 }

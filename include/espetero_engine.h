@@ -91,6 +91,10 @@ int esp_engine_pass_pos(const esp_engine* e, int32_t* out);             /* 4 * M
 int esp_engine_pass_table(const esp_engine* e, int32_t* out);
 int esp_engine_pass_saves(const esp_engine* e, esp_kvsave* out);
 int esp_engine_pass_cow(const esp_engine* e, int32_t* out);             /* 2 * n_cow */
+/* kv_row_table (src/model/impl/forest.h:1737-1749): the pass's save records as one int32[4] per row,
+ * (block, position, block2, position2), -1 none - the row_table argument of esp_attn_prep.
+ * out: 4 * max(rows, 1) ints. Fails on a row saved into more than two slots. Needs no engine. */
+int esp_kv_row_table(const esp_kvsave* saves, int32_t n_saves, int32_t rows, int32_t* out, char* err, size_t errlen);
 /* The slots take their new block lists (after the device work completed). */
 int esp_engine_pass_commit(esp_engine* e);
 /* Give the pass's new blocks back; slots are as before the pass. */

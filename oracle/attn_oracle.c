@@ -25,6 +25,18 @@
  *                            80_:568-597).
  *   esp_oracle_kv_save       40_:875-889.   esp_oracle_kv_copy_blocks  40_:894-905.
  *   esp_oracle_kv_gather     the page walk alone (40_:245-247).
+ *   esp_oracle_attn_prep     the prep kernels, one (row, head) at a time: attn_prep
+ *                            40_:41-101, g4_attn_prep 80_:76-107, q3m_attn_prep
+ *                            82_:52-87 (norm, weight, half-split rotation, query
+ *                            scale, value cast / weightless norm, folded append
+ *                            into the reference-layout pool 40_:86-100).
+ *
+ * esp_oracle_attn_prep is pinned by a float64 restatement of the closed forms
+ * (RMSNorm, rotation matrix) in tests/test_prep.py, by norm preservation of the
+ * rotation, by position 0 == no rotation, and by the folded append == kv_save of
+ * the outputs. Its cos / sin are libm's on the fp32 angle the kernels form; the
+ * reference's precise::cos / sin and rsqrt are not bit-reproducible here, so
+ * outputs agree to one unit in the last place of the storage type, not bit for bit.
  *
  * Pinned by tests/test_oracle.py: float64 brute force on gathered K/V, torch
  * CPU scaled_dot_product_attention, closed forms (V == 1, single key, equal
@@ -366,4 +378,60 @@ void esp_oracle_kv_gather(const esp_attn_params* p, const uint16_t* pool, const 
     memcpy(K_out + (size_t)j * w, pool + cached_addr(&q, blocks, &t, j, 0, 0), 2 * w);
     memcpy(V_out + (size_t)j * w, pool + cached_addr(&q, blocks, &t, j, 1, 0), 2 * w);
   }
+}
+
+/* ---- attn_prep ---- */
+static inline uint16_t st_dt(int dtype, float f) { return dtype == ESP_F16 ? esp_oracle_f2h(f) : esp_oracle_f2bf(f); }
+
+void esp_oracle_attn_prep(const esp_prep_params* p, const float* X, const float* qn_w, const float* kn_w, const int32_t* pos,
+                          const float* inv_freq, const int32_t* rope_sel, uint16_t* Q, uint16_t* Kb, uint16_t* Vb,
+                          const int32_t* row_table, uint16_t* pool_ref, int n_rows) {
+  const int HD = p->head_dim, half = p->rope_dims / 2;
+  float* x = (float*)malloc(sizeof(float) * (size_t)HD);
+  float* y = (float*)malloc(sizeof(float) * (size_t)HD);
+  for (int row = 0; row < n_rows; ++row) {
+    const float* xr = X + (size_t)row * p->x_ld;
+    for (int slot = 0; slot < p->H + 2 * p->Hkv; ++slot) {
+      const int kind = slot < p->H ? 0 : (slot < p->H + p->Hkv ? 1 : 2);
+      const int h = kind == 0 ? slot : (kind == 1 ? slot - p->H : slot - p->H - p->Hkv);
+      const float* src = xr + (kind == 0 ? p->q_off + h * p->q_hs : (kind == 1 ? p->k_off : p->v_off) + h * HD);
+      float ss = 0.0f;
+      for (int d = 0; d < HD; ++d) {
+        x[d] = src[d];
+        ss += x[d] * x[d];
+      }
+      const float inv = 1.0f / sqrtf(ss / (float)HD + p->eps);
+      if (kind == 2) {
+        for (int d = 0; d < HD; ++d) y[d] = p->v_norm ? x[d] * inv : x[d];
+      } else {
+        const float* nw = kind == 0 ? qn_w : kn_w;
+        for (int d = 0; d < HD; ++d) x[d] = x[d] * inv * nw[d];
+        for (int d = 0; d < HD; ++d) y[d] = x[d];
+        for (int f = 0; f < half; ++f) {
+          const int sel = rope_sel ? rope_sel[f] : 0;
+          const float position = (float)pos[4 * row + (sel == 0 ? 0 : (sel == 1 ? 1 : 2))];
+          const float ang = position * inv_freq[f];
+          const float c = cosf(ang), sn = sinf(ang);
+          y[f] = x[f] * c - x[f + half] * sn;
+          y[f + half] = x[f + half] * c + x[f] * sn;
+        }
+        if (kind == 0)
+          for (int d = 0; d < HD; ++d) y[d] *= p->q_scale;
+      }
+      uint16_t* out = kind == 0 ? Q + (size_t)row * p->q_ld + (size_t)h * HD
+                                : (kind == 1 ? Kb : Vb) + (size_t)row * p->kv_ld + (size_t)h * HD;
+      for (int d = 0; d < HD; ++d) out[d] = st_dt(p->dtype, y[d]);
+      if (kind != 0 && row_table) {
+        const size_t blk = (size_t)p->bt * p->kv_ld;
+        for (int w = 0; w < 2; ++w) {
+          const int b = row_table[4 * row + 2 * w], ps = row_table[4 * row + 2 * w + 1];
+          if (b < 0) continue;
+          uint16_t* dst = pool_ref + p->kv_base + (size_t)b * 2 * blk + (kind == 2 ? blk : 0) + (size_t)ps * p->kv_ld + (size_t)h * HD;
+          memcpy(dst, out, sizeof(uint16_t) * (size_t)HD);
+        }
+      }
+    }
+  }
+  free(x);
+  free(y);
 }

@@ -103,6 +103,57 @@ def kv_gather(params, pool, blocks, n_tokens):
     return K, V
 
 
+def attn_prep(params, X, qn_w, kn_w, pos, inv_freq, rope_sel, n_rows, row_table=None, pool=None):
+    """Returns Q, Kb, Vb as storage bits; writes the folded append into `pool` (reference layout) in place."""
+    Q = np.zeros((n_rows, params.q_ld), np.uint16)
+    Kb = np.zeros((n_rows, params.kv_ld), np.uint16)
+    Vb = np.zeros((n_rows, params.kv_ld), np.uint16)
+    f32 = lambda a: None if a is None else np.ascontiguousarray(a, dtype=np.float32)  # noqa: E731
+    X, qn_w, kn_w, inv_freq = f32(X), f32(qn_w), f32(kn_w), f32(inv_freq)
+    pos, rope_sel, row_table = _i32(pos), _i32(rope_sel), _i32(row_table)
+    lib().esp_oracle_attn_prep(C.byref(params), _p(X), _p(qn_w), _p(kn_w), _p(pos), _p(inv_freq), _p(rope_sel), _p(Q), _p(Kb),
+                               _p(Vb), _p(row_table), _p(pool), C.c_int(n_rows))
+    return Q, Kb, Vb
+
+
+def attn_prep_f64(params, X, qn_w, kn_w, pos, inv_freq, rope_sel, n_rows):
+    """The closed forms in float64, no storage rounding: RMSNorm x / sqrt(mean x^2 + eps) * w, the rotation
+    [[c, -s], [s, c]] on each pair (d, d + rope_dims / 2) by angle position * inv_freq, the query scale.
+    The angle is formed in fp32 as the kernels form it (a float64 angle would be a different function of
+    the integer position once position * inv_freq no longer fits 24 bits)."""
+    p = params
+    HD, half = p.head_dim, p.rope_dims // 2
+    X = np.asarray(X, np.float64).reshape(n_rows, p.x_ld)
+    Q = np.zeros((n_rows, p.H, HD))
+    K = np.zeros((n_rows, p.Hkv, HD))
+    V = np.zeros((n_rows, p.Hkv, HD))
+    pos = np.asarray(pos, np.int64).reshape(n_rows, 4)
+    sel = np.zeros(half, np.int64) if rope_sel is None else np.asarray(rope_sel, np.int64)[:half]
+    ang = (pos[:, sel].astype(np.float32) * np.asarray(inv_freq, np.float32)[None, :half]).astype(np.float64)  # [rows][half]
+    c, s = np.cos(ang), np.sin(ang)
+
+    def norm(x):
+        return x / np.sqrt((x * x).mean(-1, keepdims=True) + np.float64(np.float32(p.eps)))
+
+    def rot(x):  # x [rows][heads][HD]
+        y = x.copy()
+        a, b = x[..., :half], x[..., half:2 * half]
+        y[..., :half] = a * c[:, None, :] - b * s[:, None, :]
+        y[..., half:2 * half] = b * c[:, None, :] + a * s[:, None, :]
+        return y
+
+    for h in range(p.H):
+        Q[:, h] = X[:, p.q_off + h * p.q_hs:p.q_off + h * p.q_hs + HD]
+    for h in range(p.Hkv):
+        K[:, h] = X[:, p.k_off + h * HD:p.k_off + (h + 1) * HD]
+        V[:, h] = X[:, p.v_off + h * HD:p.v_off + (h + 1) * HD]
+    Q = rot(norm(Q) * np.asarray(qn_w, np.float64)) * np.float64(np.float32(p.q_scale))
+    K = rot(norm(K) * np.asarray(kn_w, np.float64))
+    if p.v_norm:
+        V = norm(V)
+    return Q.reshape(n_rows, -1), K.reshape(n_rows, -1), V.reshape(n_rows, -1)
+
+
 # ---- storage conversions (numpy side) ----
 def to_f32(bits, dtype):
     bits = np.asarray(bits, dtype=np.uint16)

@@ -184,3 +184,16 @@ def tree_rows(base, Tr, next_pos, leaf_tokens, leaf_offsets, noncausal=False):
 def kv_saves(base, P, n, blocks, bt):
     """add_saves: src/model/impl/forest.h:2490-2494."""
     return [(base + i, blocks[(P + i) // bt], (P + i) % bt, 0) for i in range(n)]
+
+
+def kv_row_table(saves, rows):
+    """kv_row_table: src/model/impl/forest.h:1737-1749. saves: (src_row, block, pos, _) tuples."""
+    t = [[-1, -1, -1, -1] for _ in range(max(rows, 1))]
+    for (row, block, pos, _pad) in saves:
+        e = t[row]
+        j = 0 if e[0] < 0 else 2
+        if j == 2 and e[2] >= 0:
+            raise ValueError("a row saved into more than two slots")
+        e[j], e[j + 1] = block, pos
+    return t[:rows]
+

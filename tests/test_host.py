@@ -284,3 +284,19 @@ def test_verify_chain_is_one_tree_of_root_plus_k_rows():
     assert [(int(x["src_row"]), int(x["pos"])) for x in ps["saves"]] == [(0, 4), (1, 5), (2, 6), (3, 7)]
     e.pass_commit()
     assert e.slot_len(s) == 101
+
+
+def test_row_table_matches_the_restatement_and_refuses_a_third_slot():
+    """kv_row_table (src/model/impl/forest.h:1737-1749) through the C shim against its restatement."""
+    rng = np.random.default_rng(5)
+    rows = 23
+    saves = [(int(r), int(rng.integers(0, 50)), int(rng.integers(0, 16)), 0) for r in rng.permutation(rows)[:17]]
+    saves += [(saves[3][0], 7, 9, 0), (saves[8][0], 8, 1, 0)]          # two rows go to a second slot
+    got = host.row_table(np.array(saves, abi.KVSAVE_DT), rows)
+    assert got.tolist() == ho.kv_row_table(saves, rows)
+    assert (got[[r for r in range(rows) if r not in {s[0] for s in saves}]] == -1).all()
+    with pytest.raises(abi.EspError):
+        host.row_table(np.array(saves + [(saves[3][0], 1, 1, 0)], abi.KVSAVE_DT), rows)
+    with pytest.raises(ValueError):
+        ho.kv_row_table(saves + [(saves[3][0], 1, 1, 0)], rows)
+    assert host.row_table(np.zeros(0, abi.KVSAVE_DT), 4).tolist() == [[-1] * 4] * 4
