@@ -57,6 +57,25 @@ __device__ __forceinline__ void load_to_lds16(const void* base, uint32_t lane_of
                : "s"(lds_addr), "v"(lane_off), "s"(base)
                : "memory");
 }
+// Four such loads whose global and LDS addresses both advance by 1024 bytes from one to the next:
+// the instruction's immediate offset moves both, so one LDS base and one global base serve all four.
+__device__ __forceinline__ void load_to_lds16_x4(const void* base, uint32_t o0, uint32_t o1, uint32_t o2, uint32_t o3,
+                                                 uint32_t lds_addr) {
+  lds_addr = uint32_t(__builtin_amdgcn_readfirstlane(int(lds_addr)));
+  const uint64_t b64 = reinterpret_cast<uint64_t>(base);
+  const uint32_t b_lo = uint32_t(__builtin_amdgcn_readfirstlane(int(uint32_t(b64))));
+  const uint32_t b_hi = uint32_t(__builtin_amdgcn_readfirstlane(int(uint32_t(b64 >> 32))));
+  base = reinterpret_cast<const void*>(uint64_t(b_lo) | (uint64_t(b_hi) << 32));
+  asm volatile(
+      "s_mov_b32 m0, %0\n\ts_nop 0\n\t"
+      "global_load_lds_dwordx4 %1, %5\n\t"
+      "global_load_lds_dwordx4 %2, %5 offset:1024\n\t"
+      "global_load_lds_dwordx4 %3, %5 offset:2048\n\t"
+      "global_load_lds_dwordx4 %4, %5 offset:3072"
+      :
+      : "s"(lds_addr), "v"(o0), "v"(o1), "v"(o2), "v"(o3), "s"(base)
+      : "memory");
+}
 __device__ __forceinline__ void wait_loads() { asm volatile("s_waitcnt vmcnt(0)" ::: "memory"); }
 
 constexpr int swap23(int x) { return (x & ~12) | ((x & 4) << 1) | ((x & 8) >> 1); }
@@ -191,9 +210,11 @@ __global__ __launch_bounds__(256, OCC) void attn_tiled_kernel(const KArgs a, int
   // position `lane % CH` of row q RPI + lane / CH, i.e. global chunk position ^ pi(row).
   const int r0 = lane / CH;
   const uint32_t kcol0 = uint32_t(((lane % CH) ^ r0) << 4);
-  uint32_t koff_c[KP];  // cached keys: rows HD elements apart
+  // cached keys: rows HD elements apart, i.e. instruction q's rows start 1024 q bytes further; that part
+  // travels in the instruction's immediate offset
+  uint32_t koff_c[KP];
 #pragma unroll
-  for (int q = 0; q < KP; ++q) koff_c[q] = uint32_t((q * RPI + r0) * ROWB) + (kcol0 ^ uint32_t(swap23(q * RPI) << 4));
+  for (int q = 0; q < KP; ++q) koff_c[q] = uint32_t(r0 * ROWB) + (kcol0 ^ uint32_t(swap23(q * RPI) << 4));
   // V^T instruction q covers dims 32 q ..: this lane brings keys 8 (lane / 32) .. + 7 of dim 32 q + lane % 32.
   const uint32_t voff_c = uint32_t(l32 * a.bt * 2 + hb * 16);
   const uint32_t voff_b = uint32_t(l32 * 32 + hb * 16);
@@ -212,9 +233,15 @@ __global__ __launch_bounds__(256, OCC) void attn_tiled_kernel(const KArgs a, int
       const char* vb = hbp + (size_t(a.bt) * HD + t0) * 2;
       const size_t vstep = size_t(64) * a.bt;  // 32 V^T rows of bt elements
 #pragma unroll
-      for (int q = 0; q < KP; ++q) load_to_lds16(kb, koff_c[q], kdst + q * 1024);
+      for (int q = 0; q < KP; q += 4)
+        load_to_lds16_x4(kb + q * 1024, koff_c[q], koff_c[q + 1], koff_c[q + 2], koff_c[q + 3], kdst + q * 1024);
+      if (a.bt == 16) {  // 32 V^T rows of 16 tokens are 1024 bytes as well
 #pragma unroll
-      for (int q = 0; q < VP; ++q) load_to_lds16(vb + q * vstep, voff_c, vdst + q * 1024);
+        for (int q = 0; q < VP; q += 4) load_to_lds16_x4(vb + q * 1024, voff_c, voff_c, voff_c, voff_c, vdst + q * 1024);
+      } else {
+#pragma unroll
+        for (int q = 0; q < VP; ++q) load_to_lds16(vb + q * vstep, voff_c, vdst + q * 1024);
+      }
     } else if (s < n_sb) {
       const int g = a0 + (s - n_c);
       const int lim = min(15, a.n_rows - 1 - 16 * g);  // batch rows past the pass's last row do not exist
@@ -225,7 +252,7 @@ __global__ __launch_bounds__(256, OCC) void attn_tiled_kernel(const KArgs a, int
       for (int q = 0; q < KP; ++q)
         load_to_lds16(kb, uint32_t(min(q * RPI + r0, lim)) * kld + (kcol0 ^ uint32_t(swap23(q * RPI) << 4)), kdst + q * 1024);
 #pragma unroll
-      for (int q = 0; q < VP; ++q) load_to_lds16(vb + q * 1024, voff_b, vdst + q * 1024);
+      for (int q = 0; q < VP; q += 4) load_to_lds16_x4(vb + q * 1024, voff_b, voff_b, voff_b, voff_b, vdst + q * 1024);
     } else {  // past the range: K stays whatever it was (S is masked), V^T must be finite
 #pragma unroll
       for (int q = 0; q < VP; ++q)
