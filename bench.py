@@ -317,6 +317,29 @@ def prep_cpu_baseline(w):
             "max_abs_err_vs_gpu": err}
 
 
+def graph_replay(w, torch, steps=16, replays=8):
+    """The same steps captured once in a HIP graph and replayed: what a caller that enqueues a chain of
+    passes without host work in between (a decode chain) pays per step."""
+    try:
+        g = torch.cuda.CUDAGraph()
+        side = torch.cuda.Stream()
+        torch.cuda.synchronize()
+        with torch.cuda.stream(side):
+            with torch.cuda.graph(g, stream=side):
+                for i in range(steps):
+                    w.step(i)
+        torch.cuda.synchronize()
+        g.replay()
+        torch.cuda.synchronize()
+        t0 = time.perf_counter()
+        for _ in range(replays):
+            g.replay()
+        torch.cuda.synchronize()
+        return {"us_per_step": round((time.perf_counter() - t0) / (replays * steps) * 1e6, 3), "steps_per_graph": steps}
+    except RuntimeError as e:  # reported, never hidden: the timed figures above do not depend on it
+        return {"error": str(e).splitlines()[0][:200]}
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
@@ -391,6 +414,7 @@ def main():
                      "kernel_us_avg": round(kern_ms * 1e3, 3), "kernel_us_min": round(kern_min_ms * 1e3, 3),
                      "alg_bytes": int(w.alg_bytes), "alg_flops": int(w.alg_flops)},
     }
+    out["graph_replay"] = graph_replay(w, torch)
     if not args.no_cpu:
         w.step(0)   # leave rotation set 0's output in O: the CPU sample is checked against it
         torch.cuda.synchronize()

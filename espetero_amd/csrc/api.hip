@@ -18,6 +18,8 @@ hipError_t launch_kv_gather(const esp_attn_params* p, const void* pool, const in
                             void* V_out, hipStream_t st);
 hipError_t launch_kv_relayout(const esp_attn_params* p, const void* src, void* dst, int to_native, int n_blocks,
                               hipStream_t st);
+hipError_t launch_chain_advance(esp_tree* trees, int n_trees, int32_t* pos, int32_t* row_table, const int32_t* blocks, int bt,
+                                int ring, hipStream_t st);
 hipError_t launch_vt_stage(const esp_attn_params* p, const void* Vb, void* vt, int n_rows, hipStream_t st);
 hipError_t launch_attn_prep(const PrepArgs& a, int n_rows, hipStream_t st);
 int stream_workgroups_per_cu(int HD, int NC);
@@ -177,6 +179,8 @@ int esp_attn_forward(const esp_attn_params* p, const void* Q, const void* Kb, co
   if (fam < 0 && p->rows_per_tile > esp::tiled_max_rows(p->head_dim))
     return fail(err, errlen, ESP_EUNSUPPORTED, "rows_per_tile %d: the tiled kernel takes at most %d rows per tile at head_dim %d",
                 p->rows_per_tile, esp::tiled_max_rows(p->head_dim), p->head_dim);
+  if (fam > 0 && n_tiles > 65535)
+    return fail(err, errlen, ESP_EUNSUPPORTED, "%d tiles in one pass: the streaming kernel's grid takes at most 65535", n_tiles);
   const Carve c = carve(p, n_rows, n_parts);
   if (!workspace || workspace_bytes < c.total)
     return fail(err, errlen, ESP_EWORKSPACE, "workspace %zu bytes, %zu needed", workspace_bytes, c.total);
@@ -280,6 +284,19 @@ int esp_kv_relayout(const esp_attn_params* p, const void* src_pool, int32_t src_
   if (!src_pool || !dst_pool) return fail(err, errlen, ESP_EINVAL, "NULL argument");
   hipError_t e = esp::launch_kv_relayout(p, src_pool, dst_pool, dst_layout == ESP_LAYOUT_NATIVE, n_blocks, static_cast<hipStream_t>(stream));
   return e == hipSuccess ? ESP_OK : hip_fail(err, errlen, "kv_relayout launch", e);
+}
+
+int esp_chain_advance(esp_tree* trees, int32_t n_trees, int32_t* pos, int32_t* row_table, const int32_t* blocks, int32_t bt,
+                      int32_t ring, void* stream, char* err, size_t errlen) {
+  if (n_trees < 0) return fail(err, errlen, ESP_EINVAL, "negative count");
+  if (n_trees == 0) return ESP_OK;
+  if (!trees || !pos) return fail(err, errlen, ESP_EINVAL, "trees and pos must not be NULL");
+  if (bt <= 0 || bt % 16) return fail(err, errlen, ESP_EINVAL, "bt %d: tokens per block must be a positive multiple of 16", bt);
+  if (ring < 0) return fail(err, errlen, ESP_EINVAL, "ring negative");
+  if (row_table && !ring && !blocks) return fail(err, errlen, ESP_EINVAL, "blocks is NULL on a layer without rings");
+  const hipError_t e = esp::launch_chain_advance(trees, n_trees, pos, row_table, blocks, bt, ring, static_cast<hipStream_t>(stream));
+  if (e != hipSuccess) return hip_fail(err, errlen, "chain_advance launch", e);
+  return ESP_OK;
 }
 
 int esp_attn_prep(const esp_prep_params* p, const float* X, const float* qn_w, const float* kn_w, const int32_t* pos,

@@ -43,8 +43,9 @@ __global__ __launch_bounds__(256, OCC) void attn_stream_kernel(const KArgs a) {
   const int lane = threadIdx.x & 63;
   const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
   const int c16 = lane & 15, q4 = lane >> 4;
-  const esp_tile tile = a.tiles[blockIdx.y];
+  esp_tile tile = a.tiles[blockIdx.y];
   const esp_tree tree = a.trees[tile.tree];
+  if (tile.k1 == INT32_MAX) tile.k1 = tree.P;  // open-ended range: up to the tree's cached length as it is now
   // The planner may carry the tree's block-list offset in the tile (pad = table + 1): one
   // dependent load less before the first KV page can be requested.
   const int table = tile.pad > 0 ? tile.pad - 1 : tree.table;

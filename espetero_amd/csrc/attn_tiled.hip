@@ -107,8 +107,9 @@ __global__ __launch_bounds__(256, OCC) void attn_tiled_kernel(const KArgs a, int
   const int lane = threadIdx.x & 63;
   const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
   const int l32 = lane & 31, hb = lane >> 5;
-  const esp_tile tile = a.tiles[tile_i];
+  esp_tile tile = a.tiles[tile_i];
   const esp_tree tree = a.trees[tile.tree];
+  if (tile.k1 == INT32_MAX) tile.k1 = tree.P;  // open-ended range: up to the tree's cached length as it is now
   const int table = tile.pad > 0 ? tile.pad - 1 : tree.table;
   const int end = tree.base + tree.M;
   const int rows_live = min(a.R, end - tile.r0);

@@ -128,6 +128,37 @@ __global__ __launch_bounds__(256) void vt_stage_kernel(const uint16_t* Vb, uint1
   }
 }
 
+// One decode step further for every single-row tree of a device-resident pass: the row's own
+// key joins the cache (P + 1), its position components move on by one, and its pool entry becomes
+// the next token's (block list, or the slot's ring). The reference's decode chain
+// (src/model/model.mm:779-850) has the host encode every step's records; here the device moves
+// them on, so a chain of steps is enqueued - or captured in a graph - with no host work between.
+__global__ __launch_bounds__(256) void chain_advance_kernel(esp_tree* trees, int n_trees, int4* pos, int4* row_table,
+                                                            const int32_t* blocks, int bt, int ring) {
+  const int i = blockIdx.x * 256 + threadIdx.x;
+  if (i >= n_trees) return;
+  esp_tree t = trees[i];
+  t.P += 1;
+  trees[i] = t;
+  int4 ps = pos[t.base];
+  ps.x += 1;
+  ps.y += 1;
+  ps.z += 1;
+  pos[t.base] = ps;
+  if (row_table) {
+    const int bi = t.P / bt;
+    const int b = ring ? t.table + bi % ring : blocks[t.table + bi];
+    row_table[t.base] = make_int4(b, t.P % bt, -1, -1);
+  }
+}
+
+hipError_t launch_chain_advance(esp_tree* trees, int n_trees, int32_t* pos, int32_t* row_table, const int32_t* blocks, int bt,
+                                int ring, hipStream_t st) {
+  hipLaunchKernelGGL(chain_advance_kernel, dim3((n_trees + 255) / 256), dim3(256), 0, st, trees, n_trees,
+                     reinterpret_cast<int4*>(pos), reinterpret_cast<int4*>(row_table), blocks, bt, ring);
+  return hipGetLastError();
+}
+
 hipError_t launch_kv_save(const esp_attn_params* p, const void* Kb, const void* Vb, void* pool, const esp_kvsave* e, int n,
                           hipStream_t st) {
   const long total = long(n) * (p->Hkv * p->head_dim / 8);

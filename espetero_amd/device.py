@@ -113,6 +113,13 @@ def attn_prep(params, X, qn_w, kn_w, pos, inv_freq, rope_sel, Q, Kb, Vb, row_tab
                                            _stream(stream), err, _ERRLEN), err)
 
 
+def chain_advance(trees, n_trees, pos, row_table, blocks, bt, ring=0, stream=None):
+    """Device tensors: trees (TREE_DT bytes), pos / row_table int32 [rows][4], blocks int32."""
+    err = C.create_string_buffer(_ERRLEN)
+    abi.check(abi.attn_lib().esp_chain_advance(_ptr(trees), n_trees, _ptr(pos), _ptr(row_table), _ptr(blocks), bt, ring,
+                                               _stream(stream), err, _ERRLEN), err)
+
+
 class DevicePass:
     """One planned pass resident on the device: uploads the records once and
     replays esp_attn_forward (what a decode chain does between host syncs)."""

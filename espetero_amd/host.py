@@ -103,6 +103,16 @@ def plan_tiles(trees, groups, window, pos, options):
     return tiles, jobs, npart.value
 
 
+def open_ended(tiles, trees):
+    """Tiles of a decode chain: every tile whose cached range ends at its tree's cached length P gets
+    k1 = INT32_MAX, which the kernels read as "up to P as the device holds it now", so the same records
+    serve every step of a chain that esp_chain_advance moves on."""
+    tiles = np.array(tiles, dtype=abi.TILE_DT, copy=True)
+    P = np.asarray(trees["P"])[tiles["tree"]]
+    tiles["k1"] = np.where(tiles["k1"] == P, np.int32(2**31 - 1), tiles["k1"])
+    return tiles
+
+
 def row_table(saves, rows):
     """KVSAVE_DT records -> int32 [rows][4] = (block, position, block2, position2), -1 none."""
     saves = np.ascontiguousarray(saves, dtype=abi.KVSAVE_DT)

@@ -239,6 +239,26 @@ int esp_attn_prep(const esp_prep_params* p, const float* X, const float* qn_w, c
                   const float* inv_freq, const int32_t* rope_sel, void* Q, void* Kb, void* Vb, const int32_t* row_table,
                   void* kv_pool, int32_t n_rows, void* stream, char* err, size_t errlen);
 
+/* ---- decode chains ---------------------------------------------------------------
+ * The reference runs K greedy decode steps as one GPU chain (run_chain,
+ * src/model/model.mm:779-850, docs/design.md:226-243): the host encodes the K
+ * passes one after the other (run_forest per step, each with its own tree,
+ * position and KV-entry records from the pass arena) and waits once at the end. Here the records stay where they are and the
+ * device moves them on, so a chain is a sequence of enqueues with no host work
+ * in between, and can be captured in a HIP graph:
+ *   - a tile whose k1 is INT32_MAX ends at its tree's cached length P as the
+ *     trees array holds it when the kernel runs (both attention kernels);
+ *   - esp_chain_advance turns the records of a pass of single-row trees into
+ *     those of the next step: P + 1, every position component + 1, and the
+ *     row's row_table entry (esp_attn_prep) = the pool entry of position P + 1
+ *     taken from the tree's block list (or its ring). The block lists must
+ *     already hold the blocks the chain will reach (the reference reserves
+ *     them before the pass too: target_new_blocks, forest.h:1821-1829, model.mm:575).
+ * trees, pos (int32[4] per row), row_table (int32[4] per row, may be NULL),
+ * blocks: device memory. Trees with M != 1 are not meant for it. */
+int esp_chain_advance(esp_tree* trees, int32_t n_trees, int32_t* pos, int32_t* row_table, const int32_t* blocks, int32_t bt,
+                      int32_t ring, void* stream, char* err, size_t errlen);
+
 #ifdef __cplusplus
 }
 #endif

@@ -1,0 +1,157 @@
+"""A decode chain kept on the device: prep (with the folded append) -> attention -> esp_chain_advance,
+K steps enqueued back to back and captured in a HIP graph, against the CPU checker driven step by step
+from the host (the reference's statement about its own chains: "tokens are identical to step-by-step
+decoding", docs/design.md:232)."""
+import numpy as np
+import pytest
+import torch
+
+from espetero_amd import abi, device, host, synth
+from oracle import binding as ob
+
+pytestmark = pytest.mark.gpu
+
+H, HKV, HD, BT, K = 8, 2, 128, 16, 10
+P0 = [70, 33, 500, 1030, 16, 0]
+
+
+def _setup(seed=12):
+    rng = np.random.default_rng(seed)
+    n = len(P0)
+    ap = synth.make_params(H, HKV, HD, abi.ESP_F16, BT, rows_per_tile=1)
+    pp, a = synth.make_prep("omni", H, HKV, HD, abi.ESP_F16, n, seed=seed, bt=BT)
+    nb = [(p + K + BT) // BT for p in P0]                      # room for the K tokens the chain appends
+    n_blocks = sum(nb) + 3
+    perm = rng.permutation(n_blocks).astype(np.int32)
+    blocks = perm[:sum(nb)].copy()
+    trees = np.zeros(n, abi.TREE_DT)
+    kvw = HKV * HD
+    pool = np.zeros(n_blocks * 2 * BT * kvw, np.uint16)       # reference layout
+    pv = pool.reshape(n_blocks, 2, BT, kvw)
+    off = 0
+    for i, p in enumerate(P0):
+        trees[i] = (i, p, off, 1)
+        for j in range(p):
+            b = blocks[off + j // BT]
+            pv[b, 0, j % BT] = ob.from_f32(rng.standard_normal(kvw).astype(np.float32) * 0.5, ap.dtype)
+            pv[b, 1, j % BT] = ob.from_f32(rng.standard_normal(kvw).astype(np.float32) * 0.5, ap.dtype)
+        off += nb[i]
+    X = (rng.standard_normal((K, n, pp.x_ld)).astype(np.float32) * 0.5)   # values as in the other tests: |v| < 4, half a unit in the last place of an output < 1e-3
+    return ap, pp, a, trees, blocks, pool, n_blocks, X
+
+
+def _host_chain(ap, trees, blocks, pool, Q, Kb, Vb):
+    """The checker, one step at a time, every record rebuilt on the host. Q / Kb / Vb [K][n][...]: the
+    prepared rows of every step (storage bits); each step's K / V row joins the cache after its attention."""
+    n = len(trees)
+    pool = pool.copy()
+    trees = trees.copy()
+    out = []
+    for s in range(K):
+        pos = np.zeros((n, 4), np.int32)
+        pos[:, :3] = trees["P"][:, None]
+        desc = np.zeros((n, 4), np.int32)
+        out.append(ob.attn_direct(ap, Q[s], Kb[s], Vb[s], pool, blocks, desc, pos, trees, n_threads=4))
+        e = np.zeros(n, abi.KVSAVE_DT)
+        e["src_row"], e["block"], e["pos"] = np.arange(n), blocks[trees["table"] + trees["P"] // BT], trees["P"] % BT
+        ob.kv_save(ap, Kb[s], Vb[s], pool, e)
+        trees["P"] += 1
+    return np.stack(out), pool
+
+
+def test_device_chain_matches_the_checker_step_by_step_and_replays_identically():
+    device.init(0)
+    ap, pp, a, trees, blocks, pool_ref, n_blocks, X = _setup()
+    n = len(trees)
+
+    dev = lambda x: torch.from_numpy(np.ascontiguousarray(x)).cuda()  # noqa: E731
+    ref = dev(pool_ref.view(np.int16))
+    pool0 = torch.empty_like(ref)
+    device.kv_relayout(ap, ref, abi.ESP_LAYOUT_REFERENCE, pool0, abi.ESP_LAYOUT_NATIVE, n_blocks)
+    resident, groups = device.plan_hint(ap)
+    tiles, jobs, n_parts = host.plan_tiles(trees, groups, 0, None, host.options_mi355x(1, resident))
+    tiles = host.open_ended(tiles, trees)
+    assert (tiles["k1"] == 2**31 - 1).sum() == n               # one open range per sequence
+    pos0 = np.zeros((n, 4), np.int32)
+    pos0[:, :3] = trees["P"][:, None]
+    table0 = np.full((n, 4), -1, np.int32)
+    table0[:, 0] = blocks[trees["table"] + trees["P"] // BT]
+    table0[:, 1] = trees["P"] % BT
+    # device-resident state of the chain, and its initial values to go back to before every run
+    init = dict(trees=device.to_dev(trees), pos=dev(pos0), table=dev(table0), pool=pool0)
+    st = {k: v.clone() for k, v in init.items()}
+    blocks_d = dev(blocks)
+    dp = device.DevicePass(ap, trees, tiles, jobs, n_parts, n, blocks, None, None)
+    dp.trees = st["trees"]                                      # the pass reads the records the chain advances
+    Xd, qn, kn = dev(X), dev(a["qn_w"]), dev(a["kn_w"])
+    inv_freq, sel = dev(a["inv_freq"]), dev(a["rope_sel"])
+    Q = torch.zeros(K, n, ap.q_ld, dtype=torch.float16, device="cuda")      # every step's prepared rows are kept
+    Kb = torch.zeros(K, n, ap.kv_ld, dtype=torch.float16, device="cuda")
+    Vb = torch.zeros_like(Kb)
+    O = torch.zeros(K, n, ap.q_ld, dtype=torch.float16, device="cuda")
+
+    def chain():
+        for s in range(K):
+            device.attn_prep(pp, Xd[s], qn, kn, st["pos"], inv_freq, sel, Q[s], Kb[s], Vb[s], st["table"], st["pool"], n)
+            dp.run(Q[s], Kb[s], Vb[s], st["pool"], O[s])
+            device.chain_advance(st["trees"], n, st["pos"], st["table"], blocks_d, BT)
+
+    def reset():
+        for k in st:
+            st[k].copy_(init[k])
+        O.zero_()
+
+    bits = lambda t: t.view(torch.int16).cpu().numpy().view(np.uint16)  # noqa: E731
+    ref_out = {}
+
+    def check(tag):
+        torch.cuda.synchronize()
+        if not ref_out:   # the checker runs on the rows the device prepared, so that this compares attention with attention
+            ref_out["want"], ref_out["pool"] = _host_chain(ap, trees, blocks, pool_ref, bits(Q), bits(Kb), bits(Vb))
+        want = ref_out["want"]
+        got = ob.to_f32(bits(O), ap.dtype)
+        err = float(np.abs(got - ob.to_f32(want, ap.dtype)).max())
+        print(f"chain {tag}: max abs err {err:.2e}", flush=True)
+        assert err <= 2e-3, (tag, err)
+        # the records ended where K steps of host bookkeeping end
+        t = st["trees"].cpu().numpy().view(abi.TREE_DT)
+        assert (t["P"] == trees["P"] + K).all()
+        assert (st["pos"].cpu().numpy()[:, 0] == trees["P"] + K).all()
+        return O.clone()
+
+    reset()
+    chain()                                                     # enqueued eagerly, no host work in between
+    eager = check("eager")
+    # the prep inside the chain saw the positions the device advanced: its rows are the checker's rows for
+    # host-built positions (to the prep kernel's bar of one unit in the last place)
+    for s_ in range(K):
+        pos = np.zeros((n, 4), np.int32)
+        pos[:, :3] = (trees["P"] + s_)[:, None]
+        qw, kw, vw = ob.attn_prep(pp, X[s_], a["qn_w"], a["kn_w"], pos, a["inv_freq"], a["rope_sel"], n)
+        for g_, w_ in ((bits(Q[s_]), qw), (bits(Kb[s_]), kw), (bits(Vb[s_]), vw)):
+            assert np.abs(ob.to_f32(g_, ap.dtype).astype(np.float64) - ob.to_f32(w_, ap.dtype)).max() <= 2.0 ** -8
+    # every appended token is in the pool where host bookkeeping puts it: bit for bit
+    Kg = torch.zeros((max(P0) + K) * ap.kv_ld, dtype=torch.float16, device="cuda")
+    Vg = torch.zeros_like(Kg)
+    for i, p in enumerate(P0):
+        device.kv_gather(ap, st["pool"], blocks_d[int(trees[i]["table"]):], p + K, Kg, Vg)
+        torch.cuda.synchronize()
+        kw, vw = ob.kv_gather(ap, ref_out["pool"], blocks[int(trees[i]["table"]):], p + K)
+        assert np.array_equal(bits(Kg)[:(p + K) * ap.kv_ld].reshape(p + K, -1), kw)
+        assert np.array_equal(bits(Vg)[:(p + K) * ap.kv_ld].reshape(p + K, -1), vw)
+
+    # the same chain as one HIP graph, replayed with eager work and synchronisations in between
+    reset()
+    torch.cuda.synchronize()
+    g = torch.cuda.CUDAGraph()
+    side = torch.cuda.Stream()
+    with torch.cuda.stream(side):
+        with torch.cuda.graph(g, stream=side):
+            chain()
+    torch.cuda.synchronize()
+    for rep in range(3):
+        reset()
+        torch.cuda.synchronize()
+        g.replay()
+        got = check(f"graph replay {rep}")
+        assert torch.equal(got.view(torch.int16), eager.view(torch.int16))

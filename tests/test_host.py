@@ -300,3 +300,14 @@ def test_row_table_matches_the_restatement_and_refuses_a_third_slot():
     with pytest.raises(ValueError):
         ho.kv_row_table(saves + [(saves[3][0], 1, 1, 0)], rows)
     assert host.row_table(np.zeros(0, abi.KVSAVE_DT), 4).tolist() == [[-1] * 4] * 4
+
+
+def test_open_ended_marks_exactly_the_ranges_that_end_at_the_cached_length():
+    trees = np.array([(0, 5000, 0, 1), (1, 40, 400, 1), (2, 0, 500, 1)], abi.TREE_DT)
+    tiles, jobs, n_parts = host.plan_tiles(trees, 4, 0, None, host.options_mi355x(1, 64))
+    opened = host.open_ended(tiles, trees)
+    last = tiles["k1"] == trees["P"][tiles["tree"]]
+    assert last.sum() == 3 and (tiles["last"][last] == 1).all()        # one per tree, and it is the part with the batch keys
+    assert (opened["k1"][last] == 2**31 - 1).all() and (opened["k1"][~last] == tiles["k1"][~last]).all()
+    for f in ("tree", "r0", "k0", "part", "last", "b0", "pad"):
+        assert (opened[f] == tiles[f]).all()
