@@ -81,6 +81,8 @@ ATTN_SYMBOLS = {
     "esp_kv_copy_blocks": (C.c_int, (_P, _V, _V, C.c_int32, C.c_int32, C.c_uint64, _V) + _ERR),
     "esp_kv_gather": (C.c_int, (_P, _V, _V, C.c_int32, _V, _V, _V) + _ERR),
     "esp_kv_relayout": (C.c_int, (_P, _V, C.c_int32, _V, C.c_int32, C.c_int32, _V) + _ERR),
+    "esp_kv_export_blocks": (C.c_int, (_P, _V, _V, C.c_int32, _V, _V) + _ERR),
+    "esp_kv_import_blocks": (C.c_int, (_P, _V, _V, C.c_int32, _V, _V) + _ERR),
     "esp_chain_advance": (C.c_int, (_V, C.c_int32, _V, _V, _V, C.c_int32, C.c_int32, _V) + _ERR),
     "esp_attn_prep": (C.c_int, (C.POINTER(PrepParams), _V, _V, _V, _V, _V, _V, _V, _V, _V, _V, _V, C.c_int32, _V) + _ERR),
 }

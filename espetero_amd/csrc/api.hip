@@ -17,7 +17,7 @@ hipError_t launch_kv_copy_blocks(const esp_attn_params* p, void* pool, const int
 hipError_t launch_kv_gather(const esp_attn_params* p, const void* pool, const int32_t* blocks, int n, void* K_out,
                             void* V_out, hipStream_t st);
 hipError_t launch_kv_relayout(const esp_attn_params* p, const void* src, void* dst, int to_native, int n_blocks,
-                              hipStream_t st);
+                              const int32_t* ids, hipStream_t st);
 hipError_t launch_chain_advance(esp_tree* trees, int n_trees, int32_t* pos, int32_t* row_table, const int32_t* blocks, int bt,
                                 int ring, hipStream_t st);
 hipError_t launch_vt_stage(const esp_attn_params* p, const void* Vb, void* vt, int n_rows, hipStream_t st);
@@ -282,8 +282,31 @@ int esp_kv_relayout(const esp_attn_params* p, const void* src_pool, int32_t src_
     return fail(err, errlen, ESP_EINVAL, "layouts %d -> %d: one side reference, the other native", src_layout, dst_layout);
   if (n_blocks == 0) return ESP_OK;
   if (!src_pool || !dst_pool) return fail(err, errlen, ESP_EINVAL, "NULL argument");
-  hipError_t e = esp::launch_kv_relayout(p, src_pool, dst_pool, dst_layout == ESP_LAYOUT_NATIVE, n_blocks, static_cast<hipStream_t>(stream));
+  hipError_t e = esp::launch_kv_relayout(p, src_pool, dst_pool, dst_layout == ESP_LAYOUT_NATIVE, n_blocks, nullptr,
+                                         static_cast<hipStream_t>(stream));
   return e == hipSuccess ? ESP_OK : hip_fail(err, errlen, "kv_relayout launch", e);
+}
+
+int esp_kv_export_blocks(const esp_attn_params* p, const void* kv_pool, const int32_t* blocks, int32_t n_blocks, void* out,
+                         void* stream, char* err, size_t errlen) {
+  if (int rc = check_params(p, err, errlen)) return rc;
+  if (n_blocks < 0) return fail(err, errlen, ESP_EINVAL, "n_blocks negative");
+  if (n_blocks == 0) return ESP_OK;
+  if (!kv_pool || !blocks || !out) return fail(err, errlen, ESP_EINVAL, "NULL argument");
+  hipError_t e = esp::launch_kv_relayout(p, static_cast<const uint16_t*>(kv_pool) + p->kv_base, out, 0, n_blocks, blocks,
+                                         static_cast<hipStream_t>(stream));
+  return e == hipSuccess ? ESP_OK : hip_fail(err, errlen, "kv_export_blocks launch", e);
+}
+
+int esp_kv_import_blocks(const esp_attn_params* p, const void* in, const int32_t* blocks, int32_t n_blocks, void* kv_pool,
+                         void* stream, char* err, size_t errlen) {
+  if (int rc = check_params(p, err, errlen)) return rc;
+  if (n_blocks < 0) return fail(err, errlen, ESP_EINVAL, "n_blocks negative");
+  if (n_blocks == 0) return ESP_OK;
+  if (!kv_pool || !blocks || !in) return fail(err, errlen, ESP_EINVAL, "NULL argument");
+  hipError_t e = esp::launch_kv_relayout(p, in, static_cast<uint16_t*>(kv_pool) + p->kv_base, 1, n_blocks, blocks,
+                                         static_cast<hipStream_t>(stream));
+  return e == hipSuccess ? ESP_OK : hip_fail(err, errlen, "kv_import_blocks launch", e);
 }
 
 int esp_chain_advance(esp_tree* trees, int32_t n_trees, int32_t* pos, int32_t* row_table, const int32_t* blocks, int32_t bt,

@@ -62,8 +62,10 @@ __global__ __launch_bounds__(256) void kv_gather_kernel(const uint16_t* pool, co
 
 // Whole blocks between layouts. Reference block: [K | V][t][h][d] (40_:245-247).
 // One thread per (block, which, t, 8 elements of the row).
+// ids (may be null): block b of the reference-layout side is block ids[b] of the native side - the
+// blocks of one slot in logical order, as a slot checkpoint file holds them (src/model/model.mm:653-655).
 __global__ __launch_bounds__(256) void kv_relayout_kernel(const uint16_t* src, uint16_t* dst, int to_native, int n_blocks,
-                                                          int Hkv, int HD, int bt) {
+                                                          int Hkv, int HD, int bt, const int32_t* ids) {
   const int w = Hkv * HD;
   const long per_block = long(2) * bt * (w / 8);
   const long gid = long(blockIdx.x) * 256 + threadIdx.x;
@@ -76,7 +78,7 @@ __global__ __launch_bounds__(256) void kv_relayout_kernel(const uint16_t* src, u
   const int x = int(rem % (w / 8)) * 8;
   const int kvh = x / HD, d = x % HD;
   const size_t ref_off = size_t(b) * 2 * bt * w + (size_t(which) * bt + t) * w + x;
-  const size_t hb = (size_t(b) * Hkv + kvh) * size_t(2 * bt * HD);
+  const size_t hb = (size_t(ids ? ids[b] : b) * Hkv + kvh) * size_t(2 * bt * HD);
   if (which == 0) {
     const size_t nat = hb + size_t(t) * HD + d;
     if (to_native) *reinterpret_cast<u32x4*>(dst + nat) = *reinterpret_cast<const u32x4*>(src + ref_off);
@@ -184,10 +186,10 @@ hipError_t launch_kv_gather(const esp_attn_params* p, const void* pool, const in
 }
 
 hipError_t launch_kv_relayout(const esp_attn_params* p, const void* src, void* dst, int to_native, int n_blocks,
-                              hipStream_t st) {
+                              const int32_t* ids, hipStream_t st) {
   const long total = long(n_blocks) * 2 * p->bt * (p->Hkv * p->head_dim / 8);
   hipLaunchKernelGGL(kv_relayout_kernel, dim3((unsigned)((total + 255) / 256)), dim3(256), 0, st, (const uint16_t*)src,
-                     (uint16_t*)dst, to_native, n_blocks, p->Hkv, p->head_dim, p->bt);
+                     (uint16_t*)dst, to_native, n_blocks, p->Hkv, p->head_dim, p->bt, ids);
   return hipGetLastError();
 }
 

@@ -105,6 +105,18 @@ def kv_relayout(params, src, src_layout, dst, dst_layout, n_blocks, stream=None)
                                              _stream(stream), err, _ERRLEN), err)
 
 
+def kv_export_blocks(params, pool, blocks, n_blocks, out, stream=None):
+    err = C.create_string_buffer(_ERRLEN)
+    abi.check(abi.attn_lib().esp_kv_export_blocks(C.byref(params), _ptr(pool), _ptr(blocks), n_blocks, _ptr(out),
+                                                  _stream(stream), err, _ERRLEN), err)
+
+
+def kv_import_blocks(params, src, blocks, n_blocks, pool, stream=None):
+    err = C.create_string_buffer(_ERRLEN)
+    abi.check(abi.attn_lib().esp_kv_import_blocks(C.byref(params), _ptr(src), _ptr(blocks), n_blocks, _ptr(pool),
+                                                  _stream(stream), err, _ERRLEN), err)
+
+
 def attn_prep(params, X, qn_w, kn_w, pos, inv_freq, rope_sel, Q, Kb, Vb, row_table, pool, n_rows, stream=None):
     """All device tensors; rope_sel, row_table and pool may be None."""
     err = C.create_string_buffer(_ERRLEN)

@@ -5,6 +5,7 @@
 
 #include "kv_engine.hpp"
 #include "planner.hpp"
+#include "slot_file.hpp"
 
 using namespace espetero::engine;
 
@@ -176,6 +177,28 @@ int esp_kv_row_table(const esp_kvsave* saves, int32_t n_saves, int32_t rows, int
     if (err && errlen) snprintf(err, errlen, "%s", ex.what());
     return 1;
   }
+}
+int esp_slot_file_save(const char* path, int32_t len, int32_t next_pos, int32_t n_blocks, int32_t n_layers, uint64_t block_bytes,
+                       const void* kv) {
+  if (!path || len < 0 || n_blocks < 0 || n_layers < 0 || (!kv && n_blocks > 0 && n_layers > 0)) return -1;
+  espetero::engine::SlotInfo s;
+  s.len = len, s.next_pos = next_pos, s.n_blocks = n_blocks, s.n_layers = n_layers, s.block_bytes = block_bytes;
+  return espetero::engine::slot_file_save(path, s, kv) ? 0 : -1;
+}
+int esp_slot_file_info(const char* path, int32_t bt, int32_t* len, int32_t* next_pos, int32_t* n_blocks, int32_t* n_layers,
+                       uint64_t* block_bytes) {
+  if (!path || bt <= 0) return -1;
+  espetero::engine::SlotInfo s;
+  if (espetero::engine::slot_file_info(path, bt, &s) != 0) return -1;
+  *len = s.len, *next_pos = s.next_pos, *n_blocks = s.n_blocks, *n_layers = s.n_layers, *block_bytes = s.block_bytes;
+  return 0;
+}
+int esp_slot_file_load(const char* path, int32_t bt, void* kv, uint64_t kv_bytes) {
+  if (!path || bt <= 0) return -1;
+  espetero::engine::SlotInfo s;
+  if (espetero::engine::slot_file_info(path, bt, &s) != 0) return -1;
+  if (kv_bytes < uint64_t(s.n_layers) * uint64_t(s.n_blocks) * s.block_bytes) return -1;
+  return espetero::engine::slot_file_load(path, s, kv);
 }
 int esp_engine_pass_commit(esp_engine* e) { return guarded([&] { e->e.pass_commit(); }); }
 int esp_engine_pass_abort(esp_engine* e) { return guarded([&] { e->e.pass_abort(); }); }

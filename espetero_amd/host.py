@@ -49,6 +49,9 @@ ENGINE_SYMBOLS = {
     "esp_engine_pass_table": (C.c_int, (_V, _V)),
     "esp_engine_pass_saves": (C.c_int, (_V, _V)),
     "esp_engine_pass_cow": (C.c_int, (_V, _V)),
+    "esp_slot_file_save": (C.c_int, (C.c_char_p, C.c_int32, C.c_int32, C.c_int32, C.c_int32, C.c_uint64, _V)),
+    "esp_slot_file_info": (C.c_int, (C.c_char_p, C.c_int32, _V, _V, _V, _V, _V)),
+    "esp_slot_file_load": (C.c_int, (C.c_char_p, C.c_int32, _V, C.c_uint64)),
     "esp_kv_row_table": (C.c_int, (_V, C.c_int32, C.c_int32, _V, C.c_char_p, C.c_size_t)),
     "esp_engine_pass_commit": (C.c_int, (_V,)),
     "esp_engine_pass_abort": (C.c_int, (_V,)),
@@ -101,6 +104,32 @@ def plan_tiles(trees, groups, window, pos, options):
                             C.byref(nj), C.byref(npart), err, 256)
     abi.check(rc, err)
     return tiles, jobs, npart.value
+
+
+def slot_file_save(path, length, next_pos, n_layers, blocks_kv):
+    """blocks_kv: host array [n_layers][n_blocks][block elements] of storage bits in the reference's block layout."""
+    kv = np.ascontiguousarray(blocks_kv)
+    n_layers_, n_blocks = kv.shape[0], kv.shape[1]
+    assert n_layers_ == n_layers
+    block_bytes = kv[0, 0].nbytes if n_blocks else 0
+    rc = engine_lib().esp_slot_file_save(str(path).encode(), length, next_pos, n_blocks, n_layers, block_bytes,
+                                         kv.ctypes.data if kv.size else None)
+    if rc != 0:
+        raise abi.EspError(f"slot_file_save({path}) failed")
+
+
+def slot_file_load(path, bt):
+    """Returns dict(len, next_pos, n_blocks, n_layers, block_bytes, kv = uint8 [n_layers][n_blocks][block_bytes]), or None
+    for a file the loader refuses (slot_load's -1, src/model/model.mm:700-714)."""
+    v = [C.c_int32(0) for _ in range(4)]
+    bb = C.c_uint64(0)
+    if engine_lib().esp_slot_file_info(str(path).encode(), bt, *[C.byref(x) for x in v], C.byref(bb)) != 0:
+        return None
+    length, next_pos, n_blocks, n_layers = (x.value for x in v)
+    kv = np.zeros((n_layers, n_blocks, bb.value), np.uint8)
+    if engine_lib().esp_slot_file_load(str(path).encode(), bt, kv.ctypes.data if kv.size else None, kv.nbytes) != 0:
+        return None
+    return dict(len=length, next_pos=next_pos, n_blocks=n_blocks, n_layers=n_layers, block_bytes=bb.value, kv=kv)
 
 
 def open_ended(tiles, trees):

@@ -198,6 +198,16 @@ int esp_kv_gather(const esp_attn_params* p, const void* kv_pool, const int32_t* 
 int esp_kv_relayout(const esp_attn_params* p, const void* src_pool, int32_t src_layout, void* dst_pool, int32_t dst_layout,
                     int32_t n_blocks, void* stream, char* err, size_t errlen);
 
+/* The KV payload of a slot checkpoint file (src/model/model.mm:649-655 writes, :727-729 reads): for one
+ * layer (p->kv_base), the slot's blocks in logical order, each in the reference's block layout
+ * [K plane | V plane][token][kv head][dim]. export: block blocks[i] of the native pool -> block i of
+ * `out`; import: block i of `in` -> block blocks[i] of the native pool. kv_pool is the pool's base
+ * (kv_base is applied). out / in: device memory, n_blocks * 2 * bt * Hkv * head_dim elements. Bit copies. */
+int esp_kv_export_blocks(const esp_attn_params* p, const void* kv_pool, const int32_t* blocks, int32_t n_blocks, void* out,
+                         void* stream, char* err, size_t errlen);
+int esp_kv_import_blocks(const esp_attn_params* p, const void* in, const int32_t* blocks, int32_t n_blocks, void* kv_pool,
+                         void* stream, char* err, size_t errlen);
+
 /* ---- attn_prep: the step before the attention of a layer ----------------------
  * One entry point for the reference's three prep kernels:
  *   attn_prep        kernels/40_attention.metal:9-102   (AttnPrepParams; binding forest.h:2951-2977)

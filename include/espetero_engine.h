@@ -91,6 +91,17 @@ int esp_engine_pass_pos(const esp_engine* e, int32_t* out);             /* 4 * M
 int esp_engine_pass_table(const esp_engine* e, int32_t* out);
 int esp_engine_pass_saves(const esp_engine* e, esp_kvsave* out);
 int esp_engine_pass_cow(const esp_engine* e, int32_t* out);             /* 2 * n_cow */
+/* Slot checkpoint files in the reference's format (src/model/model.mm:600-752), KV section: the
+ * 120-byte CkptHeader (magic 0x554b5043, version 4), then n_layers x n_blocks blocks of block_bytes,
+ * layer-major, logical block order, each in the reference's block layout (what
+ * esp_kv_export_blocks produces per layer). The sections of other subsystems are written as absent.
+ * kv: host memory. save: 0 or -1. info / load: 0, or -1 for a missing, malformed, wrong-version or
+ * wrong-size file or one with sections this build does not take (slot_load's -1, model.mm:700-714). */
+int esp_slot_file_save(const char* path, int32_t len, int32_t next_pos, int32_t n_blocks, int32_t n_layers, uint64_t block_bytes,
+                       const void* kv);
+int esp_slot_file_info(const char* path, int32_t bt, int32_t* len, int32_t* next_pos, int32_t* n_blocks, int32_t* n_layers,
+                       uint64_t* block_bytes);
+int esp_slot_file_load(const char* path, int32_t bt, void* kv, uint64_t kv_bytes);
 /* kv_row_table (src/model/impl/forest.h:1737-1749): the pass's save records as one int32[4] per row,
  * (block, position, block2, position2), -1 none - the row_table argument of esp_attn_prep.
  * out: 4 * max(rows, 1) ints. Fails on a row saved into more than two slots. Needs no engine. */

@@ -85,3 +85,69 @@ def test_time_next_brackets_the_attention_kernel_only():
     torch.cuda.synchronize()
     us = a.elapsed_time(b) * 1e3
     assert 1.0 < us < 200.0, us
+
+
+def test_slot_checkpoint_round_trip_through_a_file(tmp_path):
+    """save -> load -> attention (src/model/model.mm:629-752): the blocks of a slot leave the native pool in the
+    reference's block layout, logical order, layer-major; loaded into other blocks of another pool they give
+    the same attention output bit for bit, and the file's payload is the checker's reference-layout pool."""
+    from espetero_amd import host
+    from gpu_utils import dev_u16, to_host_u16
+    device.init(0)
+    n_layers = 2
+    cases = [synth.make_case("slot", 20 + l, 8, 2, 128, abi.ESP_F16, 16, [(333, 1)], rows_per_tile=1) for l in range(n_layers)]
+    c0 = cases[0]
+    p = c0.params
+    nb = (333 + 15) // 16
+    blocks = np.asarray(c0.blocks[:nb], np.int32)
+    blk = 2 * p.bt * p.kv_ld
+    region = c0.n_blocks * blk
+    # a two-layer pool: layer l's region holds case l's blocks (same block ids in both layers, as in the reference)
+    ref = np.zeros(n_layers * region, np.uint16)
+    for l, c in enumerate(cases):
+        assert c.n_blocks == c0.n_blocks
+        dst = ref[l * region:(l + 1) * region].reshape(c0.n_blocks, blk)
+        dst[blocks] = c.pool_ref.reshape(c.n_blocks, blk)[c.blocks[:nb]]     # logical block i lives in block blocks[i] of every layer
+    pool = torch.zeros(n_layers * region, dtype=torch.int16, device="cuda")
+    for l in range(n_layers):
+        device.kv_relayout(p, dev_u16(ref[l * region:(l + 1) * region]), abi.ESP_LAYOUT_REFERENCE,
+                           pool[l * region:(l + 1) * region], abi.ESP_LAYOUT_NATIVE, c0.n_blocks)
+    # export, layer-major
+    out = torch.zeros(n_layers, nb, blk, dtype=torch.int16, device="cuda")
+    bd = dev_u16(blocks.view(np.uint16)).view(torch.int32)
+    for l in range(n_layers):
+        p.kv_base = l * region
+        device.kv_export_blocks(p, pool, bd, nb, out[l])
+    torch.cuda.synchronize()
+    payload = to_host_u16(out)
+    for l in range(n_layers):                                   # == the checker's blocks in logical order
+        want = ref[l * region:(l + 1) * region].reshape(c0.n_blocks, blk)[blocks]
+        assert np.array_equal(payload[l], want)
+    path = tmp_path / "slot.ckpt"
+    host.slot_file_save(path, 333, 333, n_layers, payload)
+    got = host.slot_file_load(path, p.bt)
+    assert got is not None and got["len"] == 333 and got["n_blocks"] == nb and got["n_layers"] == n_layers
+    # import into other blocks of a fresh pool
+    new_blocks = np.random.default_rng(3).permutation(c0.n_blocks).astype(np.int32)[:nb]
+    pool2 = torch.zeros_like(pool)
+    nbd = dev_u16(new_blocks.view(np.uint16)).view(torch.int32)
+    kv = got["kv"].view(np.uint16).reshape(n_layers, nb, blk)
+    for l in range(n_layers):
+        p.kv_base = l * region
+        device.kv_import_blocks(p, dev_u16(kv[l]), nbd, nb, pool2)
+    torch.cuda.synchronize()
+    # attention per layer over the original and the reloaded slot
+    resident, groups = device.plan_hint(p)
+    for l, c in enumerate(cases):
+        p.kv_base = l * region
+        tiles, jobs, n_parts = host.plan_tiles(c.trees, groups, 0, None, host.options_mi355x(1, resident))
+        Q, Kb, Vb = dev_u16(c.Q), dev_u16(c.Kb), dev_u16(c.Vb)
+        outs = []
+        for pl, bl in ((pool, blocks), (pool2, new_blocks)):
+            dp = device.DevicePass(p, c.trees, tiles, jobs, n_parts, c.n_rows, bl, None, None)
+            O = torch.zeros_like(Q)
+            dp.run(Q, Kb, Vb, pl, O)
+            torch.cuda.synchronize()
+            outs.append(O)
+        assert torch.equal(outs[0], outs[1]) and bool(outs[0].any())
+    p.kv_base = 0

@@ -311,3 +311,45 @@ def test_open_ended_marks_exactly_the_ranges_that_end_at_the_cached_length():
     assert (opened["k1"][last] == 2**31 - 1).all() and (opened["k1"][~last] == tiles["k1"][~last]).all()
     for f in ("tree", "r0", "k0", "part", "last", "b0", "pad"):
         assert (opened[f] == tiles[f]).all()
+
+
+def test_slot_file_round_trip_layout_and_refusals(tmp_path):
+    """The reference's checkpoint format, KV section (src/model/model.mm:600-752): 120-byte header with magic
+    0x554b5043 and version 4, then the blocks layer-major; a file of the wrong size, version or with
+    sections of other subsystems is refused (slot_load's -1, :700-714)."""
+    import struct
+    rng = np.random.default_rng(6)
+    n_layers, n_blocks, bt, kvw = 3, 5, 16, 2 * 128
+    kv = rng.integers(0, 65536, (n_layers, n_blocks, 2 * bt * kvw), dtype=np.uint16)
+    path = tmp_path / "slot.ckpt"
+    host.slot_file_save(path, 70, 70, n_layers, kv)
+    raw = path.read_bytes()
+    assert len(raw) == 120 + kv.nbytes
+    magic, version, length, next_pos = struct.unpack_from("<IIii", raw, 0)
+    assert (magic, version, length, next_pos) == (0x554B5043, 4, 70, 70)
+    assert struct.unpack_from("<iii", raw, 36) == (n_blocks, n_layers, 0)          # n_blocks, n_layers, n_linear
+    assert struct.unpack_from("<Q", raw, 48)[0] == 2 * bt * kvw * 2                # block_bytes
+    assert raw[120:] == kv.tobytes()                                               # layer-major, logical order
+    got = host.slot_file_load(path, bt)
+    assert (got["len"], got["next_pos"], got["n_blocks"], got["n_layers"]) == (70, 70, n_blocks, n_layers)
+    assert np.array_equal(got["kv"].view(np.uint16).reshape(kv.shape), kv)
+    # refusals
+    assert host.slot_file_load(tmp_path / "missing.ckpt", bt) is None
+    (tmp_path / "short.ckpt").write_bytes(raw[:-2])
+    assert host.slot_file_load(tmp_path / "short.ckpt", bt) is None
+    bad = bytearray(raw)
+    struct.pack_into("<I", bad, 4, 3)                                              # another version
+    (tmp_path / "v3.ckpt").write_bytes(bytes(bad))
+    assert host.slot_file_load(tmp_path / "v3.ckpt", bt) is None
+    bad = bytearray(raw)
+    struct.pack_into("<i", bad, 44, 2)                                             # n_linear: state of other layers follows
+    (tmp_path / "lin.ckpt").write_bytes(bytes(bad))
+    assert host.slot_file_load(tmp_path / "lin.ckpt", bt) is None
+    bad = bytearray(raw)
+    struct.pack_into("<i", bad, 8, n_blocks * bt + 1)                              # more tokens than the blocks hold
+    (tmp_path / "len.ckpt").write_bytes(bytes(bad))
+    assert host.slot_file_load(tmp_path / "len.ckpt", bt) is None
+    # an empty slot is a header alone
+    host.slot_file_save(tmp_path / "empty.ckpt", 0, 0, n_layers, np.zeros((n_layers, 0, 2 * bt * kvw), np.uint16))
+    e = host.slot_file_load(tmp_path / "empty.ckpt", bt)
+    assert e["n_blocks"] == 0 and (tmp_path / "empty.ckpt").stat().st_size == 120
