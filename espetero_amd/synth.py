@@ -170,7 +170,7 @@ def make_prep(kind, H, Hkv, HD, dtype, n_rows, seed=0, bt=16, max_pos=40000):
     return p, a
 
 
-# ---- the benchmark shapes (BASELINE configs), with a shrink factor for tests ----
+# ---- the five benchmark shapes, with a shrink factor for tests ----
 def c1_single_decode(ctx=1024):
     return make_case("c1_single_decode", 1, 32, 4, 128, abi.ESP_F16, 16, [(ctx, 1)], rows_per_tile=1)
 
