@@ -213,11 +213,39 @@ class ChunkedPrefill:
             d.kv_save(self.params, self.Kb[rows], self.Vb[rows], self.pool, saves, rows.stop - rows.start)
 
 
+class LayerMix:
+    """Six consecutive attention layers of the sliding + global model: five with the 1024-token window,
+    one with full attention, as one step (decode or prefill shape)."""
+
+    launches_per_step = 6
+
+    def __init__(self, name, sliding, full):
+        self.name, self.sliding, self.full = name, sliding, full
+        for k in ("bound", "dtype", "H", "Hkv", "HD", "bt", "seqs", "n_rows", "params", "n_sets", "torch", "device"):
+            setattr(self, k, getattr(full, k))
+        self.window = sliding.window
+        self.tiles = list(sliding.tiles) * 5 + list(full.tiles)
+        self.n_parts = 5 * sliding.n_parts + full.n_parts
+        self.pool_pages = sliding.pool_pages + full.pool_pages
+        self.alg_bytes = 5 * sliding.alg_bytes + full.alg_bytes
+        self.alg_flops = 5 * sliding.alg_flops + full.alg_flops
+        self.O = full.O
+
+    def step(self, i, ev=None):
+        for l in range(6):
+            w = self.full if l == 5 else self.sliding
+            w.step(6 * i + l, ev[l] if ev else None)
+
+
 def make_workload(name, workgroups=None, contiguous=False, page=16):
     from espetero_amd import abi, synth
     from functools import partial
     F16, BF16 = abi.ESP_F16, abi.ESP_BF16
     Workload_ = partial(Workload, workgroups=workgroups, contiguous=contiguous)
+    if name in ("c4_decode_mix", "c4_prefill_mix"):   # the 5 : 1 layer mix of config 4 as one step
+        kind = name[3:-4]
+        return LayerMix(name, make_workload(f"c4_{kind}_sliding", workgroups, contiguous, page),
+                        make_workload(f"c4_{kind}_global", workgroups, contiguous, page))
     if name == "c3_chunked_prefill":   # the whole of config 3 as one step
         return ChunkedPrefill(name, bt=page, workgroups=workgroups)
     if name == "c3_attn_prep":   # the rows of one C3 prefill chunk, Qwen3-Omni arrangement (82_qwen3_omni.metal:30-88)
@@ -261,7 +289,7 @@ def measured_traffic(workload):
 
 WORKLOADS = ["c1_single_decode", "c2_batched_decode", "c3_prefill_p0", "c3_prefill_p2048", "c3_prefill_p4096",
              "c3_prefill_p6144", "c4_decode_sliding", "c4_decode_global", "c4_prefill_sliding", "c4_prefill_global",
-             "c5_verify", "c3_chunked_prefill", "c3_attn_prep", "c4_attn_prep"]
+             "c5_verify", "c4_decode_mix", "c4_prefill_mix", "c3_chunked_prefill", "c3_attn_prep", "c4_attn_prep"]
 
 
 def cpu_baseline(w, budget_s=20.0):
@@ -523,6 +551,8 @@ def main():
             out["cpu_baseline"] = prep_cpu_baseline(w)
         elif isinstance(w, ChunkedPrefill):
             out["cpu_baseline"] = chunked_cpu_baseline(w)
+        elif isinstance(w, LayerMix):
+            out["cpu_baseline"] = cpu_baseline(w.full)   # the full-attention layer of the mix
         else:
             out["cpu_baseline"] = cpu_baseline(w)
     print(json.dumps(out), flush=True)
