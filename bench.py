@@ -155,6 +155,44 @@ class PrepWorkload:
                               self.Q, self.Kb, self.Vb, self.table, self.pool, self.n_rows)
 
 
+class GateWorkload:
+    """esp_head_gate over the rows of one prefill pass: O *= sigmoid(x . Wg[h]) in place (the reference's
+    form), or with dots_only the fp32 dots alone, which the attention's own epilogue then applies."""
+
+    kernel = "head_gate_kernel"
+
+    def __init__(self, name, H, HD, D, dtype, n_rows, dots_only=False, seed=9):
+        import torch
+        from espetero_amd import abi, device, synth
+        self.torch, self.device = torch, device
+        self.name, self.bound, self.dtype = name, "hbm", dtype
+        self.H, self.Hkv, self.HD, self.bt, self.window = H, H, HD, 0, 0
+        self.seqs, self.n_rows, self.tiles, self.n_parts, self.pool_pages = [(0, n_rows)], n_rows, [], 0, 0
+        self.dots_only = dots_only
+        p, a = synth.make_gate(H, HD, D, dtype, n_rows, seed=seed)
+        self.params, self.host = p, a
+        tdt = torch.float16 if dtype == abi.ESP_F16 else torch.bfloat16
+        dev = lambda x: torch.from_numpy(np.ascontiguousarray(x).view(np.int16)).cuda().view(tdt)  # noqa: E731
+        self.n_sets = 4   # rotation sets of X and O so that a step never finds its input in a cache
+        g = torch.Generator(device="cuda")
+        g.manual_seed(seed)
+        mk = lambda *sh: (torch.randn(*sh, generator=g, device="cuda") * 0.5).to(tdt)  # noqa: E731
+        self.X = [dev(a["X"])] + [mk(n_rows, p.x_ld) for _ in range(self.n_sets - 1)]
+        self.Os = [dev(a["O"])] + [mk(n_rows, p.q_ld) for _ in range(self.n_sets - 1)]
+        self.O = self.Os[0]
+        self.Wg = dev(a["Wg"])
+        self.dots = torch.zeros(n_rows, H, dtype=torch.float32, device="cuda")
+        self.alg_bytes = n_rows * D * 2 + H * D * 2 + (n_rows * H * 4 if dots_only else 2 * n_rows * H * HD * 2)
+        self.alg_flops = 0
+
+    def step(self, i, ev=None):
+        if ev:
+            self.device.time_next(ev[0], ev[1])
+        k = i % self.n_sets
+        self.device.head_gate(self.params, None if self.dots_only else self.Os[k], self.X[k], self.Wg,
+                              self.dots if self.dots_only else None, self.n_rows)
+
+
 class ChunkedPrefill:
     """One sequence of 8192 tokens in four 2048-token chunks against the paged cache: chunk c attends to
     the 2048 c cached tokens and causally to itself, then its K / V rows are appended (esp_kv_save).
@@ -252,6 +290,8 @@ def make_workload(name, workgroups=None, contiguous=False, page=16):
         return PrepWorkload(name, "omni", 40, 8, 128, BF16, 2048, bt=page)
     if name == "c4_attn_prep":   # the rows of one C4 prefill pass, Qwen3.5 arrangement (40_attention.metal:9-102)
         return PrepWorkload(name, "qwen35", 16, 8, 256, F16, 8 * 1024, bt=page)
+    if name in ("c4_head_gate", "c4_head_gate_dots"):   # the rows of one C4 prefill pass; model width 2560 (assumed: a 4B Spark)
+        return GateWorkload(name, 16, 256, 2560, F16, 8 * 1024, dots_only=name.endswith("dots"))
     if name == "c1_single_decode":
         return Workload_(name, 32, 4, 128, F16, page, [(1024, 1)], pool_pages=(64 * 16) * 16 // page, seed=1)
     if name == "c2_batched_decode":
@@ -289,7 +329,8 @@ def measured_traffic(workload):
 
 WORKLOADS = ["c1_single_decode", "c2_batched_decode", "c3_prefill_p0", "c3_prefill_p2048", "c3_prefill_p4096",
              "c3_prefill_p6144", "c4_decode_sliding", "c4_decode_global", "c4_prefill_sliding", "c4_prefill_global",
-             "c5_verify", "c4_decode_mix", "c4_prefill_mix", "c3_chunked_prefill", "c3_attn_prep", "c4_attn_prep"]
+             "c5_verify", "c4_decode_mix", "c4_prefill_mix", "c3_chunked_prefill", "c3_attn_prep", "c4_attn_prep",
+             "c4_head_gate", "c4_head_gate_dots"]
 
 
 def cpu_baseline(w, budget_s=20.0):
@@ -403,6 +444,26 @@ def prep_cpu_baseline(w):
     return {"value": round(w.alg_bytes * rows / w.n_rows / dt / 1e9, 6), "unit": "GB/s", "cores": 1, "kind": "port",
             "sample": f"{rows} of {w.n_rows} rows, {dt:.2f} s single-threaded", "host_cpus": os.cpu_count(),
             "max_abs_err_vs_gpu": err}
+
+
+def gate_cpu_baseline(w):
+    """The CPU checker's head gate on rows of rotation set 0, single-threaded, against a fresh GPU run on the same rows."""
+    import torch
+    from oracle import binding as ob
+    a, p = w.host, w.params
+    rows = min(w.n_rows, 1024)
+    t0 = time.perf_counter()
+    want, want_dots = ob.head_gate(p, a["O"][:rows], a["X"][:rows], a["Wg"], rows, want_dots=True)
+    dt = time.perf_counter() - t0
+    O = torch.from_numpy(np.ascontiguousarray(a["O"][:rows]).view(np.int16)).cuda()
+    w.device.head_gate(p, O, w.X[0], w.Wg, w.dots, rows)
+    torch.cuda.synchronize()
+    f = lambda b: ob.to_f32(b, p.dtype).astype(np.float64)  # noqa: E731
+    err = float(np.abs(f(O.cpu().numpy().view(np.uint16)) - f(want)).max())
+    derr = float(np.abs(w.dots[:rows].cpu().numpy() - want_dots).max())
+    return {"value": round(w.alg_bytes * rows / w.n_rows / dt / 1e9, 6), "unit": "GB/s", "cores": 1, "kind": "port",
+            "sample": f"{rows} of {w.n_rows} rows, {dt:.2f} s single-threaded", "host_cpus": os.cpu_count(),
+            "max_abs_err_vs_gpu": err, "max_abs_dot_err_vs_gpu": derr}
 
 
 def chunked_cpu_baseline(w, rows=24):
@@ -520,7 +581,9 @@ def main():
     kern_min_ms = float(np.min(per_step))
 
     if w.bound == "hbm":
-        metric, unit = ("attn-prep HBM GB/s" if isinstance(w, PrepWorkload) else "decode-attn HBM GB/s"), "GB/s"
+        metric = ("attn-prep HBM GB/s" if isinstance(w, PrepWorkload) else
+                  "head-gate HBM GB/s" if isinstance(w, GateWorkload) else "decode-attn HBM GB/s")
+        unit = "GB/s"
         value = w.alg_bytes / wall / 1e9
         achieved, peak = w.alg_bytes / (kern_ms * 1e-3) / 1e9, HBM_PEAK_GBS
     else:
@@ -549,6 +612,8 @@ def main():
         torch.cuda.synchronize()
         if isinstance(w, PrepWorkload):
             out["cpu_baseline"] = prep_cpu_baseline(w)
+        elif isinstance(w, GateWorkload):
+            out["cpu_baseline"] = gate_cpu_baseline(w)
         elif isinstance(w, ChunkedPrefill):
             out["cpu_baseline"] = chunked_cpu_baseline(w)
         elif isinstance(w, LayerMix):

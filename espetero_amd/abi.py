@@ -40,7 +40,7 @@ class AttnParams(C.Structure):
                 ("q_ld", C.c_int32), ("kv_ld", C.c_int32), ("bt", C.c_int32), ("window", C.c_int32),
                 ("ring", C.c_int32), ("bidi", C.c_int32), ("rows_per_tile", C.c_int32), ("scale", C.c_float),
                 ("kv_base", C.c_uint64), ("gate", C.c_void_p), ("gate_ld", C.c_int32), ("gate_hs", C.c_int32),
-                ("gate_off", C.c_int32), ("reserved", C.c_int32)]
+                ("gate_off", C.c_int32), ("gate_headwise", C.c_int32)]
 
 
 class PrepParams(C.Structure):
@@ -49,6 +49,11 @@ class PrepParams(C.Structure):
                 ("v_off", C.c_int32), ("q_ld", C.c_int32), ("kv_ld", C.c_int32), ("rope_dims", C.c_int32),
                 ("v_norm", C.c_int32), ("bt", C.c_int32), ("eps", C.c_float), ("q_scale", C.c_float),
                 ("kv_base", C.c_uint64)]
+
+
+class GateParams(C.Structure):
+    _fields_ = [("H", C.c_int32), ("head_dim", C.c_int32), ("D", C.c_int32), ("dtype", C.c_int32),
+                ("q_ld", C.c_int32), ("x_ld", C.c_int32)]
 
 
 TREE_DT = np.dtype([("base", "<i4"), ("P", "<i4"), ("table", "<i4"), ("M", "<i4")])
@@ -63,6 +68,7 @@ assert C.sizeof(Combine) == COMBINE_DT.itemsize == 16
 assert C.sizeof(KVSave) == KVSAVE_DT.itemsize == 16
 assert C.sizeof(AttnParams) == 80
 assert C.sizeof(PrepParams) == 72
+assert C.sizeof(GateParams) == 24
 
 # name -> (restype, argtypes); every symbol the header declares.
 _P = C.POINTER(AttnParams)
@@ -84,6 +90,7 @@ ATTN_SYMBOLS = {
     "esp_kv_export_blocks": (C.c_int, (_P, _V, _V, C.c_int32, _V, _V) + _ERR),
     "esp_kv_import_blocks": (C.c_int, (_P, _V, _V, C.c_int32, _V, _V) + _ERR),
     "esp_chain_advance": (C.c_int, (_V, C.c_int32, _V, _V, _V, C.c_int32, C.c_int32, _V) + _ERR),
+    "esp_head_gate": (C.c_int, (C.POINTER(GateParams), _V, _V, _V, _V, C.c_int32, _V) + _ERR),
     "esp_attn_prep": (C.c_int, (C.POINTER(PrepParams), _V, _V, _V, _V, _V, _V, _V, _V, _V, _V, _V, C.c_int32, _V) + _ERR),
 }
 

@@ -22,6 +22,7 @@ hipError_t launch_chain_advance(esp_tree* trees, int n_trees, int32_t* pos, int3
                                 int ring, hipStream_t st);
 hipError_t launch_vt_stage(const esp_attn_params* p, const void* Vb, void* vt, int n_rows, hipStream_t st);
 hipError_t launch_attn_prep(const PrepArgs& a, int n_rows, hipStream_t st);
+hipError_t launch_head_gate(int dt, const GateArgs& a, hipStream_t st);
 int stream_workgroups_per_cu(int HD, int NC);
 int tiled_workgroups_per_cu(int HD);
 int tiled_max_rows(int HD);
@@ -54,6 +55,7 @@ int check_params(const esp_attn_params* p, char* err, size_t errlen) {
   if (p->kv_ld < p->Hkv * p->head_dim || p->kv_ld % 8) return fail(err, errlen, ESP_EINVAL, "kv_ld %d", p->kv_ld);
   if (p->kv_base % 8) return fail(err, errlen, ESP_EINVAL, "kv_base must be a multiple of 8 elements");
   if (p->window < 0 || p->ring < 0) return fail(err, errlen, ESP_EINVAL, "window / ring negative");
+  if (p->gate_headwise != 0 && p->gate_headwise != 1) return fail(err, errlen, ESP_EINVAL, "gate_headwise %d (0 or 1)", p->gate_headwise);
   return ESP_OK;
 }
 
@@ -93,6 +95,7 @@ esp::KArgs make_args(const esp_attn_params* p, const Carve& c, void* workspace, 
   a.gate_ld = p->gate_ld;
   a.gate_hs = p->gate_hs;
   a.gate_off = p->gate_off;
+  a.gate_ds = p->gate_headwise ? 0 : 1;
   a.H = p->H;
   a.Hkv = p->Hkv;
   a.G = p->H / p->Hkv;
@@ -319,6 +322,30 @@ int esp_chain_advance(esp_tree* trees, int32_t n_trees, int32_t* pos, int32_t* r
   if (row_table && !ring && !blocks) return fail(err, errlen, ESP_EINVAL, "blocks is NULL on a layer without rings");
   const hipError_t e = esp::launch_chain_advance(trees, n_trees, pos, row_table, blocks, bt, ring, static_cast<hipStream_t>(stream));
   if (e != hipSuccess) return hip_fail(err, errlen, "chain_advance launch", e);
+  return ESP_OK;
+}
+
+int esp_head_gate(const esp_gate_params* p, void* O, const void* X, const void* Wg, float* dots, int32_t n_rows,
+                  void* stream, char* err, size_t errlen) {
+  if (!p) return fail(err, errlen, ESP_EINVAL, "params is NULL");
+  if (p->H <= 0 || p->H > 64) return fail(err, errlen, p->H <= 0 ? ESP_EINVAL : ESP_EUNSUPPORTED, "H=%d (1 .. 64)", p->H);
+  if (p->head_dim <= 0 || p->head_dim % 8 || p->head_dim > 1024)
+    return fail(err, errlen, ESP_EINVAL, "head_dim %d: a multiple of 8, at most 1024", p->head_dim);
+  if (p->D <= 0 || p->D % 8) return fail(err, errlen, ESP_EINVAL, "D %d: a positive multiple of 8", p->D);
+  if (p->dtype != ESP_F16 && p->dtype != ESP_BF16) return fail(err, errlen, ESP_EINVAL, "dtype %d", p->dtype);
+  if (p->x_ld < p->D || p->x_ld % 8) return fail(err, errlen, ESP_EINVAL, "x_ld %d", p->x_ld);
+  if (O && (p->q_ld < p->H * p->head_dim || p->q_ld % 8)) return fail(err, errlen, ESP_EINVAL, "q_ld %d", p->q_ld);
+  if (n_rows < 0) return fail(err, errlen, ESP_EINVAL, "negative count");
+  if (!O && !dots) return fail(err, errlen, ESP_EINVAL, "neither O nor dots");
+  if (n_rows == 0) return ESP_OK;
+  if (!X || !Wg) return fail(err, errlen, ESP_EINVAL, "X and Wg must not be NULL");
+  int shift = -1;
+  for (int s = 3; s <= 10; ++s)
+    if (p->head_dim == 1 << s) shift = s;
+  esp::GateArgs a{static_cast<uint16_t*>(O), static_cast<const uint16_t*>(X), static_cast<const uint16_t*>(Wg), dots,
+                  n_rows, p->H, p->head_dim, shift, p->D, p->q_ld, p->x_ld};
+  const hipError_t e = esp::launch_head_gate(p->dtype, a, static_cast<hipStream_t>(stream));
+  if (e != hipSuccess) return hip_fail(err, errlen, "head_gate launch", e);
   return ESP_OK;
 }
 

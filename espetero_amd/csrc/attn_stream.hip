@@ -397,9 +397,9 @@ __global__ __launch_bounds__(256, OCC) void attn_stream_kernel(const KArgs a) {
       const float inv = L > 0.0f ? 1.0f / L : 0.0f;
       o *= inv;
       if (a.gate) {
-        const float* g = a.gate + size_t(row) * a.gate_ld + size_t(h) * a.gate_hs + a.gate_off + d;
+        const float* g = a.gate + size_t(row) * a.gate_ld + size_t(h) * a.gate_hs + a.gate_off + d * a.gate_ds;
 #pragma unroll
-        for (int e = 0; e < 4; ++e) o[e] = o[e] / (1.0f + __expf(-g[e]));
+        for (int e = 0; e < 4; ++e) o[e] = o[e] / (1.0f + __expf(-g[e * a.gate_ds]));
       }
       u32x2 out = {pack2<DT>(o[0], o[1]), pack2<DT>(o[2], o[3])};
       *reinterpret_cast<u32x2*>(a.O + size_t(row) * a.q_ld + size_t(h) * HD + d) = out;
@@ -460,9 +460,9 @@ __global__ __launch_bounds__(256) void attn_combine_kernel(const KArgs a, const 
   const float inv = L > 0.0f ? 1.0f / L : 0.0f;
   o *= inv;
   if (a.gate) {
-    const float* g = a.gate + size_t(row) * a.gate_ld + size_t(h) * a.gate_hs + a.gate_off + d;
+    const float* g = a.gate + size_t(row) * a.gate_ld + size_t(h) * a.gate_hs + a.gate_off + d * a.gate_ds;
 #pragma unroll
-    for (int e = 0; e < 4; ++e) o[e] = o[e] / (1.0f + __expf(-g[e]));
+    for (int e = 0; e < 4; ++e) o[e] = o[e] / (1.0f + __expf(-g[e * a.gate_ds]));
   }
   u32x2 out = {pack2<DT>(o[0], o[1]), pack2<DT>(o[2], o[3])};
   *reinterpret_cast<u32x2*>(a.O + size_t(row) * a.q_ld + size_t(h) * HD + d) = out;

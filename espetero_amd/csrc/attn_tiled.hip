@@ -594,7 +594,7 @@ __global__ __launch_bounds__(256, OCC) void attn_tiled_kernel(const KArgs a, int
 #pragma unroll
       for (int j = 0; j < 4; ++j) {
         o[j] = acc[nt][4 * i4 + j] * inv;
-        if (gp) o[j] = o[j] / (1.0f + __expf(-gp[dd + j]));
+        if (gp) o[j] = o[j] / (1.0f + __expf(-gp[(dd + j) * a.gate_ds]));
       }
       *reinterpret_cast<u32x2*>(op + dd) = u32x2{pack2<DT>(o[0], o[1]), pack2<DT>(o[2], o[3])};
     }

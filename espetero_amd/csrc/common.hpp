@@ -97,7 +97,7 @@ struct KArgs {
   float* parts_ml;  // [part][Hkv][cols][2]    running max (log2 units), sum
   uint16_t* vt_stage;  // batch V transposed: [Hkv][n_rows16 / 16][HD][16]
   const float* gate;
-  int32_t gate_ld, gate_hs, gate_off;
+  int32_t gate_ld, gate_hs, gate_off, gate_ds;  // gate_ds: 1 per-dim gates, 0 one gate per head
   int32_t H, Hkv, G, q_ld, kv_ld, bt, window, ring, bidi, R, cols, n_rows;
   float scale_log2;
   uint64_t kv_base;
@@ -129,6 +129,15 @@ struct PrepArgs {
   const int4* row_table;
   uint16_t* pool;
   esp_prep_params p;
+};
+
+// Everything the head gate kernel reads (esp_head_gate).
+struct GateArgs {
+  uint16_t* O;
+  const uint16_t* X;
+  const uint16_t* Wg;
+  float* dots;
+  int32_t n_rows, H, hd, hd_shift, D, q_ld, x_ld;  // hd_shift: log2(hd), -1 when hd is no power of two
 };
 
 // Events the next attention kernel launch records its own begin and end into (esp_attn_time_next);

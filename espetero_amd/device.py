@@ -125,6 +125,13 @@ def attn_prep(params, X, qn_w, kn_w, pos, inv_freq, rope_sel, Q, Kb, Vb, row_tab
                                            _stream(stream), err, _ERRLEN), err)
 
 
+def head_gate(params, O, X, Wg, dots, n_rows, stream=None):
+    """Device tensors. O (gated in place) or dots (fp32 [n_rows][H], written) may be None, not both."""
+    err = C.create_string_buffer(_ERRLEN)
+    abi.check(abi.attn_lib().esp_head_gate(C.byref(params), _ptr(O), _ptr(X), _ptr(Wg), _ptr(dots), n_rows,
+                                           _stream(stream), err, _ERRLEN), err)
+
+
 def chain_advance(trees, n_trees, pos, row_table, blocks, bt, ring=0, stream=None):
     """Device tensors: trees (TREE_DT bytes), pos / row_table int32 [rows][4], blocks int32."""
     err = C.create_string_buffer(_ERRLEN)

@@ -170,6 +170,23 @@ def make_prep(kind, H, Hkv, HD, dtype, n_rows, seed=0, bt=16, max_pos=40000):
     return p, a
 
 
+def make_gate(H, HD, D, dtype, n_rows, seed=0, q_ld=None, x_ld=None):
+    """Inputs of one esp_head_gate call (sp_head_gate, kernels/85_spark.metal:96-128): O as an
+    attention leaves it, the layer's normed input X and the gate rows Wg, as storage bits.
+    Wg ~ N(0, 1) * 2 / sqrt(D) puts the dots at about N(0, 1): gates across the whole sigmoid."""
+    rng = np.random.default_rng(seed)
+    p = abi.GateParams()
+    p.H, p.head_dim, p.D, p.dtype = H, HD, D, dtype
+    p.q_ld = q_ld or H * HD
+    p.x_ld = x_ld or D
+    a = dict(
+        O=_bits(rng.standard_normal((n_rows, p.q_ld), dtype=np.float32) * 0.5, dtype),
+        X=_bits(rng.standard_normal((n_rows, p.x_ld), dtype=np.float32) * 0.5, dtype),
+        Wg=_bits(rng.standard_normal((H, D), dtype=np.float32) * (2.0 / np.sqrt(D)), dtype),
+    )
+    return p, a
+
+
 # ---- the five benchmark shapes, with a shrink factor for tests ----
 def c1_single_decode(ctx=1024):
     return make_case("c1_single_decode", 1, 32, 4, 128, abi.ESP_F16, 16, [(ctx, 1)], rows_per_tile=1)

@@ -109,7 +109,9 @@ typedef struct esp_attn_params {
   int32_t gate_ld;       /* gate[row * gate_ld + h * gate_hs + gate_off + d] */
   int32_t gate_hs;
   int32_t gate_off;
-  int32_t reserved;
+  int32_t gate_headwise; /* 1: one gate value per (row, head), the address above without "+ d": the
+                            head-wise gate of 85_spark.metal:96-128 taken into the output's one
+                            rounding, its dots computed before the pass by esp_head_gate */
 } esp_attn_params;
 
 /* Library / device check. Safe to call more than once. */
@@ -268,6 +270,31 @@ int esp_attn_prep(const esp_prep_params* p, const float* X, const float* qn_w, c
  * blocks: device memory. Trees with M != 1 are not meant for it. */
 int esp_chain_advance(esp_tree* trees, int32_t n_trees, int32_t* pos, int32_t* row_table, const int32_t* blocks, int32_t bt,
                       int32_t ring, void* stream, char* err, size_t errlen);
+
+/* ---- the head-wise output gate: the step after the attention of a layer ----------
+ * sp_head_gate (kernels/85_spark.metal:96-128, SpGateParams :99-104; binding
+ * src/model/impl/gemma.h:481-492): O[row, h, :] *= sigmoid(x[row] . Wg[h]) with x the layer's
+ * normed input and Wg = g_proj, one gate per (row, query head). The reference runs one
+ * threadgroup per (head, row) after the attention and rounds O a second time. Two ways here:
+ *   - O != NULL: as the reference, in place: O = storage(float(O) * gate), dots NULL or not;
+ *   - dots != NULL: the pre-activation dots x . Wg[h] as fp32 [n_rows][H], to be handed to
+ *     the attention as params.gate with gate_headwise = 1 (gate_ld = H, gate_hs = 1,
+ *     gate_off = 0): the attention then multiplies before its one rounding and O makes no
+ *     second trip through memory. This call can run before the attention (x is the layer's input).
+ * At least one of O and dots. X [n_rows][x_ld], Wg [H][D], O [n_rows][q_ld]: storage type
+ * (the reference: fp16). D % 8 == 0 (the reference: % 4), head_dim % 8 == 0 and <= 1024
+ * as in the reference (:98), H <= 64. */
+typedef struct esp_gate_params {
+  int32_t H;        /* query heads */
+  int32_t head_dim; /* SpGateParams.hd */
+  int32_t D;        /* model width: length of the dots */
+  int32_t dtype;    /* ESP_F16 | ESP_BF16 */
+  int32_t q_ld;     /* O row stride, elements (SpGateParams.q_ld) */
+  int32_t x_ld;     /* X row stride, elements (the reference: D) */
+} esp_gate_params;
+
+int esp_head_gate(const esp_gate_params* p, void* O, const void* X, const void* Wg, float* dots, int32_t n_rows,
+                  void* stream, char* err, size_t errlen);
 
 #ifdef __cplusplus
 }

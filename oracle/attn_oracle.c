@@ -31,6 +31,16 @@
  *                            scale, value cast / weightless norm, folded append
  *                            into the reference-layout pool 40_:86-100).
  *
+ *   esp_oracle_head_gate     sp_head_gate 85_spark.metal:108-128: the fp32 dot of the
+ *                            row's input with the head's gate row, the sigmoid, and
+ *                            O rounded a second time after the product.
+ *
+ * esp_oracle_head_gate is pinned in tests/test_gate.py by closed forms (x == 0 halves
+ * O exactly, a one-hot gate row gives sigmoid of one input element, a saturated
+ * dot leaves O or clears it) and by a float64 restatement; its summation order
+ * (left to right) is not the reference's (strided partial sums, 85_:121-122), so
+ * gates agree to fp32 rounding and outputs to one unit in the last place.
+ *
  * esp_oracle_attn_prep is pinned by a float64 restatement of the closed forms
  * (RMSNorm, rotation matrix) in tests/test_prep.py, by norm preservation of the
  * rotation, by position 0 == no rotation, and by the folded append == kv_save of
@@ -146,7 +156,7 @@ static inline int cached_visible(const esp_attn_params* p, const int32_t* pos, i
 
 static inline float gate_of(const esp_attn_params* p, int row, int h, int d) {
   if (!p->gate) return 1.0f;
-  const float g = p->gate[(size_t)row * p->gate_ld + (size_t)h * p->gate_hs + p->gate_off + d];
+  const float g = p->gate[(size_t)row * p->gate_ld + (size_t)h * p->gate_hs + p->gate_off + (p->gate_headwise ? 0 : d)];
   return 1.0f / (1.0f + expf(-g));
 }
 
@@ -434,4 +444,23 @@ void esp_oracle_attn_prep(const esp_prep_params* p, const float* X, const float*
   }
   free(x);
   free(y);
+}
+
+/* ---- sp_head_gate ---- */
+void esp_oracle_head_gate(const esp_gate_params* p, uint16_t* O, const uint16_t* X, const uint16_t* Wg, float* dots, int n_rows) {
+  for (int row = 0; row < n_rows; ++row)
+    for (int h = 0; h < p->H; ++h) {
+      const uint16_t* x = X + (size_t)row * p->x_ld;
+      const uint16_t* w = Wg + (size_t)h * p->D;
+      float acc = 0.0f;
+      for (int i = 0; i < p->D; ++i)
+        acc += (p->dtype == ESP_F16 ? esp_oracle_h2f(x[i]) : esp_oracle_bf2f(x[i])) *
+               (p->dtype == ESP_F16 ? esp_oracle_h2f(w[i]) : esp_oracle_bf2f(w[i]));
+      if (dots) dots[(size_t)row * p->H + h] = acc;
+      if (!O) continue;
+      const float g = 1.0f / (1.0f + expf(-acc));
+      uint16_t* o = O + (size_t)row * p->q_ld + (size_t)h * p->head_dim;
+      for (int d = 0; d < p->head_dim; ++d)
+        o[d] = st_dt(p->dtype, (p->dtype == ESP_F16 ? esp_oracle_h2f(o[d]) : esp_oracle_bf2f(o[d])) * g);
+    }
 }

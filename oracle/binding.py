@@ -116,6 +116,25 @@ def attn_prep(params, X, qn_w, kn_w, pos, inv_freq, rope_sel, n_rows, row_table=
     return Q, Kb, Vb
 
 
+def head_gate(params, O, X, Wg, n_rows, want_dots=False):
+    """sp_head_gate on storage bits: returns the gated copy of O (None when O is None) and, if asked, the fp32 dots."""
+    out = None if O is None else np.array(_u16(O), copy=True)
+    dots = np.zeros((n_rows, params.H), np.float32) if want_dots else None
+    lib().esp_oracle_head_gate(C.byref(params), _p(out), _p(_u16(X)), _p(_u16(Wg)), _p(dots), C.c_int(n_rows))
+    return (out, dots) if want_dots else out
+
+
+def head_gate_f64(params, O, X, Wg, n_rows):
+    """The closed form in float64, no second rounding: float(O) * sigmoid(x . Wg[h]); also returns the dots."""
+    x = to_f32(np.asarray(X)[:, :params.D], params.dtype).astype(np.float64)
+    w = to_f32(np.asarray(Wg), params.dtype).astype(np.float64).reshape(params.H, params.D)
+    dots = x @ w.T
+    g = 1.0 / (1.0 + np.exp(-dots))
+    o = to_f32(np.asarray(O)[:, :params.H * params.head_dim], params.dtype).astype(np.float64)
+    o = o.reshape(n_rows, params.H, params.head_dim) * g[:, :, None]
+    return o, dots
+
+
 def attn_prep_f64(params, X, qn_w, kn_w, pos, inv_freq, rope_sel, n_rows):
     """The closed forms in float64, no storage rounding: RMSNorm x / sqrt(mean x^2 + eps) * w, the rotation
     [[c, -s], [s, c]] on each pair (d, d + rope_dims / 2) by angle position * inv_freq, the query scale.
