@@ -482,11 +482,11 @@ static hipError_t launch_stream_t(const KArgs& a, int n_tiles, hipStream_t st) {
   constexpr int SBU = HD == 128 ? 2 : 1;
   constexpr int NBUF = stream_nbuf(HD, NC), OCC = stream_occ(HD, NC);
   const size_t smem = stream_smem_bytes(HD, NC);
-  auto k = a.bt == 16 ? attn_stream_kernel<DT, HD, NC, SBU, NBUF, 16, OCC> : attn_stream_kernel<DT, HD, NC, SBU, NBUF, 0, OCC>;
-  if (smem > 48 * 1024) {
-    hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(k), hipFuncAttributeMaxDynamicSharedMemorySize, int(smem));
-    if (e != hipSuccess) return e;
-  }
+  constexpr auto k16 = attn_stream_kernel<DT, HD, NC, SBU, NBUF, 16, OCC>;
+  constexpr auto kbt = attn_stream_kernel<DT, HD, NC, SBU, NBUF, 0, OCC>;
+  const auto k = a.bt == 16 ? k16 : kbt;
+  const hipError_t e = a.bt == 16 ? allow_dynamic_lds<k16>(smem) : allow_dynamic_lds<kbt>(smem);
+  if (e != hipSuccess) return e;
   launch_timed(k, dim3(a.Hkv, n_tiles), dim3(256), smem, st, a);
   return hipGetLastError();
 }

@@ -609,11 +609,9 @@ size_t tiled_smem_bytes(int HD) { return size_t(4) * 64 * HD * 2 + 64; }  // two
 template <int DT, int HD>
 static hipError_t launch_tiled_t(const KArgs& a, int n_tiles, hipStream_t st) {
   const size_t smem = tiled_smem_bytes(HD);
-  auto k = attn_tiled_kernel<DT, HD, tiled_occ(HD)>;
-  if (smem > 48 * 1024) {
-    hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(k), hipFuncAttributeMaxDynamicSharedMemorySize, int(smem));
-    if (e != hipSuccess) return e;
-  }
+  constexpr auto k = attn_tiled_kernel<DT, HD, tiled_occ(HD)>;
+  const hipError_t e = allow_dynamic_lds<k>(smem);
+  if (e != hipSuccess) return e;
   launch_timed(k, dim3(unsigned(n_tiles) * a.H), dim3(256), smem, st, a, n_tiles);
   return hipGetLastError();
 }

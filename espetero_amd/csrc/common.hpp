@@ -7,6 +7,8 @@
 #include <hip/hip_ext.h>
 #include <stdint.h>
 
+#include <atomic>
+
 #include "../../include/espetero_attn.h"
 
 namespace esp {
@@ -146,6 +148,22 @@ struct TimeNext {
   hipEvent_t start = nullptr, stop = nullptr;
 };
 TimeNext take_time_next();  // returns the pair and clears it
+
+// Raises a kernel's dynamic LDS limit above the 48 KB default, once per device: the attribute
+// belongs to the function on that device and stays for the life of the process.
+template <auto Kern>
+inline hipError_t allow_dynamic_lds(size_t bytes) {
+  if (bytes <= 48 * 1024) return hipSuccess;
+  static std::atomic<uint64_t> done{0};  // one bit per device ordinal
+  int dev = 0;
+  hipError_t e = hipGetDevice(&dev);
+  if (e != hipSuccess) return e;
+  const uint64_t bit = uint64_t(1) << (dev & 63);
+  if (dev < 64 && (done.load(std::memory_order_acquire) & bit)) return hipSuccess;
+  e = hipFuncSetAttribute(reinterpret_cast<const void*>(Kern), hipFuncAttributeMaxDynamicSharedMemorySize, int(bytes));
+  if (e == hipSuccess && dev < 64) done.fetch_or(bit, std::memory_order_release);
+  return e;
+}
 
 // Launches k; with a pending event pair the launch itself timestamps the kernel's begin and end.
 template <typename K, typename... Args>

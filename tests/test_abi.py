@@ -73,3 +73,34 @@ def test_argument_errors_come_back_as_codes_not_crashes():
     rc = lib.esp_attn_forward(C.byref(p), None, None, None, None, None, None, None, None, None, 1, None, 1, None, 0, 0, 1,
                               None, 0, None, err, 256)
     assert rc == 1 and b"must not be NULL" in err.value
+
+
+def test_prep_gate_and_chain_argument_errors():
+    """The entry points beside the attention refuse bad arguments on the host too."""
+    from espetero_amd import synth
+    lib = abi.attn_lib()
+    err = C.create_string_buffer(256)
+    g, _ = synth.make_gate(16, 256, 2560, abi.ESP_F16, 1)
+    assert lib.esp_head_gate(C.byref(g), None, None, None, None, 4, None, err, 256) == 1 and b"neither O nor dots" in err.value
+    g.H = 65
+    assert lib.esp_head_gate(C.byref(g), None, None, None, None, 4, None, err, 256) == 2 and b"1 .. 64" in err.value
+    g.H, g.D = 16, 2564
+    assert lib.esp_head_gate(C.byref(g), None, None, None, None, 4, None, err, 256) == 1 and b"multiple of 8" in err.value
+    g.D, g.head_dim = 2560, 2048
+    assert lib.esp_head_gate(C.byref(g), None, None, None, None, 4, None, err, 256) == 1 and b"at most 1024" in err.value
+    g.head_dim = 256
+    dots = (C.c_float * 64)()
+    assert lib.esp_head_gate(C.byref(g), None, None, None, dots, 0, None, err, 256) == 0           # nothing to do
+    assert lib.esp_head_gate(C.byref(g), None, None, None, dots, 4, None, err, 256) == 1 and b"X and Wg" in err.value
+    p, _ = synth.make_prep("gemma", 8, 2, 128, abi.ESP_F16, 1)
+    p.rope_dims = 48
+    assert lib.esp_attn_prep(C.byref(p), None, None, None, None, None, None, None, None, None, None, None, 1, None, err, 256) == 1
+    assert b"power of two" in err.value
+    p.rope_dims, p.x_ld = 128, 100
+    assert lib.esp_attn_prep(C.byref(p), None, None, None, None, None, None, None, None, None, None, None, 1, None, err, 256) == 1
+    assert lib.esp_chain_advance(None, 3, None, None, None, 16, 0, None, err, 256) == 1 and b"trees and pos" in err.value
+    assert lib.esp_chain_advance(None, 0, None, None, None, 16, 0, None, err, 256) == 0
+    a = synth.make_params(32, 4, 128, abi.ESP_F16, 16)
+    a.gate_headwise = 2
+    assert lib.esp_attn_forward(C.byref(a), None, None, None, None, None, None, None, None, None, 1, None, 1, None, 0, 0, 1,
+                                None, 0, None, err, 256) == 1 and b"gate_headwise" in err.value
