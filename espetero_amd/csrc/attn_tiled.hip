@@ -212,10 +212,9 @@ __global__ __launch_bounds__(256, OCC) void attn_tiled_kernel(const KArgs a, int
   const int r0 = lane / CH;
   const uint32_t kcol0 = uint32_t(((lane % CH) ^ r0) << 4);
   // cached keys: rows HD elements apart, i.e. instruction q's rows start 1024 q bytes further; that part
-  // travels in the instruction's immediate offset
-  uint32_t koff_c[KP];
-#pragma unroll
-  for (int q = 0; q < KP; ++q) koff_c[q] = uint32_t(r0 * ROWB) + (kcol0 ^ uint32_t(swap23(q * RPI) << 4));
+  // travels in the instruction's immediate offset. Instruction q's lane offset is
+  // r0 ROWB + (kcol0 ^ kswz(q)); fill() derives it where it is used.
+  auto kswz = [](int q) constexpr { return uint32_t(swap23(q * RPI) << 4); };
   // V^T instruction q covers dims 32 q ..: this lane brings keys 8 (lane / 32) .. + 7 of dim 32 q + lane % 32.
   const uint32_t voff_c = uint32_t(l32 * a.bt * 2 + hb * 16);
   const uint32_t voff_b = uint32_t(l32 * 32 + hb * 16);
@@ -225,6 +224,12 @@ __global__ __launch_bounds__(256, OCC) void attn_tiled_kernel(const KArgs a, int
     const int s = 4 * step + wave;
     const uint32_t kdst = lds_base + stage * KBUF + wave * (16 * ROWB);
     const uint32_t vdst = lds_base + VOFF + stage * VBUF + wave * SUBV;
+    // The per-instruction lane offsets are derived here, in every call, from two registers. Computed
+    // once in front of the loops (which the compiler does with anything loop-invariant, hence the
+    // empty asm) they would occupy a register each for the whole kernel and end up in scratch
+    // memory, whose reloads wait on the same counter as the staging loads and serialise them.
+    uint32_t kc = kcol0, kr = uint32_t(r0);
+    asm volatile("" : "+v"(kc), "+v"(kr));
     if (decltype(interior)::value || s < n_c) {
       const int js = (c0 + s) << 4;
       const int b = block_id(step);
@@ -233,9 +238,11 @@ __global__ __launch_bounds__(256, OCC) void attn_tiled_kernel(const KArgs a, int
       const char* kb = hbp + size_t(t0) * ROWB;
       const char* vb = hbp + (size_t(a.bt) * HD + t0) * 2;
       const size_t vstep = size_t(64) * a.bt;  // 32 V^T rows of bt elements
+      const uint32_t kro = kr * ROWB;
 #pragma unroll
       for (int q = 0; q < KP; q += 4)
-        load_to_lds16_x4(kb + q * 1024, koff_c[q], koff_c[q + 1], koff_c[q + 2], koff_c[q + 3], kdst + q * 1024);
+        load_to_lds16_x4(kb + q * 1024, kro + (kc ^ kswz(q)), kro + (kc ^ kswz(q + 1)), kro + (kc ^ kswz(q + 2)),
+                         kro + (kc ^ kswz(q + 3)), kdst + q * 1024);
       if (a.bt == 16) {  // 32 V^T rows of 16 tokens are 1024 bytes as well
 #pragma unroll
         for (int q = 0; q < VP; q += 4) load_to_lds16_x4(vb + q * 1024, voff_c, voff_c, voff_c, voff_c, vdst + q * 1024);
@@ -245,13 +252,19 @@ __global__ __launch_bounds__(256, OCC) void attn_tiled_kernel(const KArgs a, int
       }
     } else if (s < n_sb) {
       const int g = a0 + (s - n_c);
-      const int lim = min(15, a.n_rows - 1 - 16 * g);  // batch rows past the pass's last row do not exist
+      const int lim = a.n_rows - 1 - 16 * g;  // batch rows past the pass's last row do not exist
       const char* kb = reinterpret_cast<const char*>(a.Kb + size_t(16 * g) * a.kv_ld + size_t(kvh) * HD);
       const char* vb = reinterpret_cast<const char*>(a.vt_stage + (size_t(kvh) * n_groups + g) * size_t(HD) * 16);
       const uint32_t kld = uint32_t(a.kv_ld) * 2;
+      if (lim >= 15) {  // all 16 rows exist: instruction q's rows start q RPI rows further, which goes into its base
+        const uint32_t kro = kr * kld;
 #pragma unroll
-      for (int q = 0; q < KP; ++q)
-        load_to_lds16(kb, uint32_t(min(q * RPI + r0, lim)) * kld + (kcol0 ^ uint32_t(swap23(q * RPI) << 4)), kdst + q * 1024);
+        for (int q = 0; q < KP; ++q) load_to_lds16(kb + size_t(q * RPI) * kld, kro + (kc ^ kswz(q)), kdst + q * 1024);
+      } else {  // the pass's last group: rows past the end repeat the last one (their scores are masked)
+#pragma unroll
+        for (int q = 0; q < KP; ++q)
+          load_to_lds16(kb, uint32_t(min(q * RPI + int(kr), lim)) * kld + (kc ^ kswz(q)), kdst + q * 1024);
+      }
 #pragma unroll
       for (int q = 0; q < VP; q += 4) load_to_lds16_x4(vb + q * 1024, voff_b, voff_b, voff_b, voff_b, vdst + q * 1024);
     } else {  // past the range: K stays whatever it was (S is masked), V^T must be finite
