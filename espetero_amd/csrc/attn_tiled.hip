@@ -131,6 +131,7 @@ __global__ __launch_bounds__(256, OCC) void attn_tiled_kernel(const KArgs a, int
 
   // ---- tile-wide facts about the rows (for the batch range and the no-mask fast path)
   int k_last = -1, seg_max = 0, qpos_max = 0;
+  bool anc_any = false;  // does any row of the tile see ancestors (keys below its segment)?
   {
     int kl = -1, sm = 0, am = 0, qm = INT32_MIN;
     if (row_ok) {
@@ -167,6 +168,7 @@ __global__ __launch_bounds__(256, OCC) void attn_tiled_kernel(const KArgs a, int
     anc_max = __builtin_amdgcn_readfirstlane(anc_max);
     qpos_max = __builtin_amdgcn_readfirstlane(qpos_max);
     if (anc_max > 0 || a.bidi) seg_max = INT32_MAX;  // rows that see beyond the causal rule: always mask
+    anc_any = anc_max > 0;
   }
 
   // ---- the key range as 16-key sub-blocks: cached [k0, k1), then batch rows [b0, k_last]
@@ -404,12 +406,25 @@ __global__ __launch_bounds__(256, OCC) void attn_tiled_kernel(const KArgs a, int
           lo = 1;
           hi = 0;
         }
+        // In units of this lane's 8 keys (j = jb + e): e in [ea, ea + ew], one unsigned compare per key;
+        // an empty interval becomes ea = 8, ew = 0, which no e in 0 .. 7 satisfies.
+        const int jb = j0 + 8 * hb;
+        int ea = lo - jb, ew = hi - lo;
+        if (ew < 0) {
+          ea = 8;
+          ew = 0;
+        }
+        if (batch && (anc_any || batch_window)) {  // ancestors, per-key positions: the rare shapes
 #pragma unroll
-        for (int e = 0; e < 8; ++e) {
-          const int j = j0 + 8 * hb + e;
-          bool vis = (j >= lo && j <= hi) || (j >= 0 && j < anc);
-          if (batch && batch_window && vis) vis = qpos - a.pos[tree.base + j].x < a.window;
-          sv[8 * t + e] = vis ? sv[8 * t + e] : -INFINITY;
+          for (int e = 0; e < 8; ++e) {
+            const int j = jb + e;
+            bool vis = unsigned(e - ea) <= unsigned(ew) || (j >= 0 && j < anc);
+            if (batch_window && vis) vis = qpos - a.pos[tree.base + j].x < a.window;
+            sv[8 * t + e] = vis ? sv[8 * t + e] : -INFINITY;
+          }
+        } else {
+#pragma unroll
+          for (int e = 0; e < 8; ++e) sv[8 * t + e] = unsigned(e - ea) <= unsigned(ew) ? sv[8 * t + e] : -INFINITY;
         }
       }
     }
