@@ -78,6 +78,9 @@ __device__ __forceinline__ void load_to_lds16_x4(const void* base, uint32_t o0, 
 }
 __device__ __forceinline__ void wait_loads() { asm volatile("s_waitcnt vmcnt(0)" ::: "memory"); }
 
+// s_waitcnt immediates (gfx9 layout): only the LDS / scalar-memory counter, at most 8 or 0 outstanding.
+constexpr int kWaitLgkm8 = 0xC07F | (8 << 8), kWaitLgkm0 = 0xC07F;
+
 constexpr int swap23(int x) { return (x & ~12) | ((x & 4) << 1) | ((x & 8) >> 1); }
 
 template <int DT, int HD, int OCC>
@@ -302,8 +305,14 @@ __global__ __launch_bounds__(256, OCC) void attn_tiled_kernel(const KArgs a, int
   {
     const int prow = (l32 & 0x13) | ((l32 & 4) << 1) | ((l32 & 8) >> 1);  // pi(l32)
 #pragma unroll
-    for (int ks = 0; ks < KS; ++ks) kaddr[ks] = uint32_t(prow * ROWB + (((2 * ks + hb) ^ (l32 & 15)) << 4));
+    for (int ks = 0; ks < KS; ++ks) kaddr[ks] = lds_base + uint32_t(prow * ROWB + (((2 * ks + hb) ^ (l32 & 15)) << 4));
   }
+
+  const uint32_t vaddr = lds_base + uint32_t(VOFF + lane * 16);  // the V^T stages start at VOFF: immediates stay below 64 KB
+  // Operand reads take LDS byte addresses (base register + immediate): stage, half step and operand
+  // number are compile-time parts of the immediate, so no address arithmetic is issued in the loop.
+  using lds_u32x4 = const __attribute__((address_space(3))) u32x4;
+  auto lds_ptr = [](uint32_t addr) __attribute__((always_inline)) { return reinterpret_cast<lds_u32x4*>(addr); };
 
   f32x16 acc[NT];
   float m_run = -INFINITY, l_run = 0.0f;  // l_run: this lane's share (16 of every 32 keys) of the row's sum
@@ -336,16 +345,15 @@ __global__ __launch_bounds__(256, OCC) void attn_tiled_kernel(const KArgs a, int
   auto read_group = [&]<int S, int G>(u32x4 (&buf)[GP]) __attribute__((always_inline)) {
     if constexpr (G < 2 * GK) {
       constexpr int kt = G / GK, ks0 = (G % GK) * GP;
-      const char* kp = lds + S * KBUF + kt * 32 * ROWB;
 #pragma unroll
-      for (int j = 0; j < GP; ++j) buf[j] = *reinterpret_cast<const u32x4*>(kp + kaddr[ks0 + j]);
+      for (int j = 0; j < GP; ++j) buf[j] = *lds_ptr(kaddr[ks0 + j] + uint32_t(S * KBUF + kt * 32 * ROWB));
     } else {
       // Operand o = 2 nt + t of half step kt: keys 8 hb .. 8 hb + 7 of sub-block 2 kt + t, dims 32 nt .. : the
       // lane's 16 bytes of that sub-block's dim group.
       constexpr int kt = (G - 2 * GK) / GK, o0 = ((G - 2 * GK) % GK) * GP;
-      const char* vp = lds + VOFF + S * VBUF + 2 * kt * SUBV + lane * 16;
 #pragma unroll
-      for (int j = 0; j < GP; ++j) buf[j] = *reinterpret_cast<const u32x4*>(vp + ((o0 + j) & 1) * SUBV + ((o0 + j) >> 1) * 1024);
+      for (int j = 0; j < GP; ++j)
+        buf[j] = *lds_ptr(vaddr + uint32_t(S * VBUF + 2 * kt * SUBV + ((o0 + j) & 1) * SUBV + ((o0 + j) >> 1) * 1024));
     }
   };
   // Operands [J0, J1) of group G.
@@ -479,6 +487,10 @@ __global__ __launch_bounds__(256, OCC) void attn_tiled_kernel(const KArgs a, int
   // Q K^T finished with the previous group.
   auto phase = [&]<int S, int G>(int step, auto interior) __attribute__((always_inline)) {
     if constexpr (G + 1 < NG) read_group.template operator()<S, G + 1>(ring[(G + 1) & 1]);
+    // One wait for the whole group (its GP reads went out a group ago; the GP just issued stay in
+    // flight) instead of one in front of every matrix instruction: at one wavefront per SIMD every
+    // issued instruction, a wait included, is time the matrix pipe idles.
+    __builtin_amdgcn_s_waitcnt(G + 1 < NG ? kWaitLgkm8 : kWaitLgkm0);
     if constexpr (G == GK || G == 2 * GK) {
       // The first matrix instructions of the group go out before the branchy part of the softmax,
       // whose wait for the previous group's results they cover; the rest carry the arithmetic,
@@ -534,6 +546,7 @@ __global__ __launch_bounds__(256, OCC) void attn_tiled_kernel(const KArgs a, int
     __syncthreads();
     if (decltype(interior)::value || i + 2 < n_steps) fill(i + 2, S, interior);
     read_group.template operator()<S ^ 1, 0>(ring[0]);
+    __builtin_amdgcn_s_waitcnt(kWaitLgkm8);
     __builtin_amdgcn_sched_barrier(0);
     mma_group.template operator()<NG - 1, 0, GP>(ring[(NG - 1) & 1]);
     __builtin_amdgcn_sched_barrier(0);
