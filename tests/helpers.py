@@ -36,3 +36,26 @@ def brute(case):
     c = case
     H, HD = c.params.H, c.params.head_dim
     return ob.brute_force(c.params, c.Q, c.Kb, c.Vb, c.pool_ref, c.blocks, c.desc, c.pos, c.trees).reshape(c.n_rows, H * HD)
+
+
+GOLDEN = __import__("os").path.join(__import__("os").path.dirname(__import__("os").path.abspath(__file__)), "golden")
+
+
+def golden_names(prefix):
+    import os
+    return sorted(f[len(prefix) + 1:-4] for f in os.listdir(GOLDEN) if f.startswith(prefix + "_") and f.endswith(".npz"))
+
+
+def load_golden_attention(name):
+    """A committed attention fixture as (Case, expected O float64 [n_rows][H * head_dim])."""
+    import json
+    import os
+    z = np.load(os.path.join(GOLDEN, f"attention_{name}.npz"), allow_pickle=False)
+    m = json.loads(str(z["meta"]))
+    p = synth.make_params(m["H"], m["Hkv"], m["head_dim"], m["dtype"], m["bt"], window=m["window"], ring=m["ring"],
+                          scale=m["scale"], rows_per_tile=m["rows_per_tile"], bidi=m["bidi"])
+    trees = np.ascontiguousarray(z["trees"]).view(abi.TREE_DT).reshape(-1)
+    seqs = [(int(t["P"]), int(t["M"])) for t in trees]
+    case = synth.Case(name, p, z["Q"], z["Kb"], z["Vb"], z["pool_ref"], m["n_blocks"], z["blocks"], trees, z["desc"], z["pos"],
+                      m["n_rows"], dict(seqs=seqs, seed=None))
+    return case, z["O"]
