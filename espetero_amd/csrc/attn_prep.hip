@@ -74,7 +74,8 @@ __global__ __launch_bounds__(256) void attn_prep_kernel(const PrepArgs a, int n_
     f32x4 xv[R];
 #pragma unroll
     for (int r = 0; r < R; ++r)
-      xv[r] = r < rows ? *reinterpret_cast<const f32x4*>(a.X + size_t(row0 + r) * p.x_ld + col) : f32x4{0, 0, 0, 0};
+      xv[r] = r < rows ? __builtin_nontemporal_load(reinterpret_cast<const f32x4*>(a.X + size_t(row0 + r) * p.x_ld + col))
+                       : f32x4{0, 0, 0, 0};  // read once: no reason to keep it in a cache
     f32x4 w = {1, 1, 1, 1};
     if (kind != 2) w = *reinterpret_cast<const f32x4*>((kind == 0 ? a.qn_w : a.kn_w) + d0);
 #pragma unroll

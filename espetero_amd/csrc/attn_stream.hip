@@ -20,6 +20,8 @@
 // merge their (m, l, O) through LDS in wave order at the end. Each wavefront
 // keeps a ring of register sets: the loads of the next units are in flight
 // while the current unit is in the matrix cores.
+#include <type_traits>
+
 #include "common.hpp"
 
 namespace esp {
@@ -123,10 +125,12 @@ __global__ __launch_bounds__(256, OCC) void attn_stream_kernel(const KArgs a) {
       const uint16_t* vp = valid ? hb + bt * HD + t0 + lane_v : a.Q;
       const int ks = valid ? 32 : 0;
       const int vs = valid ? 16 * bt : 0;
+      // Every cached byte is read once per pass: non-temporal loads keep the stream from displacing
+      // what the caches could still serve (measured: 184 -> 164 us on 1 GB of keys at head dim 256).
 #pragma unroll
-      for (int kk = 0; kk < KK; ++kk) U.k[sb][kk] = *reinterpret_cast<const u32x4*>(kp + ks * kk);
+      for (int kk = 0; kk < KK; ++kk) U.k[sb][kk] = __builtin_nontemporal_load(reinterpret_cast<const u32x4*>(kp + ks * kk));
 #pragma unroll
-      for (int mt = 0; mt < MT; ++mt) U.v[sb][mt] = *reinterpret_cast<const u32x2*>(vp + vs * mt);
+      for (int mt = 0; mt < MT; ++mt) U.v[sb][mt] = __builtin_nontemporal_load(reinterpret_cast<const u32x2*>(vp + vs * mt));
     }
   };
 
@@ -431,30 +435,37 @@ __global__ __launch_bounds__(256) void attn_combine_kernel(const KArgs a, const 
   // measured 39 us against 11 us for the same change, 40_attention.metal:801-803).
   float M = -INFINITY, L = 0.0f;
   f32x4 o = {0, 0, 0, 0};
-  for (int s = 0; s < job.nparts; s += 8) {
-    float m8[8], l8[8];
-    f32x4 o8[8];
+  // N records at a time, all their loads issued before the first use. Slots past the last record
+  // repeat record s (a cache hit) with weight 0: loads under a branch would wait for one another.
+  auto merge = [&]<int N>(int s, std::integral_constant<int, N>) __attribute__((always_inline)) {
+    float mN[N], lN[N];
+    f32x4 oN[N];
 #pragma unroll
-    for (int i = 0; i < 8; ++i) {
+    for (int i = 0; i < N; ++i) {
       const bool in = s + i < job.nparts;
       const size_t rec = rec0 + size_t(in ? s + i : s) * stride;
-      m8[i] = in ? a.parts_ml[rec * 2] : -INFINITY;
-      l8[i] = a.parts_ml[rec * 2 + 1];
-      o8[i] = *reinterpret_cast<const f32x4*>(a.parts_o + rec * HD + d);
+      mN[i] = in ? a.parts_ml[rec * 2] : -INFINITY;
+      lN[i] = a.parts_ml[rec * 2 + 1];
+      oN[i] = *reinterpret_cast<const f32x4*>(a.parts_o + rec * HD + d);
     }
     float Mn = M;
 #pragma unroll
-    for (int i = 0; i < 8; ++i) Mn = fmaxf(Mn, m8[i]);
+    for (int i = 0; i < N; ++i) Mn = fmaxf(Mn, mN[i]);
     const float c = (M == -INFINITY) ? 0.0f : fast_exp2(M - Mn);
     L *= c;
     o *= c;
     M = Mn;
 #pragma unroll
-    for (int i = 0; i < 8; ++i) {
-      const float w = (m8[i] == -INFINITY) ? 0.0f : fast_exp2(m8[i] - M);
-      L += w * l8[i];
-      o += o8[i] * w;
+    for (int i = 0; i < N; ++i) {
+      const float w = (mN[i] == -INFINITY) ? 0.0f : fast_exp2(mN[i] - M);
+      L += w * lN[i];
+      o += oN[i] * w;
     }
+  };
+  if (job.nparts <= 2) {  // the split of a prefill tile: two records, nothing to repeat
+    merge(0, std::integral_constant<int, 2>{});
+  } else {
+    for (int s = 0; s < job.nparts; s += 8) merge(s, std::integral_constant<int, 8>{});
   }
   const int row = job.r0 + r;
   const float inv = L > 0.0f ? 1.0f / L : 0.0f;
