@@ -19,7 +19,7 @@
 // (rope_dims / 2 entries each) are computed once per workgroup into LDS and shared
 // by its heads: the reference computes them once per (row, head).
 // The folded append writes K rows as they are. V lies transposed in the pool
-// (tokens contiguous per dim): when the 8 rows go to 8 consecutive, 8-aligned
+// (16-token sub-blocks, tokens contiguous per dim): when the 8 rows go to 8 consecutive, 8-aligned
 // positions of one block - every full group of a prefill chunk - their V is
 // staged in LDS and leaves as one 16-byte store per (head, dim); any other
 // arrangement (decode rows of different sequences, a row saved into two slots)
@@ -127,24 +127,24 @@ __global__ __launch_bounds__(256) void attn_prep_kernel(const PrepArgs a, int n_
         if (kind == 1) {
           *reinterpret_cast<u32x2*>(hb + size_t(ps) * HD + d0) = out;
         } else {
-          uint16_t* vt = hb + size_t(p.bt) * HD + size_t(d0) * p.bt + ps;
+          uint16_t* vt = hb + vt_elem(p.bt, HD, ps, d0);
           vt[0] = uint16_t(out[0] & 0xffffu);
-          vt[p.bt] = uint16_t(out[0] >> 16);
-          vt[2 * p.bt] = uint16_t(out[1] & 0xffffu);
-          vt[3 * p.bt] = uint16_t(out[1] >> 16);
+          vt[kVtDim] = uint16_t(out[0] >> 16);
+          vt[2 * kVtDim] = uint16_t(out[1] & 0xffffu);
+          vt[3 * kVtDim] = uint16_t(out[1] >> 16);
         }
       }
     }
   }
   if (!run) return;
   __syncthreads();
-  // 8 tokens of one (head, dim): 16 contiguous bytes of the transposed V plane.
+  // 8 tokens of one (head, dim): 16 contiguous bytes inside one 16-token sub-block of the transposed V plane.
   for (int i = tid; i < HPP * HD; i += 256) {
     const int slot = slot0 + i / HD, d = i % HD;
     if (slot < p.H + p.Hkv || slot >= n_slots) continue;  // not a value head
     const int h = slot - p.H - p.Hkv;
     uint16_t* hb = a.pool + p.kv_base + (size_t(ent[0].x) * p.Hkv + h) * size_t(2 * p.bt * HD);
-    uint16_t* dst = hb + size_t(p.bt) * HD + size_t(d) * p.bt + ent[0].y;
+    uint16_t* dst = hb + vt_elem(p.bt, HD, ent[0].y, d);
 #pragma unroll
     for (int g = 0; g < R / 8; ++g) {
       u32x4 v;

@@ -112,7 +112,7 @@ __global__ __launch_bounds__(256, OCC) void attn_stream_kernel(const KArgs a) {
   // in flight is the same on every path and the hardware load counter can be waited
   // on exactly. A sub-block past the range's last page re-reads that page.
   const int last_js = (max(tile.k1, tile.k0 + 1) - 1) & ~15;
-  const int lane_k = (c16 * HD + 8 * q4), lane_v = c16 * bt + 4 * q4;
+  const int lane_k = (c16 * HD + 8 * q4), lane_v = c16 * kVtDim + 4 * q4;
   auto load_cached = [&](int u, Unit<HD, SBU>& U, const bool valid) {
     const int j0 = (valid ? u : cp0) << USH;
 #pragma unroll
@@ -122,9 +122,9 @@ __global__ __launch_bounds__(256, OCC) void attn_stream_kernel(const KArgs a) {
       const int t0 = js % bt;
       const uint16_t* hb = a.pool + head_base(a, HD, b, kvh);
       const uint16_t* kp = valid ? hb + t0 * HD + lane_k : a.Q;
-      const uint16_t* vp = valid ? hb + bt * HD + t0 + lane_v : a.Q;
+      const uint16_t* vp = valid ? hb + vt_elem(bt, HD, t0, 0) + lane_v : a.Q;  // t0 is a multiple of 16: the sub-block's start
       const int ks = valid ? 32 : 0;
-      const int vs = valid ? 16 * bt : 0;
+      const int vs = valid ? 16 * kVtDim : 0;
       // Every cached byte is read once per pass: non-temporal loads keep the stream from displacing
       // what the caches could still serve (measured: 184 -> 164 us on 1 GB of keys at head dim 256).
 #pragma unroll

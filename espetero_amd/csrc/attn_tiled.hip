@@ -221,8 +221,8 @@ __global__ __launch_bounds__(256, OCC) void attn_tiled_kernel(const KArgs a, int
   // r0 ROWB + (kcol0 ^ kswz(q)); fill() derives it where it is used.
   auto kswz = [](int q) constexpr { return uint32_t(swap23(q * RPI) << 4); };
   // V^T instruction q covers dims 32 q ..: this lane brings keys 8 (lane / 32) .. + 7 of dim 32 q + lane % 32.
-  const uint32_t voff_c = uint32_t(l32 * a.bt * 2 + hb * 16);
-  const uint32_t voff_b = uint32_t(l32 * 32 + hb * 16);
+  // (32 V^T rows of 16 tokens are 1024 bytes, in the pool's sub-blocks and in the staged batch rows alike)
+  const uint32_t voff = uint32_t(l32 * 32 + hb * 16);
 
   // interior: the caller knows that all four sub-blocks of the step are cached keys.
   auto fill = [&](int step, int stage, auto interior) __attribute__((always_inline)) {
@@ -241,20 +241,14 @@ __global__ __launch_bounds__(256, OCC) void attn_tiled_kernel(const KArgs a, int
       const int t0 = a.bt == 16 ? 0 : js % a.bt;
       const char* hbp = reinterpret_cast<const char*>(a.pool + head_base(a, HD, b, kvh));
       const char* kb = hbp + size_t(t0) * ROWB;
-      const char* vb = hbp + (size_t(a.bt) * HD + t0) * 2;
-      const size_t vstep = size_t(64) * a.bt;  // 32 V^T rows of bt elements
+      const char* vb = hbp + vt_elem(a.bt, HD, t0, 0) * 2;  // the 16-token sub-block: 32 HD contiguous bytes
       const uint32_t kro = kr * ROWB;
 #pragma unroll
       for (int q = 0; q < KP; q += 4)
         load_to_lds16_x4(kb + q * 1024, kro + (kc ^ kswz(q)), kro + (kc ^ kswz(q + 1)), kro + (kc ^ kswz(q + 2)),
                          kro + (kc ^ kswz(q + 3)), kdst + q * 1024);
-      if (a.bt == 16) {  // 32 V^T rows of 16 tokens are 1024 bytes as well
 #pragma unroll
-        for (int q = 0; q < VP; q += 4) load_to_lds16_x4(vb + q * 1024, voff_c, voff_c, voff_c, voff_c, vdst + q * 1024);
-      } else {
-#pragma unroll
-        for (int q = 0; q < VP; ++q) load_to_lds16(vb + q * vstep, voff_c, vdst + q * 1024);
-      }
+      for (int q = 0; q < VP; q += 4) load_to_lds16_x4(vb + q * 1024, voff, voff, voff, voff, vdst + q * 1024);
     } else if (s < n_sb) {
       const int g = a0 + (s - n_c);
       const int lim = a.n_rows - 1 - 16 * g;  // batch rows past the pass's last row do not exist
@@ -271,7 +265,7 @@ __global__ __launch_bounds__(256, OCC) void attn_tiled_kernel(const KArgs a, int
           load_to_lds16(kb, uint32_t(min(q * RPI + int(kr), lim)) * kld + (kc ^ kswz(q)), kdst + q * 1024);
       }
 #pragma unroll
-      for (int q = 0; q < VP; q += 4) load_to_lds16_x4(vb + q * 1024, voff_b, voff_b, voff_b, voff_b, vdst + q * 1024);
+      for (int q = 0; q < VP; q += 4) load_to_lds16_x4(vb + q * 1024, voff, voff, voff, voff, vdst + q * 1024);
     } else {  // past the range: K stays whatever it was (S is masked), V^T must be finite
 #pragma unroll
       for (int q = 0; q < VP; ++q)

@@ -106,9 +106,17 @@ struct KArgs {
 };
 
 // Native pool: element offset of (block b, KV head h); K rows follow at
-// t * HD + d, V transposed at bt * HD + d * bt + t.
+// t * HD + d; V follows the K rows transposed in sub-blocks of 16 tokens,
+// each [HD dims][16 tokens]: see vt_elem. A sub-block is 32 HD contiguous bytes
+// at any block size, which is what both attention kernels load per 16 keys.
 __device__ __forceinline__ size_t head_base(const KArgs& a, int HD, int b, int kvh) {
   return size_t(a.kv_base) + (size_t(b) * size_t(a.Hkv) + size_t(kvh)) * size_t(2 * a.bt * HD);
+}
+
+// Element offset of V[token t][dim d] from head_base; consecutive dims are kVtDim elements apart.
+constexpr int kVtDim = 16;
+__host__ __device__ __forceinline__ size_t vt_elem(int bt, int HD, int t, int d) {
+  return size_t(bt) * HD + size_t(t >> 4) * size_t(16 * HD) + size_t(d) * kVtDim + size_t(t & 15);
 }
 
 // Block holding cached key j of a tree: its block list, or its slot's ring.

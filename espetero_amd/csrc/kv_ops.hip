@@ -22,11 +22,11 @@ __global__ __launch_bounds__(256) void kv_save_kernel(const uint16_t* Kb, const 
   uint16_t* hb = pool + kv_base + (size_t(e.block) * Hkv + kvh) * size_t(2 * bt * HD);
   *reinterpret_cast<u32x4*>(hb + size_t(e.pos) * HD + d) = *reinterpret_cast<const u32x4*>(Kb + src);
   const u32x4 v = *reinterpret_cast<const u32x4*>(Vb + src);
-  uint16_t* vt = hb + size_t(bt) * HD + size_t(d) * bt + e.pos;
+  uint16_t* vt = hb + vt_elem(bt, HD, e.pos, d);
 #pragma unroll
   for (int i = 0; i < 4; ++i) {
-    vt[size_t(2 * i) * bt] = uint16_t(v[i] & 0xffffu);
-    vt[size_t(2 * i + 1) * bt] = uint16_t(v[i] >> 16);
+    vt[(2 * i) * kVtDim] = uint16_t(v[i] & 0xffffu);
+    vt[(2 * i + 1) * kVtDim] = uint16_t(v[i] >> 16);
   }
 }
 
@@ -53,10 +53,10 @@ __global__ __launch_bounds__(256) void kv_gather_kernel(const uint16_t* pool, co
   const int b = blocks[j / bt], t = j % bt;
   const uint16_t* hb = pool + kv_base + (size_t(b) * Hkv + kvh) * size_t(2 * bt * HD);
   *reinterpret_cast<u32x4*>(K_out + size_t(j) * Hkv * HD + x) = *reinterpret_cast<const u32x4*>(hb + size_t(t) * HD + d);
-  const uint16_t* vt = hb + size_t(bt) * HD + size_t(d) * bt + t;
+  const uint16_t* vt = hb + vt_elem(bt, HD, t, d);
   u32x4 v;
 #pragma unroll
-  for (int i = 0; i < 4; ++i) v[i] = uint32_t(vt[size_t(2 * i) * bt]) | (uint32_t(vt[size_t(2 * i + 1) * bt]) << 16);
+  for (int i = 0; i < 4; ++i) v[i] = uint32_t(vt[(2 * i) * kVtDim]) | (uint32_t(vt[(2 * i + 1) * kVtDim]) << 16);
   *reinterpret_cast<u32x4*>(V_out + size_t(j) * Hkv * HD + x) = v;
 }
 
@@ -84,18 +84,18 @@ __global__ __launch_bounds__(256) void kv_relayout_kernel(const uint16_t* src, u
     if (to_native) *reinterpret_cast<u32x4*>(dst + nat) = *reinterpret_cast<const u32x4*>(src + ref_off);
     else *reinterpret_cast<u32x4*>(dst + ref_off) = *reinterpret_cast<const u32x4*>(src + nat);
   } else {
-    const size_t nat = hb + size_t(bt) * HD + size_t(d) * bt + t;
+    const size_t nat = hb + vt_elem(bt, HD, t, d);
     if (to_native) {
       const u32x4 v = *reinterpret_cast<const u32x4*>(src + ref_off);
 #pragma unroll
       for (int i = 0; i < 4; ++i) {
-        dst[nat + size_t(2 * i) * bt] = uint16_t(v[i] & 0xffffu);
-        dst[nat + size_t(2 * i + 1) * bt] = uint16_t(v[i] >> 16);
+        dst[nat + (2 * i) * kVtDim] = uint16_t(v[i] & 0xffffu);
+        dst[nat + (2 * i + 1) * kVtDim] = uint16_t(v[i] >> 16);
       }
     } else {
       u32x4 v;
 #pragma unroll
-      for (int i = 0; i < 4; ++i) v[i] = uint32_t(src[nat + size_t(2 * i) * bt]) | (uint32_t(src[nat + size_t(2 * i + 1) * bt]) << 16);
+      for (int i = 0; i < 4; ++i) v[i] = uint32_t(src[nat + (2 * i) * kVtDim]) | (uint32_t(src[nat + (2 * i + 1) * kVtDim]) << 16);
       *reinterpret_cast<u32x4*>(dst + ref_off) = v;
     }
   }

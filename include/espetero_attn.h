@@ -26,9 +26,11 @@
  * src/model/impl/model.h:396), arranged for 64-wide wavefronts as
  *   block b, KV head h : base = kv_base + (b * Hkv + h) * 2 * bt * head_dim
  *   K[token t][dim d]  : base + t * head_dim + d                (row major)
- *   V[token t][dim d]  : base + bt * head_dim + d * bt + t      (transposed)
- * so one (block, head) is a single contiguous run and V is already the
- * k-contiguous operand of the P.V matrix product. The reference's layout
+ *   V[token t][dim d]  : base + bt * head_dim + (t / 16) * 16 * head_dim + d * 16 + t % 16
+ *                        (transposed, in sub-blocks of 16 tokens)
+ * so one (block, head) is a single contiguous run, V is already the
+ * k-contiguous operand of the P.V matrix product, and 16 keys of K or of V
+ * are 32 * head_dim contiguous bytes whatever the block size. The reference's layout
  * (ESP_LAYOUT_REFERENCE, kernels/40_attention.metal:245-247) is
  *   K/V[which][t][h][d]: kv_base + (2 b + which) * bt * kv_ld + t * kv_ld + h * head_dim + d
  * and is accepted only by esp_kv_relayout (import / export of blocks).
