@@ -8,25 +8,55 @@
 namespace esp {
 
 // kv_save (kernels/40_attention.metal:875-889): entry = (source row, block,
-// position). One thread per (entry, 8 elements of the KV row).
+// position). One workgroup per (16 consecutive entries, KV head); a thread moves 8
+// elements of a row. K rows are copied as they are. V lies transposed in 16-token
+// sub-blocks: when the 16 entries fill one sub-block in order (every full group of
+// a prefill chunk's append) their V rows meet in LDS and leave as the sub-block's
+// contiguous [HD][16] bytes; any other arrangement (decode rows of different
+// sequences, a ragged tail) stores elements.
+constexpr int kSaveRows = 16;
 __global__ __launch_bounds__(256) void kv_save_kernel(const uint16_t* Kb, const uint16_t* Vb, uint16_t* pool,
                                                       const esp_kvsave* entries, int n, int Hkv, int HD, int kv_ld, int bt,
                                                       uint64_t kv_base) {
-  const int per = Hkv * HD / 8;
-  const long gid = long(blockIdx.x) * 256 + threadIdx.x;
-  if (gid >= long(n) * per) return;
-  const esp_kvsave e = entries[gid / per];
-  const int x = int(gid % per) * 8;
-  const int kvh = x / HD, d = x % HD;
-  const size_t src = size_t(e.src_row) * kv_ld + x;
-  uint16_t* hb = pool + kv_base + (size_t(e.block) * Hkv + kvh) * size_t(2 * bt * HD);
-  *reinterpret_cast<u32x4*>(hb + size_t(e.pos) * HD + d) = *reinterpret_cast<const u32x4*>(Kb + src);
-  const u32x4 v = *reinterpret_cast<const u32x4*>(Vb + src);
-  uint16_t* vt = hb + vt_elem(bt, HD, e.pos, d);
+  constexpr int R = kSaveRows;
+  __shared__ __attribute__((aligned(16))) uint16_t vs[R][256 + 8];  // HD <= 256; the pad spreads the column reads over the banks
+  const int tid = threadIdx.x, g0 = blockIdx.x * R, kvh = blockIdx.y;
+  const int cnt = min(R, n - g0);
+  const esp_kvsave e0 = entries[g0];
+  bool mine = true;
+  if (tid < R) {
+    const esp_kvsave e = entries[g0 + min(tid, cnt - 1)];
+    mine = tid < cnt && e.block == e0.block && e.pos == e0.pos + tid;
+  }
+  const bool run = __syncthreads_and(mine) && cnt == R && (e0.pos & 15) == 0;
+  const int tpr = HD / 8;  // threads per row
+  for (int r = tid / tpr; r < cnt; r += 256 / tpr) {
+    const esp_kvsave e = entries[g0 + r];
+    const int d = (tid % tpr) * 8;
+    const size_t src = size_t(e.src_row) * kv_ld + size_t(kvh) * HD + d;
+    uint16_t* hb = pool + kv_base + (size_t(e.block) * Hkv + kvh) * size_t(2 * bt * HD);
+    *reinterpret_cast<u32x4*>(hb + size_t(e.pos) * HD + d) = *reinterpret_cast<const u32x4*>(Kb + src);
+    const u32x4 v = *reinterpret_cast<const u32x4*>(Vb + src);
+    if (run) {
+      *reinterpret_cast<u32x4*>(&vs[r][d]) = v;
+    } else {
+      uint16_t* vt = hb + vt_elem(bt, HD, e.pos, d);
 #pragma unroll
-  for (int i = 0; i < 4; ++i) {
-    vt[(2 * i) * kVtDim] = uint16_t(v[i] & 0xffffu);
-    vt[(2 * i + 1) * kVtDim] = uint16_t(v[i] >> 16);
+      for (int i = 0; i < 4; ++i) {
+        vt[(2 * i) * kVtDim] = uint16_t(v[i] & 0xffffu);
+        vt[(2 * i + 1) * kVtDim] = uint16_t(v[i] >> 16);
+      }
+    }
+  }
+  if (!run) return;
+  __syncthreads();
+  uint16_t* hb = pool + kv_base + (size_t(e0.block) * Hkv + kvh) * size_t(2 * bt * HD);
+  for (int i = tid; i < 2 * HD; i += 256) {  // (dim, half of the 16 tokens): 16 contiguous bytes of the sub-block
+    const int d = i >> 1, t8 = 8 * (i & 1);
+    u32x4 v;
+#pragma unroll
+    for (int e = 0; e < 4; ++e) v[e] = uint32_t(vs[t8 + 2 * e][d]) | (uint32_t(vs[t8 + 2 * e + 1][d]) << 16);
+    *reinterpret_cast<u32x4*>(hb + vt_elem(bt, HD, e0.pos + t8, d)) = v;
   }
 }
 
@@ -163,9 +193,9 @@ hipError_t launch_chain_advance(esp_tree* trees, int n_trees, int32_t* pos, int3
 
 hipError_t launch_kv_save(const esp_attn_params* p, const void* Kb, const void* Vb, void* pool, const esp_kvsave* e, int n,
                           hipStream_t st) {
-  const long total = long(n) * (p->Hkv * p->head_dim / 8);
-  hipLaunchKernelGGL(kv_save_kernel, dim3((unsigned)((total + 255) / 256)), dim3(256), 0, st, (const uint16_t*)Kb,
-                     (const uint16_t*)Vb, (uint16_t*)pool, e, n, p->Hkv, p->head_dim, p->kv_ld, p->bt, p->kv_base);
+  hipLaunchKernelGGL(kv_save_kernel, dim3(unsigned((n + kSaveRows - 1) / kSaveRows), unsigned(p->Hkv)), dim3(256), 0, st,
+                     (const uint16_t*)Kb, (const uint16_t*)Vb, (uint16_t*)pool, e, n, p->Hkv, p->head_dim, p->kv_ld, p->bt,
+                     p->kv_base);
   return hipGetLastError();
 }
 

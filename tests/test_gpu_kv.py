@@ -49,6 +49,14 @@ def test_relayout_gather_save_copy_are_bit_exact(HD, Hkv, bt, dtype):
                    [(3, int(table[8]), 1, 0)], abi.KVSAVE_DT)
     device.kv_save(p, dev_u16(Kb), dev_u16(Vb), nat, device.to_dev(ent), len(ent))
     ob.kv_save(p, Kb, Vb, ref, ent)
+    # a prefill-like append: 40 consecutive rows from a 16-aligned token on (two whole sub-blocks through the
+    # staged path, a ragged tail through element stores), source rows in reverse order
+    rows2 = 40
+    Kb2 = rng.integers(0, 65536, (rows2, p.kv_ld)).astype(np.uint16)
+    Vb2 = rng.integers(0, 65536, (rows2, p.kv_ld)).astype(np.uint16)
+    ent2 = np.array([(rows2 - 1 - r, int(table[(64 + r) // bt]), (64 + r) % bt, 0) for r in range(rows2)], abi.KVSAVE_DT)
+    device.kv_save(p, dev_u16(Kb2), dev_u16(Vb2), nat, device.to_dev(ent2), len(ent2))
+    ob.kv_save(p, Kb2, Vb2, ref, ent2)
     # copy on write in every layer region
     p.kv_base = 0
     pairs = np.array([(int(table[0]), int(table[8])), (int(table[2]), 23 if 23 not in table[:9] else int(table[7]))], np.int32)
