@@ -18,7 +18,7 @@
 //   O^T[HD][cols]      += V^T[HD][32] . P^T        v_mfma_f32_16x16x32 (A = V^T straight from HBM: the pool keeps V transposed)
 // with no LDS on the way. The 4 wavefronts take 32-key units round robin and
 // merge their (m, l, O) through LDS in wave order at the end. Each wavefront
-// keeps a ring of register sets: the loads of the next units are in flight
+// alternates between two register sets: the loads of the next unit are in flight
 // while the current unit is in the matrix cores.
 #include <type_traits>
 
@@ -33,9 +33,9 @@ struct Unit {  // operands of one unit of SBU 16-key sub-blocks
 };
 
 // SBU: 16-key sub-blocks per unit (2: P.V on 16x16x32 tiles; 1: on 16x16x16 tiles, for
-// head dims whose operands would not fit the register ring otherwise).
+// head dims whose operands would not fit two register sets otherwise).
 // BT: tokens per block when known at compile time (0: read from the arguments).
-template <int DT, int HD, int NC, int SBU, int NBUF, int BT, int OCC>
+template <int DT, int HD, int NC, int SBU, int BT, int OCC>
 __global__ __launch_bounds__(256, OCC) void attn_stream_kernel(const KArgs a) {
   constexpr int KK = HD / 32, MT = HD / 16, LDO = HD + 4, UK = 16 * SBU, USH = SBU == 2 ? 5 : 4;
   extern __shared__ float smem[];  // [4 waves][NC * 16 cols][LDO] O, then [4][NC * 16][2] m, l
@@ -76,25 +76,33 @@ __global__ __launch_bounds__(256, OCC) void attn_stream_kernel(const KArgs a) {
   }
 
   // ---- the cached range in units of UK keys. Interior units lie wholly inside
-  // [k0, k1) on a layer without a window: they need no masks and go through the
-  // pipelined loop. The (at most two) partial units at the ends of the range, every
-  // unit of a windowed layer, and the tree's batch rows take the general path.
+  // [k0, k1) and, on a windowed layer, wholly inside the window of every packed row:
+  // they need no masks and go through the pipelined loop. The partial units at the
+  // ends of the range, the units the window's lower edge cuts, and the tree's batch
+  // rows take the general path.
   const int cp0 = tile.k0 >> USH;
   const bool has_cached = tile.k1 > tile.k0;
   const int ulast = has_cached ? (tile.k1 - 1) >> USH : cp0 - 1;
   const int n_cached = ulast - cp0 + 1;
-  int ui0, ui1, n_edge;  // interior units [ui0, ui1)
-  bool first_edge = false, last_edge = false;
-  if (a.window > 0 || !has_cached) {
+  int ui0, ui1;  // interior units [ui0, ui1); general ones [cp0, ui0) and [ui1, ulast]
+  if (!has_cached) {
     ui0 = ui1 = cp0;
-    n_edge = n_cached;
   } else {
-    first_edge = (tile.k0 & (UK - 1)) != 0 || ((cp0 + 1) << USH) > tile.k1;
-    last_edge = (ulast != cp0 || !first_edge) && ((ulast + 1) << USH) > tile.k1;
-    ui0 = cp0 + (first_edge ? 1 : 0);
-    ui1 = ulast + 1 - (last_edge ? 1 : 0);
-    n_edge = (first_edge ? 1 : 0) + (last_edge ? 1 : 0);
+    int lo_key = tile.k0;  // first key every row sees
+    if (a.window > 0) {
+      int qm = INT32_MIN;
+#pragma unroll
+      for (int c = 0; c < NC; ++c)
+        if (ok[c]) qm = max(qm, qpos[c]);
+#pragma unroll
+      for (int o = 8; o >= 1; o >>= 1) qm = max(qm, __shfl_xor(qm, o));
+      qm = __builtin_amdgcn_readfirstlane(qm);  // the 16 columns repeat in every quarter of the wavefront
+      lo_key = max(lo_key, qm - a.window + 1);
+    }
+    ui0 = min((lo_key + UK - 1) >> USH, ulast + 1);
+    ui1 = max(ui0, tile.k1 >> USH);  // units wholly below k1
   }
+  const int n_lo = ui0 - cp0, n_edge = n_cached - (ui1 - ui0);
   int k_last = -1, bp0 = 0, n_batch = 0;  // batch range: set once the cached range has been streamed
   f32x4 acc[NC][MT];
   float m_run[NC], l_run[NC];  // running max in log2 units of the scaled score; this lane's share of the sum
@@ -107,24 +115,20 @@ __global__ __launch_bounds__(256, OCC) void attn_stream_kernel(const KArgs a) {
   }
 
   // K rows and V^T rows of cached unit u (absolute unit index) straight from the pool.
-  // Straight-line code: a unit past the wavefront's last one (valid == false) reads one
-  // 16-byte line of Q with every load instead of being skipped, so the number of loads
-  // in flight is the same on every path and the hardware load counter can be waited
-  // on exactly. A sub-block past the range's last page re-reads that page.
+  // A sub-block past the range's last page re-reads that page.
   const int last_js = (max(tile.k1, tile.k0 + 1) - 1) & ~15;
   const int lane_k = (c16 * HD + 8 * q4), lane_v = c16 * kVtDim + 4 * q4;
-  auto load_cached = [&](int u, Unit<HD, SBU>& U, const bool valid) {
-    const int j0 = (valid ? u : cp0) << USH;
+  auto load_cached = [&](int u, Unit<HD, SBU>& U) {
+    const int j0 = u << USH;
 #pragma unroll
     for (int sb = 0; sb < SBU; ++sb) {
       const int js = min(j0 + 16 * sb, last_js);  // first key of the sub-block
       const int b = block_of(a, table, js);
       const int t0 = js % bt;
       const uint16_t* hb = a.pool + head_base(a, HD, b, kvh);
-      const uint16_t* kp = valid ? hb + t0 * HD + lane_k : a.Q;
-      const uint16_t* vp = valid ? hb + vt_elem(bt, HD, t0, 0) + lane_v : a.Q;  // t0 is a multiple of 16: the sub-block's start
-      const int ks = valid ? 32 : 0;
-      const int vs = valid ? 16 * kVtDim : 0;
+      const uint16_t* kp = hb + t0 * HD + lane_k;
+      const uint16_t* vp = hb + vt_elem(bt, HD, t0, 0) + lane_v;  // t0 is a multiple of 16: the sub-block's start
+      constexpr int ks = 32, vs = 16 * kVtDim;
       // Every cached byte is read once per pass: non-temporal loads keep the stream from displacing
       // what the caches could still serve (measured: 184 -> 164 us on 1 GB of keys at head dim 256).
 #pragma unroll
@@ -298,22 +302,32 @@ __global__ __launch_bounds__(256, OCC) void attn_stream_kernel(const KArgs a) {
   };
 
   {
-    Unit<HD, SBU> U[NBUF];
-    // ---- interior units through a ring of NBUF register sets: while one unit is in the
-    // matrix cores, the loads of the next NBUF - 1 are in flight. Wavefront w takes
-    // interior units w, w + 4, ...: n_mine of them.
+    Unit<HD, SBU> U[2];
+    // ---- interior units through two register sets: while one unit is in the matrix cores,
+    // the loads of the next are in flight. Wavefront w takes interior units w, w + 4, ...:
+    // n_mine of them.
     const int n_int = ui1 - ui0;
     const int n_mine = n_int > wave ? (n_int - wave + 3) >> 2 : 0;
     if (n_mine > 0) {
+      // Two register sets, the next unit requested before the current one is consumed, and no request
+      // without a unit behind it: at the top of the loop set 0 holds (or awaits) unit i. (A deeper
+      // ring that refilled every set it consumed - with dummy loads once the units ran out, to keep
+      // the count of loads in flight fixed - was 2 to 10 % slower on every shape, short ranges most.)
       const int u0 = ui0 + wave;
-#pragma unroll
-      for (int s = 0; s < NBUF; ++s) load_cached(u0 + 4 * s, U[s], s < n_mine);
-      for (int i = 0; i < n_mine; i += NBUF) {
-#pragma unroll
-        for (int s = 0; s < NBUF; ++s) {
-          if (i + s < n_mine) compute_interior(U[s]);
-          load_cached(u0 + 4 * (i + s + NBUF), U[s], i + s + NBUF < n_mine);
-        }
+      load_cached(u0, U[0]);
+      int i = 0;
+      for (; i + 2 < n_mine; i += 2) {
+        load_cached(u0 + 4 * (i + 1), U[1]);
+        compute_interior(U[0]);
+        load_cached(u0 + 4 * (i + 2), U[0]);
+        compute_interior(U[1]);
+      }
+      if (i + 2 == n_mine) {
+        load_cached(u0 + 4 * (i + 1), U[1]);
+        compute_interior(U[0]);
+        compute_interior(U[1]);
+      } else {
+        compute_interior(U[0]);
       }
     }
     // ---- then the units that need masks: partial or windowed cached units, batch rows.
@@ -334,8 +348,8 @@ __global__ __launch_bounds__(256, OCC) void attn_stream_kernel(const KArgs a) {
     const int n_slow = n_edge + n_batch;
     for (int i = (wave + 4 - (n_int & 3)) & 3; i < n_slow; i += 4) {
       if (i < n_edge) {
-        const int u = (a.window > 0 || !has_cached) ? cp0 + i : ((i == 0 && first_edge) ? cp0 : ulast);
-        load_cached(u, U[0], true);
+        const int u = i < n_lo ? cp0 + i : ui1 + (i - n_lo);
+        load_cached(u, U[0]);
         compute_general.template operator()<false>(u << USH, U[0]);
       } else {
         const int u = bp0 + (i - n_edge);
@@ -481,20 +495,18 @@ __global__ __launch_bounds__(256) void attn_combine_kernel(const KArgs a, const 
 
 size_t stream_smem_bytes(int HD, int NC) { return size_t(4 * NC * 16) * (HD + 4 + 2) * sizeof(float); }
 
-// Resident workgroups per CU and ring depth of each variant: the single-column-tile
-// head_dim-128 kernel fits two workgroups per CU with a two-deep ring; the wider ones
-// run one workgroup per CU with a deeper ring.
+// Resident workgroups per CU of each variant: the single-column-tile head_dim-128 kernel
+// fits two; the wider ones need more than 256 VGPRs and run one.
 constexpr int stream_occ(int HD, int NC) { return (HD == 128 && NC == 1) ? 2 : 1; }
-constexpr int stream_nbuf(int HD, int NC) { return (HD == 128 && NC == 1) ? 2 : 3; }
 int stream_workgroups_per_cu(int HD, int NC) { return stream_occ(HD, NC); }
 
 template <int DT, int HD, int NC>
 static hipError_t launch_stream_t(const KArgs& a, int n_tiles, hipStream_t st) {
   constexpr int SBU = HD == 128 ? 2 : 1;
-  constexpr int NBUF = stream_nbuf(HD, NC), OCC = stream_occ(HD, NC);
+  constexpr int OCC = stream_occ(HD, NC);
   const size_t smem = stream_smem_bytes(HD, NC);
-  constexpr auto k16 = attn_stream_kernel<DT, HD, NC, SBU, NBUF, 16, OCC>;
-  constexpr auto kbt = attn_stream_kernel<DT, HD, NC, SBU, NBUF, 0, OCC>;
+  constexpr auto k16 = attn_stream_kernel<DT, HD, NC, SBU, 16, OCC>;
+  constexpr auto kbt = attn_stream_kernel<DT, HD, NC, SBU, 0, OCC>;
   const auto k = a.bt == 16 ? k16 : kbt;
   const hipError_t e = a.bt == 16 ? allow_dynamic_lds<k16>(smem) : allow_dynamic_lds<kbt>(smem);
   if (e != hipSuccess) return e;
