@@ -48,7 +48,8 @@ int hip_fail(char* err, size_t errlen, const char* what, hipError_t e) {
 int check_params(const esp_attn_params* p, char* err, size_t errlen) {
   if (!p) return fail(err, errlen, ESP_EINVAL, "params is NULL");
   if (p->H <= 0 || p->Hkv <= 0 || p->H % p->Hkv) return fail(err, errlen, ESP_EINVAL, "H=%d Hkv=%d: H must be a positive multiple of Hkv", p->H, p->Hkv);
-  if (p->head_dim != 128 && p->head_dim != 256) return fail(err, errlen, ESP_EUNSUPPORTED, "head_dim %d (128 or 256)", p->head_dim);
+  if (p->head_dim != 128 && p->head_dim != 256 && p->head_dim != 512)
+    return fail(err, errlen, ESP_EUNSUPPORTED, "head_dim %d (128, 256 or 512)", p->head_dim);
   if (p->dtype != ESP_F16 && p->dtype != ESP_BF16) return fail(err, errlen, ESP_EINVAL, "dtype %d", p->dtype);
   if (p->bt <= 0 || p->bt % 16) return fail(err, errlen, ESP_EINVAL, "bt %d: tokens per block must be a positive multiple of 16", p->bt);
   if (p->q_ld < p->H * p->head_dim || p->q_ld % 8) return fail(err, errlen, ESP_EINVAL, "q_ld %d", p->q_ld);
@@ -64,7 +65,7 @@ int check_params(const esp_attn_params* p, char* err, size_t errlen) {
 int family(const esp_attn_params* p) {
   const int packed = p->rows_per_tile * (p->H / p->Hkv);
   const int nc = (packed + 15) / 16;
-  if (nc <= 2 && nc * p->head_dim <= 256) return nc;
+  if (nc == 1 || (nc == 2 && p->head_dim == 128)) return nc;  // two column tiles fit the registers at head dim 128 only
   return -1;
 }
 

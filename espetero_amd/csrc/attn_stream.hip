@@ -20,6 +20,14 @@
 // merge their (m, l, O) through LDS in wave order at the end. Each wavefront
 // alternates between two register sets: the loads of the next unit are in flight
 // while the current unit is in the matrix cores.
+//
+// Head dim 512 (the full-attention layers of kernels/80_gemma.metal:355-358, :561-564)
+// does not fit one wavefront's registers (accumulators, Q fragments and two operand
+// sets are 448). There the wavefronts work in pairs: both take the same 16-key unit,
+// each loads and multiplies 256 of the 512 dims, the two partial S^T meet in LDS (one
+// workgroup barrier per unit; the reference sums its per-simdgroup score partials through
+// threadgroup memory the same way, 80_gemma.metal:272-282), both run the same softmax and
+// each accumulates its 256 output dims. Two pairs take the units round robin.
 #include <type_traits>
 
 #include "common.hpp"
@@ -37,13 +45,19 @@ struct Unit {  // operands of one unit of SBU 16-key sub-blocks
 // BT: tokens per block when known at compile time (0: read from the arguments).
 template <int DT, int HD, int NC, int SBU, int BT, int OCC>
 __global__ __launch_bounds__(256, OCC) void attn_stream_kernel(const KArgs a) {
-  constexpr int KK = HD / 32, MT = HD / 16, LDO = HD + 4, UK = 16 * SBU, USH = SBU == 2 ? 5 : 4;
-  extern __shared__ float smem[];  // [4 waves][NC * 16 cols][LDO] O, then [4][NC * 16][2] m, l
+  constexpr bool PAIR = HD >= 512;      // two wavefronts per unit, HW dims each
+  constexpr int HW = PAIR ? HD / 2 : HD;
+  constexpr int NS = PAIR ? 2 : 4;       // unit streams of the workgroup
+  static_assert(!PAIR || (NC == 1 && SBU == 1), "paired wavefronts: one column tile, 16-key units");
+  constexpr int KK = HW / 32, MT = HW / 16, LDO = HD + 4, UK = 16 * SBU, USH = SBU == 2 ? 5 : 4;
+  extern __shared__ float smem[];  // [NS][NC * 16 cols][LDO] O, then [NS][NC * 16][2] m, l, then (PAIR) [2][4 waves][64] partial S^T
 
   const int bt = BT ? BT : a.bt;
   const int kvh = blockIdx.x;
   const int lane = threadIdx.x & 63;
   const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+  const int strm = PAIR ? wave >> 1 : wave;  // which of the NS unit streams
+  const int dw = PAIR ? (wave & 1) * HW : 0; // first dim of this wavefront's share of the head
   const int c16 = lane & 15, q4 = lane >> 4;
   esp_tile tile = a.tiles[blockIdx.y];
   const esp_tree tree = a.trees[tile.tree];
@@ -69,7 +83,7 @@ __global__ __launch_bounds__(256, OCC) void attn_stream_kernel(const KArgs a) {
     const int row = ok[c] ? tile.r0 + m : tile.r0;
     qpos[c] = (a.window > 0) ? a.pos[row].x : 0;
     dsc[c] = a.desc ? a.desc[row] : make_int4(0, 0, 0, 0);
-    const uint16_t* qp = a.Q + size_t(row) * a.q_ld + size_t(kvh * a.G + (ok[c] ? hg : 0)) * HD + 8 * q4;
+    const uint16_t* qp = a.Q + size_t(row) * a.q_ld + size_t(kvh * a.G + (ok[c] ? hg : 0)) * HD + dw + 8 * q4;
 #pragma unroll
     for (int kk = 0; kk < KK; ++kk)
       qf[c][kk] = ok[c] ? *reinterpret_cast<const u32x4*>(qp + 32 * kk) : u32x4{0, 0, 0, 0};
@@ -117,8 +131,8 @@ __global__ __launch_bounds__(256, OCC) void attn_stream_kernel(const KArgs a) {
   // K rows and V^T rows of cached unit u (absolute unit index) straight from the pool.
   // A sub-block past the range's last page re-reads that page.
   const int last_js = (max(tile.k1, tile.k0 + 1) - 1) & ~15;
-  const int lane_k = (c16 * HD + 8 * q4), lane_v = c16 * kVtDim + 4 * q4;
-  auto load_cached = [&](int u, Unit<HD, SBU>& U) {
+  const int lane_k = (c16 * HD + dw + 8 * q4), lane_v = (dw + c16) * kVtDim + 4 * q4;
+  auto load_cached = [&](int u, Unit<HW, SBU>& U) {
     const int j0 = u << USH;
 #pragma unroll
     for (int sb = 0; sb < SBU; ++sb) {
@@ -139,14 +153,14 @@ __global__ __launch_bounds__(256, OCC) void attn_stream_kernel(const KArgs a) {
   };
 
   // Batch units: rows of the pass (row major Kb / Vb); V gathered element by element.
-  auto load_batch = [&](int u, Unit<HD, SBU>& U) {
+  auto load_batch = [&](int u, Unit<HW, SBU>& U) {
     const int j0 = u << USH;
 #pragma unroll
     for (int sb = 0; sb < SBU; ++sb) {
       const int js = j0 + 16 * sb;
       const int jk = js + c16;
       const bool k_ok = jk <= k_last;
-      const uint16_t* kp = a.Kb + size_t(tree.base + (k_ok ? jk : 0)) * a.kv_ld + size_t(kvh) * HD + 8 * q4;
+      const uint16_t* kp = a.Kb + size_t(tree.base + (k_ok ? jk : 0)) * a.kv_ld + size_t(kvh) * HD + dw + 8 * q4;
 #pragma unroll
       for (int kk = 0; kk < KK; ++kk)
         U.k[sb][kk] = k_ok ? *reinterpret_cast<const u32x4*>(kp + 32 * kk) : u32x4{0, 0, 0, 0};
@@ -156,7 +170,7 @@ __global__ __launch_bounds__(256, OCC) void attn_stream_kernel(const KArgs a) {
 #pragma unroll
       for (int i = 0; i < 4; ++i) {
         if (jv + i > k_last) continue;
-        const uint16_t* vp = a.Vb + size_t(tree.base + jv + i) * a.kv_ld + size_t(kvh) * HD + c16;
+        const uint16_t* vp = a.Vb + size_t(tree.base + jv + i) * a.kv_ld + size_t(kvh) * HD + dw + c16;
 #pragma unroll
         for (int mt = 0; mt < MT; ++mt) {
           const uint32_t e = uint32_t(vp[16 * mt]) << (16 * (i & 1));
@@ -167,8 +181,15 @@ __global__ __launch_bounds__(256, OCC) void attn_stream_kernel(const KArgs a) {
     }
   };
 
-  // S^T = K . Q^T of one unit.
-  auto scores = [&](const Unit<HD, SBU>& U, f32x4 (&s)[NC][SBU]) {
+  // S^T = K . Q^T of one unit. Paired wavefronts: each has the sum over its HW dims; the halves are
+  // exchanged through LDS slot (unit count & 1) and added in the same order on both sides, so the
+  // two wavefronts of a pair go on with identical S^T. One workgroup barrier per unit: every
+  // wavefront of the workgroup passes through here (or through the bare barriers after the loops)
+  // the same number of times. A slot is rewritten two units later, behind the barrier of the unit
+  // in between, which the partner reaches only after it has read the slot.
+  int n_done = 0;  // units this wavefront has computed
+  f32x4* xch = reinterpret_cast<f32x4*>(smem + NS * NC * 16 * (LDO + 2));
+  auto scores = [&](const Unit<HW, SBU>& U, f32x4 (&s)[NC][SBU]) {
 #pragma unroll
     for (int c = 0; c < NC; ++c)
 #pragma unroll
@@ -177,9 +198,17 @@ __global__ __launch_bounds__(256, OCC) void attn_stream_kernel(const KArgs a) {
 #pragma unroll
         for (int kk = 0; kk < KK; ++kk) s[c][sb] = mfma16x32<DT>(U.k[sb][kk], qf[c][kk], s[c][sb]);
       }
+    if constexpr (PAIR) {
+      f32x4* slot = xch + (n_done & 1) * 256;
+      slot[wave * 64 + lane] = s[0][0];
+      __syncthreads();
+      const f32x4 other = slot[(wave ^ 1) * 64 + lane];
+      s[0][0] = (wave & 1) ? other + s[0][0] : s[0][0] + other;
+      ++n_done;
+    }
   };
   // Online softmax over a unit's scores x (log2 units, -inf where masked), then O^T += V^T . P^T.
-  auto softmax_pv = [&](const Unit<HD, SBU>& U, f32x4 (&x)[NC][SBU], const float (&mx_in)[NC]) {
+  auto softmax_pv = [&](const Unit<HW, SBU>& U, f32x4 (&x)[NC][SBU], const float (&mx_in)[NC]) {
     bool any_change = false;
     u32x2 pb[NC][SBU];
     float corr[NC];
@@ -227,7 +256,7 @@ __global__ __launch_bounds__(256, OCC) void attn_stream_kernel(const KArgs a) {
   };
 
   // Interior unit: every key visible to every row.
-  auto compute_interior = [&](const Unit<HD, SBU>& U) {
+  auto compute_interior = [&](const Unit<HW, SBU>& U) {
     f32x4 s[NC][SBU];
     scores(U, s);
     float mx[NC];
@@ -247,7 +276,7 @@ __global__ __launch_bounds__(256, OCC) void attn_stream_kernel(const KArgs a) {
 
   // General unit: per-key visibility. BATCH: the keys are the tree's batch rows j0 .. (tree
   // mask and window), else cached keys j0 .. (range ends and window).
-  auto compute_general = [&]<bool BATCH>(int j0, Unit<HD, SBU>& U) {
+  auto compute_general = [&]<bool BATCH>(int j0, Unit<HW, SBU>& U) {
     if constexpr (!BATCH) {
       // Cached keys outside [k0, k1) may be memory never written: their V must not reach the products.
 #pragma unroll
@@ -302,28 +331,28 @@ __global__ __launch_bounds__(256, OCC) void attn_stream_kernel(const KArgs a) {
   };
 
   {
-    Unit<HD, SBU> U[2];
+    Unit<HW, SBU> U[2];
     // ---- interior units through two register sets: while one unit is in the matrix cores,
-    // the loads of the next are in flight. Wavefront w takes interior units w, w + 4, ...:
+    // the loads of the next are in flight. Stream w takes interior units w, w + NS, ...:
     // n_mine of them.
     const int n_int = ui1 - ui0;
-    const int n_mine = n_int > wave ? (n_int - wave + 3) >> 2 : 0;
+    const int n_mine = n_int > strm ? (n_int - strm + NS - 1) / NS : 0;
     if (n_mine > 0) {
       // Two register sets, the next unit requested before the current one is consumed, and no request
       // without a unit behind it: at the top of the loop set 0 holds (or awaits) unit i. (A deeper
       // ring that refilled every set it consumed - with dummy loads once the units ran out, to keep
       // the count of loads in flight fixed - was 2 to 10 % slower on every shape, short ranges most.)
-      const int u0 = ui0 + wave;
+      const int u0 = ui0 + strm;
       load_cached(u0, U[0]);
       int i = 0;
       for (; i + 2 < n_mine; i += 2) {
-        load_cached(u0 + 4 * (i + 1), U[1]);
+        load_cached(u0 + NS * (i + 1), U[1]);
         compute_interior(U[0]);
-        load_cached(u0 + 4 * (i + 2), U[0]);
+        load_cached(u0 + NS * (i + 2), U[0]);
         compute_interior(U[1]);
       }
       if (i + 2 == n_mine) {
-        load_cached(u0 + 4 * (i + 1), U[1]);
+        load_cached(u0 + NS * (i + 1), U[1]);
         compute_interior(U[0]);
         compute_interior(U[1]);
       } else {
@@ -346,7 +375,7 @@ __global__ __launch_bounds__(256, OCC) void attn_stream_kernel(const KArgs a) {
       n_batch = max(0, ((k_last + UK) >> USH) - bp0);
     }
     const int n_slow = n_edge + n_batch;
-    for (int i = (wave + 4 - (n_int & 3)) & 3; i < n_slow; i += 4) {
+    for (int i = (strm + NS - n_int % NS) % NS; i < n_slow; i += NS) {
       if (i < n_edge) {
         const int u = i < n_lo ? cp0 + i : ui1 + (i - n_lo);
         load_cached(u, U[0]);
@@ -357,11 +386,15 @@ __global__ __launch_bounds__(256, OCC) void attn_stream_kernel(const KArgs a) {
         compute_general.template operator()<true>(u << USH, U[0]);
       }
     }
+    if constexpr (PAIR) {  // the other pair may have one unit more: its barrier needs this wavefront too
+      const int most = (n_int + n_slow + NS - 1) / NS;
+      for (int i = n_done; i < most; ++i) __syncthreads();
+    }
   }
 
-  // ---- merge the 4 wavefronts in wave order
-  float* o_sh = smem;                          // [4][NC * 16][LDO]
-  float* ml_sh = smem + 4 * NC * 16 * LDO;     // [4][NC * 16][2]
+  // ---- merge the NS streams in order (paired wavefronts hold the same m and l and one half of the dims each)
+  float* o_sh = smem;                          // [NS][NC * 16][LDO]
+  float* ml_sh = smem + NS * NC * 16 * LDO;    // [NS][NC * 16][2]
 #pragma unroll
   for (int c = 0; c < NC; ++c) {
     float l = l_run[c];
@@ -369,8 +402,8 @@ __global__ __launch_bounds__(256, OCC) void attn_stream_kernel(const KArgs a) {
     l += __shfl_xor(l, 32);
     l_run[c] = l;
     if (q4 == 0) {
-      ml_sh[(wave * NC * 16 + 16 * c + c16) * 2] = m_run[c];
-      ml_sh[(wave * NC * 16 + 16 * c + c16) * 2 + 1] = l;
+      ml_sh[(strm * NC * 16 + 16 * c + c16) * 2] = m_run[c];
+      ml_sh[(strm * NC * 16 + 16 * c + c16) * 2 + 1] = l;
     }
   }
   __syncthreads();
@@ -379,9 +412,9 @@ __global__ __launch_bounds__(256, OCC) void attn_stream_kernel(const KArgs a) {
     const int col = 16 * c + c16;
     float M = -INFINITY;
 #pragma unroll
-    for (int w = 0; w < 4; ++w) M = fmaxf(M, ml_sh[(w * NC * 16 + col) * 2]);
+    for (int w = 0; w < NS; ++w) M = fmaxf(M, ml_sh[(w * NC * 16 + col) * 2]);
     const float f = (m_run[c] == -INFINITY) ? 0.0f : fast_exp2(m_run[c] - M);
-    float* dst = o_sh + size_t(wave * NC * 16 + col) * LDO + 4 * q4;
+    float* dst = o_sh + size_t(strm * NC * 16 + col) * LDO + dw + 4 * q4;
 #pragma unroll
     for (int mt = 0; mt < MT; ++mt) *reinterpret_cast<f32x4*>(dst + 16 * mt) = acc[c][mt] * f;
   }
@@ -393,11 +426,11 @@ __global__ __launch_bounds__(256, OCC) void attn_stream_kernel(const KArgs a) {
     if (col >= a.cols || m >= rows_live) continue;
     float M = -INFINITY;
 #pragma unroll
-    for (int w = 0; w < 4; ++w) M = fmaxf(M, ml_sh[(w * NC * 16 + col) * 2]);
+    for (int w = 0; w < NS; ++w) M = fmaxf(M, ml_sh[(w * NC * 16 + col) * 2]);
     float L = 0.0f;
     f32x4 o = {0, 0, 0, 0};
 #pragma unroll
-    for (int w = 0; w < 4; ++w) {
+    for (int w = 0; w < NS; ++w) {
       const float mw = ml_sh[(w * NC * 16 + col) * 2];
       const float f = (mw == -INFINITY) ? 0.0f : fast_exp2(mw - M);
       L += f * ml_sh[(w * NC * 16 + col) * 2 + 1];
@@ -493,7 +526,10 @@ __global__ __launch_bounds__(256) void attn_combine_kernel(const KArgs a, const 
   *reinterpret_cast<u32x2*>(a.O + size_t(row) * a.q_ld + size_t(h) * HD + d) = out;
 }
 
-size_t stream_smem_bytes(int HD, int NC) { return size_t(4 * NC * 16) * (HD + 4 + 2) * sizeof(float); }
+size_t stream_smem_bytes(int HD, int NC) {
+  if (HD >= 512) return size_t(2 * NC * 16) * (HD + 4 + 2) * sizeof(float) + 2 * 4 * 64 * 16;  // two streams + the partial S^T slots
+  return size_t(4 * NC * 16) * (HD + 4 + 2) * sizeof(float);
+}
 
 // Resident workgroups per CU of each variant: the single-column-tile head_dim-128 kernel
 // fits two; the wider ones need more than 256 VGPRs and run one.
@@ -502,7 +538,7 @@ int stream_workgroups_per_cu(int HD, int NC) { return stream_occ(HD, NC); }
 
 template <int DT, int HD, int NC>
 static hipError_t launch_stream_t(const KArgs& a, int n_tiles, hipStream_t st) {
-  constexpr int SBU = HD == 128 ? 2 : 1;
+  constexpr int SBU = HD == 128 ? 2 : 1;  // 256 and 512 (256 dims per wavefront): 16-key units
   constexpr int OCC = stream_occ(HD, NC);
   const size_t smem = stream_smem_bytes(HD, NC);
   constexpr auto k16 = attn_stream_kernel<DT, HD, NC, SBU, 16, OCC>;
@@ -514,16 +550,18 @@ static hipError_t launch_stream_t(const KArgs& a, int n_tiles, hipStream_t st) {
   return hipGetLastError();
 }
 
-// dt, HD, NC are validated by the caller: HD in {128, 256}, NC in {1, 2}, NC * HD <= 256.
+// dt, HD, NC are validated by the caller: (HD, NC) in {(128, 1), (128, 2), (256, 1), (512, 1)}.
 hipError_t launch_stream(int dt, int HD, int NC, const KArgs& a, int n_tiles, hipStream_t st) {
   if (dt == ESP_F16) {
     if (HD == 128 && NC == 1) return launch_stream_t<ESP_F16, 128, 1>(a, n_tiles, st);
     if (HD == 128 && NC == 2) return launch_stream_t<ESP_F16, 128, 2>(a, n_tiles, st);
     if (HD == 256 && NC == 1) return launch_stream_t<ESP_F16, 256, 1>(a, n_tiles, st);
+    if (HD == 512 && NC == 1) return launch_stream_t<ESP_F16, 512, 1>(a, n_tiles, st);
   } else {
     if (HD == 128 && NC == 1) return launch_stream_t<ESP_BF16, 128, 1>(a, n_tiles, st);
     if (HD == 128 && NC == 2) return launch_stream_t<ESP_BF16, 128, 2>(a, n_tiles, st);
     if (HD == 256 && NC == 1) return launch_stream_t<ESP_BF16, 256, 1>(a, n_tiles, st);
+    if (HD == 512 && NC == 1) return launch_stream_t<ESP_BF16, 512, 1>(a, n_tiles, st);
   }
   return hipErrorInvalidValue;
 }
@@ -535,6 +573,8 @@ hipError_t launch_combine(int dt, int HD, const KArgs& a, const esp_combine* job
   else if (dt == ESP_F16 && HD == 256) hipLaunchKernelGGL((attn_combine_kernel<ESP_F16, 256>), grid, dim3(256), 0, st, a, jobs, n_jobs);
   else if (dt == ESP_BF16 && HD == 128) hipLaunchKernelGGL((attn_combine_kernel<ESP_BF16, 128>), grid, dim3(256), 0, st, a, jobs, n_jobs);
   else if (dt == ESP_BF16 && HD == 256) hipLaunchKernelGGL((attn_combine_kernel<ESP_BF16, 256>), grid, dim3(256), 0, st, a, jobs, n_jobs);
+  else if (dt == ESP_F16 && HD == 512) hipLaunchKernelGGL((attn_combine_kernel<ESP_F16, 512>), grid, dim3(256), 0, st, a, jobs, n_jobs);
+  else if (dt == ESP_BF16 && HD == 512) hipLaunchKernelGGL((attn_combine_kernel<ESP_BF16, 512>), grid, dim3(256), 0, st, a, jobs, n_jobs);
   else return hipErrorInvalidValue;
   return hipGetLastError();
 }

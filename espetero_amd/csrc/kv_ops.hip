@@ -19,7 +19,7 @@ __global__ __launch_bounds__(256) void kv_save_kernel(const uint16_t* Kb, const 
                                                       const esp_kvsave* entries, int n, int Hkv, int HD, int kv_ld, int bt,
                                                       uint64_t kv_base) {
   constexpr int R = kSaveRows;
-  __shared__ __attribute__((aligned(16))) uint16_t vs[R][256 + 8];  // HD <= 256; the pad spreads the column reads over the banks
+  __shared__ __attribute__((aligned(16))) uint16_t vs[R][512 + 8];  // HD <= 512; the pad spreads the column reads over the banks
   const int tid = threadIdx.x, g0 = blockIdx.x * R, kvh = blockIdx.y;
   const int cnt = min(R, n - g0);
   const esp_kvsave e0 = entries[g0];
@@ -136,7 +136,7 @@ __global__ __launch_bounds__(256) void kv_relayout_kernel(const uint16_t* src, u
 // head): the 16 x HD tile is transposed through LDS.
 __global__ __launch_bounds__(256) void vt_stage_kernel(const uint16_t* Vb, uint16_t* vt, int n_rows, int n_groups, int HD,
                                                        int kv_ld) {
-  __shared__ uint16_t sh[16][256 + 2];
+  __shared__ uint16_t sh[16][512 + 2];  // HD <= 512
   const int g = blockIdx.x, kvh = blockIdx.y;
   for (int i = threadIdx.x; i < 16 * (HD / 8); i += 256) {
     const int r = i / (HD / 8), x = (i % (HD / 8)) * 8;

@@ -47,6 +47,21 @@ def test_stream_kernel_matches_checker(kw):
     _check(small_case(seed=31, fill_unused=not kw.get("ring_layer", False), **kw))
 
 
+# ---- head dim 512 (Gemma 4's full-attention layers): wavefront pairs share a unit
+@pytest.mark.parametrize("kw", [
+    dict(seqs=((777, 1), (100, 1)), H=8, Hkv=1, rows_per_tile=1),                   # G = 8 decode
+    dict(seqs=((1, 1), (0, 1), (16, 1), (31, 1), (32, 1), (33, 1)), H=16, Hkv=2, rows_per_tile=1),  # 0, 1, 2, 3 units
+    dict(seqs=((5000, 1), (17, 1)), H=16, Hkv=2, rows_per_tile=1),                  # split + merge
+    dict(seqs=((300, 2), (45, 1)), H=8, Hkv=2, rows_per_tile=2, dtype=abi.ESP_BF16),  # G = 4, two rows, bf16
+    dict(seqs=((260, 2),), H=8, Hkv=1, rows_per_tile=2, desc_fn=lambda M: synth.verify_desc(M, 1)),  # 16 packed rows
+    dict(seqs=((200, 1),), H=4, Hkv=2, bt=64, rows_per_tile=1),                     # the reference's block size
+    dict(seqs=((900, 1), (40, 1)), H=4, Hkv=1, window=128, rows_per_tile=1),        # window (not a Gemma shape; same code)
+    dict(seqs=((90, 7),), H=4, Hkv=2, rows_per_tile=8),                             # G = 2, 8-row tiles: batch keys
+])
+def test_stream_kernel_head_dim_512(kw):
+    _check(small_case(seed=37, HD=512, fill_unused=True, **kw))
+
+
 def test_stream_kernel_reference_planner_records():
     """The kernels accept the reference planner's own records (8-row tiles, 32-key chunks)."""
     c = small_case(seed=32, seqs=((1024, 1),), H=32, Hkv=4, rows_per_tile=8)
