@@ -637,7 +637,7 @@ __global__ __launch_bounds__(256, OCC) void attn_tiled_kernel(const KArgs a, int
 
 // Workgroups per compute unit and the largest tile each variant takes.
 constexpr int tiled_occ(int HD) { return HD == 128 ? 2 : 1; }
-int tiled_max_rows(int) { return 128; }
+int tiled_max_rows(int HD) { return HD == 512 ? 64 : 128; }  // 512: attn_tiled512_kernel's 2 row groups x 2 dim halves
 int tiled_workgroups_per_cu(int HD) { return tiled_occ(HD); }
 size_t tiled_smem_bytes(int HD) { return size_t(4) * 64 * HD * 2 + 64; }  // two stages of K (64 rows) and V^T (64 keys), 16 ints
 
@@ -651,7 +651,10 @@ static hipError_t launch_tiled_t(const KArgs& a, int n_tiles, hipStream_t st) {
   return hipGetLastError();
 }
 
+hipError_t launch_tiled512(int dt, const KArgs& a, int n_tiles, hipStream_t st);
+
 hipError_t launch_tiled(int dt, int HD, const KArgs& a, int n_tiles, hipStream_t st) {
+  if (HD == 512 && (dt == ESP_F16 || dt == ESP_BF16)) return launch_tiled512(dt, a, n_tiles, st);
   if (dt == ESP_F16 && HD == 128) return launch_tiled_t<ESP_F16, 128>(a, n_tiles, st);
   if (dt == ESP_F16 && HD == 256) return launch_tiled_t<ESP_F16, 256>(a, n_tiles, st);
   if (dt == ESP_BF16 && HD == 128) return launch_tiled_t<ESP_BF16, 128>(a, n_tiles, st);

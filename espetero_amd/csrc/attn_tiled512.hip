@@ -1,0 +1,326 @@
+// Tiled MFMA attention at head dim 512: prefill and chunked prefill of the
+// full-attention layers whose heads are 512 wide (the reference's
+// g4_attention512_s{1,2,4,8}, kernels/80_gemma.metal:157-342, :355-358).
+//
+// Semantics as in the tiled kernel of the narrower heads: cached keys [k0, k1)
+// through the block table or ring, then the tree's batch keys (`last` tiles) under
+// the tree mask (80_:284) and the window (80_:285), online softmax in fp32, P
+// rounded to the storage type before P.V, output O / l (0 when no key is visible)
+// with the optional sigmoid gate, or a partial record for the merge.
+//
+// Mapping to gfx950. A 512-dim head does not fit one wavefront (32 rows x 512 dims
+// of fp32 accumulators alone are 256 registers), so a workgroup is one tile of up to
+// 64 query rows x one query head, and its 4 wavefronts are 2 row groups x 2 dim
+// halves: wavefront (rg, dh) owns rows 32 rg .. and dims 256 dh .. of them. Keys
+// advance in steps of 32 (two 16-key sub-blocks). Per step a wavefront computes
+//   S^T[32 keys][32 rows] over its 256 dims    v_mfma_f32_32x32x16, A = K from LDS, B = Q^T in registers
+//   the two halves of a row group meet in LDS and are added in one order on both sides
+//   (the reference sums its per-simdgroup score partials the same way, 80_:272-282)
+//   P^T = exp2(S^T - m)                         identical in both wavefronts of the pair
+//   O^T[256 dims][32 rows] += V^T . P^T         A = V^T (its 256 dims) from LDS
+// K and V^T of the next step travel global memory -> registers while the current
+// step is in the matrix cores, and registers -> the other LDS stage behind it.
+//
+// LDS layout of a stage: K as 32 rows of 1024 + 16 bytes (the pad makes the 16-byte
+// operand reads of 16 consecutive lanes hit 64 different banks); the lane with S^T row
+// l reads key row pi(l) (pi swaps bits 2 and 3), so that the 8 P values a lane packs
+// for one P.V instruction are 8 consecutive keys, which is how V^T lies in memory.
+// V^T per sub-block as [dim][16 keys] with 16 bytes of padding after every 8 dims.
+#include "common.hpp"
+
+namespace esp {
+
+namespace {
+constexpr int kHD = 512, kHW = 256;                  // dims of a head; dims one wavefront multiplies and accumulates
+constexpr int kRowB = kHD * 2 + 16;                  // bytes of a K row in LDS
+constexpr int kKStage = 32 * kRowB;                  // K of one stage
+constexpr int kVSub = kHD * 32 + (kHD / 8) * 16;     // V^T of one sub-block
+constexpr int kStage = kKStage + 2 * kVSub;
+constexpr int kXch = 4 * 4 * 64 * 16;                // partial S^T: [wavefront][4][lane] 16-byte pieces
+constexpr int kLds = 2 * kStage + kXch + 64;         // two stages, the exchange, 16 ints
+}  // namespace
+
+template <int DT>
+__global__ __launch_bounds__(256, 1) void attn_tiled512_kernel(const KArgs a, int n_tiles) {
+  constexpr int KS = kHW / 16, NT = kHW / 32;
+  extern __shared__ __attribute__((aligned(16))) char lds[];
+  f32x4* xch = reinterpret_cast<f32x4*>(lds + 2 * kStage);
+  int(*red)[4] = reinterpret_cast<int(*)[4]>(lds + 2 * kStage + kXch);
+
+  // Workgroup -> (KV head, head in group, tile): consecutive ids differ in KV head first, the heads
+  // sharing a KV head land on the same XCD's L2; tiles run last to first (longest key ranges first).
+  const int kvh = blockIdx.x % a.Hkv;
+  const int rest = blockIdx.x / a.Hkv;
+  const int hg = rest % a.G;
+  const int tile_i = n_tiles - 1 - rest / a.G;
+  const int h = kvh * a.G + hg;
+  const int tid = threadIdx.x;
+  const int lane = tid & 63;
+  const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+  const int rg = wave >> 1, dw = (wave & 1) * kHW;
+  const int l32 = lane & 31, hb = lane >> 5;
+  esp_tile tile = a.tiles[tile_i];
+  const esp_tree tree = a.trees[tile.tree];
+  if (tile.k1 == INT32_MAX) tile.k1 = tree.P;  // open-ended range: up to the tree's cached length as it is now
+  const int table = tile.pad > 0 ? tile.pad - 1 : tree.table;
+  const int end = tree.base + tree.M;
+  const int rows_live = min(a.R, end - tile.r0);
+  const int rr0 = tile.r0 - tree.base;
+
+  // ---- this lane's row and its Q fragments (this wavefront's dims)
+  const int m_row = 32 * rg + l32;
+  const bool row_ok = m_row < rows_live;
+  const int row = row_ok ? tile.r0 + m_row : tile.r0;
+  const int rr = rr0 + m_row;
+  const int4 d = a.desc ? a.desc[row] : make_int4(0, 0, 0, 0);
+  const int qpos = a.window > 0 ? a.pos[row].x : 0;
+  u32x4 qf[KS];
+  {
+    const uint16_t* qp = a.Q + size_t(row) * a.q_ld + size_t(h) * kHD + dw + 8 * hb;
+#pragma unroll
+    for (int ks = 0; ks < KS; ++ks) qf[ks] = row_ok ? *reinterpret_cast<const u32x4*>(qp + 16 * ks) : u32x4{0, 0, 0, 0};
+  }
+
+  // ---- the last batch key any row of the tile sees
+  int k_last = -1;
+  {
+    int kl = row_ok ? max(rr, max(d.z - 1, a.bidi ? d.w - 1 : -1)) : -1;
+#pragma unroll
+    for (int o = 32; o >= 1; o >>= 1) kl = max(kl, __shfl_xor(kl, o));
+    if (lane == 0) red[wave][0] = kl;
+    __syncthreads();
+    k_last = max(max(red[0][0], red[1][0]), max(red[2][0], red[3][0]));
+    k_last = __builtin_amdgcn_readfirstlane(min(k_last, tree.M - 1));
+  }
+
+  // ---- the key range as 16-key sub-blocks: cached [k0, k1), then batch rows [b0, k_last]
+  const int c0 = tile.k0 >> 4;
+  const int n_c = tile.k1 > tile.k0 ? ((tile.k1 + 15) >> 4) - c0 : 0;
+  const int a0 = (tree.base + tile.b0) >> 4;  // batch sub-blocks are groups of 16 absolute rows
+  const int n_b = (tile.last && k_last >= tile.b0) ? ((tree.base + k_last) >> 4) - a0 + 1 : 0;
+  const int n_sb = n_c + n_b;
+  const int n_steps = (n_sb + 1) >> 1;
+  const int n_groups = (a.n_rows + 15) >> 4;
+
+  // ---- staging. K: instruction q brings key row 4 q + wave of the sub-block, this lane its 16-byte chunk
+  // `lane` of the 64. V^T: instruction q brings the 16-byte pieces 256 q + tid of the sub-block's 1024;
+  // piece c holds keys 8 (c % 2) .. + 7 of dim c / 2.
+  u32x4 kreg[8], vreg[8];
+  auto gload = [&](int step) __attribute__((always_inline)) {
+#pragma unroll
+    for (int t = 0; t < 2; ++t) {
+      const int sidx = 2 * step + t;
+      if (sidx < n_c) {
+        const int js = (c0 + sidx) << 4;
+        const int b = block_of(a, table, js);
+        const int t0 = js % a.bt;
+        const char* hbp = reinterpret_cast<const char*>(a.pool + head_base(a, kHD, b, kvh));
+        const char* kb = hbp + size_t(t0) * (kHD * 2) + lane * 16;
+        const char* vb = hbp + vt_elem(a.bt, kHD, t0, 0) * 2 + tid * 16;
+#pragma unroll
+        for (int q = 0; q < 4; ++q) kreg[4 * t + q] = *reinterpret_cast<const u32x4*>(kb + (4 * q + wave) * (kHD * 2));
+#pragma unroll
+        for (int q = 0; q < 4; ++q) vreg[4 * t + q] = *reinterpret_cast<const u32x4*>(vb + q * 4096);
+        if (js < tile.k0 || js + 16 > tile.k1) {
+          // Cached keys outside [k0, k1) may be memory never written: their V must not reach the products.
+          const int jv = js + 8 * (tid & 1);
+          u32x4 msk;
+#pragma unroll
+          for (int e = 0; e < 4; ++e) {
+            const bool lo = jv + 2 * e >= tile.k0 && jv + 2 * e < tile.k1;
+            const bool hi = jv + 2 * e + 1 >= tile.k0 && jv + 2 * e + 1 < tile.k1;
+            msk[e] = (lo ? 0xffffu : 0u) | (hi ? 0xffff0000u : 0u);
+          }
+#pragma unroll
+          for (int q = 0; q < 4; ++q) vreg[4 * t + q] &= msk;
+        }
+      } else if (sidx < n_sb) {
+        const int g = a0 + (sidx - n_c);
+        const int lim = a.n_rows - 1 - 16 * g;  // batch rows past the pass's last row do not exist: repeat the last (masked)
+        const char* kb = reinterpret_cast<const char*>(a.Kb + size_t(16 * g) * a.kv_ld + size_t(kvh) * kHD) + lane * 16;
+        const char* vb = reinterpret_cast<const char*>(a.vt_stage + (size_t(kvh) * n_groups + g) * size_t(kHD) * 16) + tid * 16;
+#pragma unroll
+        for (int q = 0; q < 4; ++q)
+          kreg[4 * t + q] = *reinterpret_cast<const u32x4*>(kb + size_t(min(4 * q + wave, lim)) * size_t(a.kv_ld) * 2);
+#pragma unroll
+        for (int q = 0; q < 4; ++q) vreg[4 * t + q] = *reinterpret_cast<const u32x4*>(vb + q * 4096);
+      } else {  // past the range: S is masked, V^T must be finite
+#pragma unroll
+        for (int q = 0; q < 4; ++q) {
+          kreg[4 * t + q] = u32x4{0, 0, 0, 0};
+          vreg[4 * t + q] = u32x4{0, 0, 0, 0};
+        }
+      }
+    }
+  };
+  auto sstore = [&](int stage) __attribute__((always_inline)) {
+    char* st = lds + stage * kStage;
+#pragma unroll
+    for (int t = 0; t < 2; ++t)
+#pragma unroll
+      for (int q = 0; q < 4; ++q) {
+        *reinterpret_cast<u32x4*>(st + (16 * t + 4 * q + wave) * kRowB + lane * 16) = kreg[4 * t + q];
+        const int c = 256 * q + tid, dim = c >> 1;
+        *reinterpret_cast<u32x4*>(st + kKStage + t * kVSub + dim * 32 + (dim >> 3) * 16 + (c & 1) * 16) = vreg[4 * t + q];
+      }
+  };
+
+  // ---- operand reads: per-lane byte offsets inside a stage
+  const int prow = (l32 & 0x13) | ((l32 & 4) << 1) | ((l32 & 8) >> 1);  // pi(l32)
+  const int koff = prow * kRowB + dw * 2 + hb * 16;                     // + 32 ks
+  const int vdim = dw + l32;
+  const int voff = kKStage + vdim * 32 + (vdim >> 3) * 16 + hb * 16;    // + t kVSub + nt (32 * 32 + 4 * 16)
+
+  f32x16 acc[NT];
+  float m_run = -INFINITY, l_run = 0.0f;  // l_run: this lane's share (16 of every 32 keys) of the row's sum
+#pragma unroll
+  for (int nt = 0; nt < NT; ++nt)
+#pragma unroll
+    for (int i = 0; i < 16; ++i) acc[nt][i] = 0.0f;
+
+  auto compute = [&](int step, int stage) __attribute__((always_inline)) {
+    const char* st = lds + stage * kStage;
+    // s[4 i + j] is S^T row 8 i + 4 hb + j, which is key 16 (i / 2) + 8 hb + 4 (i % 2) + j of the step:
+    // s[8 t + e] is key 8 hb + e of sub-block t.
+    f32x16 s;
+#pragma unroll
+    for (int i = 0; i < 16; ++i) s[i] = 0.0f;
+#pragma unroll
+    for (int ks = 0; ks < KS; ++ks) s = mfma32x16<DT>(*reinterpret_cast<const u32x4*>(st + koff + 32 * ks), qf[ks], s);
+    // The other half of the dims: through LDS, added in the same order in both wavefronts of the pair.
+#pragma unroll
+    for (int v = 0; v < 4; ++v) xch[(wave * 4 + v) * 64 + lane] = f32x4{s[4 * v], s[4 * v + 1], s[4 * v + 2], s[4 * v + 3]};
+    __syncthreads();
+#pragma unroll
+    for (int v = 0; v < 4; ++v) {
+      const f32x4 o = xch[((wave ^ 1) * 4 + v) * 64 + lane];
+#pragma unroll
+      for (int j = 0; j < 4; ++j) s[4 * v + j] = (wave & 1) ? o[j] + s[4 * v + j] : s[4 * v + j] + o[j];
+    }
+    // ---- visibility
+#pragma unroll
+    for (int t = 0; t < 2; ++t) {
+      const int sidx = 2 * step + t;
+      const bool cached = sidx < n_c, batch = !cached && sidx < n_sb;
+      const int j0 = cached ? (c0 + sidx) << 4 : ((a0 + sidx - n_c) << 4) - tree.base;
+      if (cached && a.window == 0 && j0 >= tile.k0 && j0 + 16 <= tile.k1) continue;  // every key visible to every row
+      // Visible keys of the sub-block for this lane's row: j in [lo, hi], or 0 <= j < anc.
+      int lo, hi, anc = 0;
+      if (cached) {
+        lo = tile.k0;
+        hi = tile.k1 - 1;
+        if (a.window > 0) lo = max(lo, qpos - a.window + 1);
+      } else if (batch) {
+        lo = max(d.x, 0);
+        hi = min(k_last, (a.bidi && d.w > 0) ? max(rr, d.w - 1) : rr);
+        anc = min(d.z, k_last + 1);
+      } else {
+        lo = 1;
+        hi = 0;
+      }
+      const int jb = j0 + 8 * hb;
+#pragma unroll
+      for (int e = 0; e < 8; ++e) {
+        const int j = jb + e;
+        bool vis = (j >= lo && j <= hi) || (j >= 0 && j < anc);
+        if (batch && a.window > 0 && vis) vis = qpos - a.pos[tree.base + j].x < a.window;
+        s[8 * t + e] = vis ? s[8 * t + e] : -INFINITY;
+      }
+    }
+    // ---- online softmax; the two lanes of a row (hb = 0, 1) agree on the maximum
+    float mx = -INFINITY;
+#pragma unroll
+    for (int i = 0; i < 16; ++i) mx = fmaxf(mx, s[i]);
+    mx *= a.scale_log2;  // scale > 0: the max commutes with it
+    mx = fmaxf(mx, __shfl_xor(mx, 32));
+    const float m_new = fmaxf(m_run, mx);
+    const float m_safe = (m_new == -INFINITY) ? 0.0f : m_new;
+    if (__any(m_new > m_run)) {
+      const float corr = fast_exp2(m_run - m_safe);  // -inf -> 0: nothing accumulated yet
+      l_run *= corr;
+#pragma unroll
+      for (int nt = 0; nt < NT; ++nt) acc[nt] *= corr;
+      m_run = m_new;
+    }
+    u32x4 pb[2];
+    float ps = 0.0f;
+#pragma unroll
+    for (int t = 0; t < 2; ++t) {
+      float p[8];
+#pragma unroll
+      for (int e = 0; e < 8; ++e) {
+        p[e] = fast_exp2(__builtin_fmaf(s[8 * t + e], a.scale_log2, -m_safe));
+        ps += p[e];
+      }
+      pb[t] = u32x4{pack2<DT>(p[0], p[1]), pack2<DT>(p[2], p[3]), pack2<DT>(p[4], p[5]), pack2<DT>(p[6], p[7])};
+    }
+    l_run += ps;
+    // ---- O^T += V^T . P^T over this wavefront's dims
+#pragma unroll
+    for (int t = 0; t < 2; ++t)
+#pragma unroll
+      for (int nt = 0; nt < NT; ++nt)
+        acc[nt] = mfma32x16<DT>(*reinterpret_cast<const u32x4*>(st + voff + t * kVSub + nt * (32 * 32 + 4 * 16)), pb[t], acc[nt]);
+  };
+
+  // At the top of iteration i stage i % 2 holds step i. The loads of step i + 1 are in flight during the
+  // step's matrix work and go into the other stage behind it; one barrier publishes them (and retires
+  // every read of the exchange area), the barrier inside compute() covers the exchange itself.
+  if (n_steps > 0) {
+    gload(0);
+    sstore(0);
+  }
+  __syncthreads();
+  for (int i = 0; i < n_steps; ++i) {
+    if (i + 1 < n_steps) gload(i + 1);
+    compute(i, i & 1);
+    if (i + 1 < n_steps) sstore((i + 1) & 1);
+    __syncthreads();
+  }
+
+  // ---- output: lane (row l32, half hb) holds dims dw + 32 nt + 8 i + 4 hb + j at acc[nt][4 i + j]
+  const float l = l_run + __shfl_xor(l_run, 32);
+  if (!row_ok) return;
+  if (tile.part >= 0) {
+    const size_t rec = (size_t(tile.part) * a.Hkv + kvh) * a.cols + size_t(m_row) * a.G + hg;
+    float* po = a.parts_o + rec * kHD + dw;
+#pragma unroll
+    for (int nt = 0; nt < NT; ++nt)
+#pragma unroll
+      for (int i4 = 0; i4 < 4; ++i4)
+        *reinterpret_cast<f32x4*>(po + 32 * nt + 8 * i4 + 4 * hb) =
+            f32x4{acc[nt][4 * i4], acc[nt][4 * i4 + 1], acc[nt][4 * i4 + 2], acc[nt][4 * i4 + 3]};
+    if (hb == 0 && dw == 0) {
+      a.parts_ml[rec * 2] = m_run;
+      a.parts_ml[rec * 2 + 1] = l;
+    }
+    return;
+  }
+  const float inv = l > 0.0f ? 1.0f / l : 0.0f;
+  uint16_t* op = a.O + size_t(row) * a.q_ld + size_t(h) * kHD + dw;
+  const float* gp = a.gate ? a.gate + size_t(row) * a.gate_ld + size_t(h) * a.gate_hs + a.gate_off + dw * a.gate_ds : nullptr;
+#pragma unroll
+  for (int nt = 0; nt < NT; ++nt)
+#pragma unroll
+    for (int i4 = 0; i4 < 4; ++i4) {
+      const int dd = 32 * nt + 8 * i4 + 4 * hb;
+      float o[4];
+#pragma unroll
+      for (int j = 0; j < 4; ++j) {
+        o[j] = acc[nt][4 * i4 + j] * inv;
+        if (gp) o[j] = o[j] / (1.0f + __expf(-gp[(dd + j) * a.gate_ds]));
+      }
+      *reinterpret_cast<u32x2*>(op + dd) = u32x2{pack2<DT>(o[0], o[1]), pack2<DT>(o[2], o[3])};
+    }
+}
+
+hipError_t launch_tiled512(int dt, const KArgs& a, int n_tiles, hipStream_t st) {
+  constexpr auto kf = attn_tiled512_kernel<ESP_F16>;
+  constexpr auto kb = attn_tiled512_kernel<ESP_BF16>;
+  const hipError_t e = dt == ESP_F16 ? allow_dynamic_lds<kf>(kLds) : allow_dynamic_lds<kb>(kLds);
+  if (e != hipSuccess) return e;
+  launch_timed(dt == ESP_F16 ? kf : kb, dim3(unsigned(n_tiles) * a.H), dim3(256), size_t(kLds), st, a, n_tiles);
+  return hipGetLastError();
+}
+
+}  // namespace esp

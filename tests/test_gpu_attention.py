@@ -122,6 +122,40 @@ def test_tiled_kernel_matches_checker(kw):
     _check(small_case(seed=41, rows_per_tile=128, **kw))
 
 
+# ---- head dim 512 prefill: 64-row tiles, wavefront pairs split the dims
+@pytest.mark.parametrize("kw", [
+    dict(seqs=((0, 200),), H=4, Hkv=2),                                 # first chunk: batch keys only
+    dict(seqs=((300, 130), (17, 5)), H=4, Hkv=2, fill_unused=True),     # chunk against a cache, ragged
+    dict(seqs=((64, 150),), H=16, Hkv=2, dtype=abi.ESP_BF16),           # G = 8 (Gemma 4's grouping), bf16
+    dict(seqs=((500, 100),), window=128, H=2, Hkv=1),                   # sliding window (not a Gemma shape; same code)
+    dict(seqs=((700, 70),), window=256, ring_layer=True, H=2, Hkv=1),   # rings
+    dict(seqs=((90, 40),), desc_fn=lambda M: synth.verify_desc(M, 30), H=4, Hkv=2),  # wide verify tree
+    dict(seqs=((128, 128),), bt=64, H=4, Hkv=2),
+    dict(seqs=((100, 140),), H=2, Hkv=1, bidi=1, desc_fn=lambda M: synth.image_desc(M, 10, 90)),   # bidirectional span
+    dict(seqs=((1203, 64), (700, 40)), bt=64, H=4, Hkv=2, fill_unused=True),  # long cached ranges, ragged end
+])
+def test_tiled_kernel_head_dim_512(kw):
+    _check(small_case(seed=44, HD=512, rows_per_tile=64, **kw))
+
+
+def test_tiled_kernel_head_dim_512_split_and_gate():
+    """Split tiles merged by the combine kernel at head dim 512, with a head-wise gate in the epilogue."""
+    import torch
+    from gpu_utils import run_case
+    c = small_case(seed=45, HD=512, seqs=((2000, 70),), H=4, Hkv=2, rows_per_tile=64)
+    _check(c, host.options_mi355x(64, 64))
+    p = c.params
+    g = np.random.default_rng(1).standard_normal((c.n_rows, p.H)).astype(np.float32)
+    gd = torch.from_numpy(g).cuda()
+    p.gate, p.gate_ld, p.gate_hs, p.gate_off, p.gate_headwise = gd.data_ptr(), p.H, 1, 0, 1
+    split = f32(run_case(c, host.options_mi355x(64, 64)), p.dtype)
+    whole = f32(run_case(c, host.options_mi355x(64, 1)), p.dtype)
+    p.gate, p.gate_headwise = None, 0
+    want = brute(c).reshape(c.n_rows, p.H, -1) / (1.0 + np.exp(-g.astype(np.float64)))[:, :, None]
+    assert np.abs(split - want.reshape(c.n_rows, -1)).max() <= 2e-3
+    assert np.abs(whole - want.reshape(c.n_rows, -1)).max() <= 2e-3
+
+
 def test_tiled_kernel_split_tiles_and_combine():
     """A single long-context tile group is split over key ranges and merged."""
     c = small_case(seed=42, seqs=((3000, 100),), H=4, Hkv=2, rows_per_tile=128)
