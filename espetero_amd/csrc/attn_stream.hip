@@ -27,7 +27,9 @@
 // each loads and multiplies 256 of the 512 dims, the two partial S^T meet in LDS (one
 // workgroup barrier per unit; the reference sums its per-simdgroup score partials through
 // threadgroup memory the same way, 80_gemma.metal:272-282), both run the same softmax and
-// each accumulates its 256 output dims. Two pairs take the units round robin.
+// each accumulates its 256 output dims. A workgroup is one such pair (128 threads, two
+// workgroups per compute unit), so the barrier ties no more than the two wavefronts
+// that need each other.
 #include <type_traits>
 
 #include "common.hpp"
@@ -44,19 +46,20 @@ struct Unit {  // operands of one unit of SBU 16-key sub-blocks
 // head dims whose operands would not fit two register sets otherwise).
 // BT: tokens per block when known at compile time (0: read from the arguments).
 template <int DT, int HD, int NC, int SBU, int BT, int OCC>
-__global__ __launch_bounds__(256, OCC) void attn_stream_kernel(const KArgs a) {
+__global__ __launch_bounds__(HD >= 512 ? 128 : 256, OCC) void attn_stream_kernel(const KArgs a) {
   constexpr bool PAIR = HD >= 512;      // two wavefronts per unit, HW dims each
   constexpr int HW = PAIR ? HD / 2 : HD;
-  constexpr int NS = PAIR ? 2 : 4;       // unit streams of the workgroup
+  constexpr int NS = PAIR ? 1 : 4;       // unit streams of the workgroup
+  constexpr int NW = PAIR ? 2 : 4;       // wavefronts of the workgroup
   static_assert(!PAIR || (NC == 1 && SBU == 1), "paired wavefronts: one column tile, 16-key units");
   constexpr int KK = HW / 32, MT = HW / 16, LDO = HD + 4, UK = 16 * SBU, USH = SBU == 2 ? 5 : 4;
-  extern __shared__ float smem[];  // [NS][NC * 16 cols][LDO] O, then [NS][NC * 16][2] m, l, then (PAIR) [2][4 waves][64] partial S^T
+  extern __shared__ float smem[];  // [NS][NC * 16 cols][LDO] O, then [NS][NC * 16][2] m, l, then (PAIR) [2][NW][64] partial S^T
 
   const int bt = BT ? BT : a.bt;
   const int kvh = blockIdx.x;
   const int lane = threadIdx.x & 63;
   const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
-  const int strm = PAIR ? wave >> 1 : wave;  // which of the NS unit streams
+  const int strm = PAIR ? 0 : wave;          // which of the NS unit streams
   const int dw = PAIR ? (wave & 1) * HW : 0; // first dim of this wavefront's share of the head
   const int c16 = lane & 15, q4 = lane >> 4;
   esp_tile tile = a.tiles[blockIdx.y];
@@ -199,7 +202,7 @@ __global__ __launch_bounds__(256, OCC) void attn_stream_kernel(const KArgs a) {
         for (int kk = 0; kk < KK; ++kk) s[c][sb] = mfma16x32<DT>(U.k[sb][kk], qf[c][kk], s[c][sb]);
       }
     if constexpr (PAIR) {
-      f32x4* slot = xch + (n_done & 1) * 256;
+      f32x4* slot = xch + (n_done & 1) * (NW * 64);
       slot[wave * 64 + lane] = s[0][0];
       __syncthreads();
       const f32x4 other = slot[(wave ^ 1) * 64 + lane];
@@ -386,7 +389,7 @@ __global__ __launch_bounds__(256, OCC) void attn_stream_kernel(const KArgs a) {
         compute_general.template operator()<true>(u << USH, U[0]);
       }
     }
-    if constexpr (PAIR) {  // the other pair may have one unit more: its barrier needs this wavefront too
+    if constexpr (PAIR && NS > 1) {  // another pair may have one unit more: its barrier needs this wavefront too
       const int most = (n_int + n_slow + NS - 1) / NS;
       for (int i = n_done; i < most; ++i) __syncthreads();
     }
@@ -420,7 +423,7 @@ __global__ __launch_bounds__(256, OCC) void attn_stream_kernel(const KArgs a) {
   }
   __syncthreads();
   // Each thread finishes 4 dims of one packed row at a time.
-  for (int i = threadIdx.x; i < NC * 16 * (HD / 4); i += 256) {
+  for (int i = threadIdx.x; i < NC * 16 * (HD / 4); i += NW * 64) {
     const int col = i / (HD / 4), d = (i % (HD / 4)) * 4;
     const int m = col / a.G, hg = col - m * a.G;
     if (col >= a.cols || m >= rows_live) continue;
@@ -527,14 +530,15 @@ __global__ __launch_bounds__(256) void attn_combine_kernel(const KArgs a, const 
 }
 
 size_t stream_smem_bytes(int HD, int NC) {
-  if (HD >= 512) return size_t(2 * NC * 16) * (HD + 4 + 2) * sizeof(float) + 2 * 4 * 64 * 16;  // two streams + the partial S^T slots
+  if (HD >= 512) return size_t(NC * 16) * (HD + 4 + 2) * sizeof(float) + 2 * 2 * 64 * 16;  // one stream + the partial S^T slots
   return size_t(4 * NC * 16) * (HD + 4 + 2) * sizeof(float);
 }
 
 // Resident workgroups per CU of each variant: the single-column-tile head_dim-128 kernel
 // fits two; the wider ones need more than 256 VGPRs and run one.
-constexpr int stream_occ(int HD, int NC) { return (HD == 128 && NC == 1) ? 2 : 1; }
-int stream_workgroups_per_cu(int HD, int NC) { return stream_occ(HD, NC); }
+constexpr int stream_occ(int HD, int NC) { return (HD == 128 && NC == 1) ? 2 : 1; }  // wavefronts per SIMD
+// Head dim 512: workgroups of two wavefronts, one per SIMD: two fill a compute unit.
+int stream_workgroups_per_cu(int HD, int NC) { return HD >= 512 ? 2 : stream_occ(HD, NC); }
 
 template <int DT, int HD, int NC>
 static hipError_t launch_stream_t(const KArgs& a, int n_tiles, hipStream_t st) {
@@ -546,7 +550,7 @@ static hipError_t launch_stream_t(const KArgs& a, int n_tiles, hipStream_t st) {
   const auto k = a.bt == 16 ? k16 : kbt;
   const hipError_t e = a.bt == 16 ? allow_dynamic_lds<k16>(smem) : allow_dynamic_lds<kbt>(smem);
   if (e != hipSuccess) return e;
-  launch_timed(k, dim3(a.Hkv, n_tiles), dim3(256), smem, st, a);
+  launch_timed(k, dim3(a.Hkv, n_tiles), dim3(HD >= 512 ? 128 : 256), smem, st, a);
   return hipGetLastError();
 }
 

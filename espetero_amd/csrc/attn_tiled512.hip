@@ -18,23 +18,27 @@
 //   (the reference sums its per-simdgroup score partials the same way, 80_:272-282)
 //   P^T = exp2(S^T - m)                         identical in both wavefronts of the pair
 //   O^T[256 dims][32 rows] += V^T . P^T         A = V^T (its 256 dims) from LDS
-// K and V^T of the next step travel global memory -> registers while the current
-// step is in the matrix cores, and registers -> the other LDS stage behind it.
+// The next step travels global memory -> the other LDS stage with global_load_lds_dwordx4
+// (no staging registers) while the current step is in the matrix cores.
 //
-// LDS layout of a stage: K as 32 rows of 1024 + 16 bytes (the pad makes the 16-byte
-// operand reads of 16 consecutive lanes hit 64 different banks); the lane with S^T row
-// l reads key row pi(l) (pi swaps bits 2 and 3), so that the 8 P values a lane packs
-// for one P.V instruction are 8 consecutive keys, which is how V^T lies in memory.
-// V^T per sub-block as [dim][16 keys] with 16 bytes of padding after every 8 dims.
+// LDS layout of a stage. K: 32 rows of 1024 bytes, unpadded; the 16-byte chunk c of row r
+// lies at chunk position c ^ (pi(r) & 15), pi = swap of row bits 2 and 3. The lane with S^T
+// row l reads key row pi(l) at position c ^ (l & 15): 16 consecutive lanes hit 16 different
+// positions, and with the rows permuted by pi the 8 P values a lane packs for one P.V
+// instruction are 8 consecutive keys, which is how V^T lies in memory. V^T per sub-block:
+// [dim][2 halves of 8 keys], the two 16-byte halves of dim d swapped when bit 3 of d is set
+// (lanes d and d + 8 of an operand read would otherwise share banks).
+#include <utility>
+
 #include "common.hpp"
+#include "lds_direct.hpp"
 
 namespace esp {
 
 namespace {
 constexpr int kHD = 512, kHW = 256;                  // dims of a head; dims one wavefront multiplies and accumulates
-constexpr int kRowB = kHD * 2 + 16;                  // bytes of a K row in LDS
-constexpr int kKStage = 32 * kRowB;                  // K of one stage
-constexpr int kVSub = kHD * 32 + (kHD / 8) * 16;     // V^T of one sub-block
+constexpr int kKStage = 32 * kHD * 2;                // K of one stage: 32 rows
+constexpr int kVSub = kHD * 32;                      // V^T of one sub-block
 constexpr int kStage = kKStage + 2 * kVSub;
 constexpr int kXch = 4 * 4 * 64 * 16;                // partial S^T: [wavefront][4][lane] 16-byte pieces
 constexpr int kLds = 2 * kStage + kXch + 64;         // two stages, the exchange, 16 ints
@@ -102,74 +106,93 @@ __global__ __launch_bounds__(256, 1) void attn_tiled512_kernel(const KArgs a, in
   const int n_steps = (n_sb + 1) >> 1;
   const int n_groups = (a.n_rows + 15) >> 4;
 
-  // ---- staging. K: instruction q brings key row 4 q + wave of the sub-block, this lane its 16-byte chunk
-  // `lane` of the 64. V^T: instruction q brings the 16-byte pieces 256 q + tid of the sub-block's 1024;
-  // piece c holds keys 8 (c % 2) .. + 7 of dim c / 2.
-  u32x4 kreg[8], vreg[8];
-  auto gload = [&](int step) __attribute__((always_inline)) {
+  // ---- staging, 16 bytes per lane straight into LDS. K: this wavefront brings rows 4 wave .. + 3 of each
+  // sub-block; the lane that fills chunk position `lane` of row r brings chunk lane ^ (pi(r) & 15), and
+  // pi(4 wave + q) = pi(4 wave) + q. V^T: this wavefront brings pieces 256 wave .. + 255 of each sub-block's
+  // 1024 (piece c: keys 8 (c % 2) .. + 7 of dim c / 2); position p holds piece p ^ ((p >> 4) & 1).
+  const uint32_t lds_base = uint32_t(uintptr_t(lds));
+  // Block ids of the cached sub-blocks, 64 at a time: lane l holds the block of sub-block ids0 + l, so the
+  // per-step lookup is a lane read instead of a dependent memory access in front of every staging load.
+  int ids = 0, ids0 = -(1 << 30);
+  auto block_id = [&](int sidx) __attribute__((always_inline)) {
+    if (sidx < ids0 || sidx >= ids0 + 64) {
+      ids0 = sidx;
+      const int sl = sidx + lane;
+      ids = sl < n_c ? block_of(a, table, (c0 + sl) << 4) : 0;
+    }
+    return __builtin_amdgcn_readlane(ids, sidx - ids0);
+  };
+  const uint32_t kx = uint32_t(swap23(4 * wave));
+  const uint32_t voff = uint32_t((lane ^ ((lane >> 4) & 1)) << 4);
+  auto fill = [&](int step, int stage) __attribute__((always_inline)) {
 #pragma unroll
     for (int t = 0; t < 2; ++t) {
       const int sidx = 2 * step + t;
+      const uint32_t kdst = lds_base + stage * kStage + (16 * t + 4 * wave) * 1024;
+      const uint32_t vdst = lds_base + stage * kStage + kKStage + t * kVSub + wave * 4096;
+      const uint32_t kl = uint32_t(lane);
       if (sidx < n_c) {
         const int js = (c0 + sidx) << 4;
-        const int b = block_of(a, table, js);
+        const int b = block_id(sidx);
         const int t0 = js % a.bt;
         const char* hbp = reinterpret_cast<const char*>(a.pool + head_base(a, kHD, b, kvh));
-        const char* kb = hbp + size_t(t0) * (kHD * 2) + lane * 16;
-        const char* vb = hbp + vt_elem(a.bt, kHD, t0, 0) * 2 + tid * 16;
-#pragma unroll
-        for (int q = 0; q < 4; ++q) kreg[4 * t + q] = *reinterpret_cast<const u32x4*>(kb + (4 * q + wave) * (kHD * 2));
-#pragma unroll
-        for (int q = 0; q < 4; ++q) vreg[4 * t + q] = *reinterpret_cast<const u32x4*>(vb + q * 4096);
-        if (js < tile.k0 || js + 16 > tile.k1) {
-          // Cached keys outside [k0, k1) may be memory never written: their V must not reach the products.
-          const int jv = js + 8 * (tid & 1);
-          u32x4 msk;
-#pragma unroll
-          for (int e = 0; e < 4; ++e) {
-            const bool lo = jv + 2 * e >= tile.k0 && jv + 2 * e < tile.k1;
-            const bool hi = jv + 2 * e + 1 >= tile.k0 && jv + 2 * e + 1 < tile.k1;
-            msk[e] = (lo ? 0xffffu : 0u) | (hi ? 0xffff0000u : 0u);
-          }
-#pragma unroll
-          for (int q = 0; q < 4; ++q) vreg[4 * t + q] &= msk;
-        }
+        const char* kb = hbp + size_t(t0 + 4 * wave) * 1024;
+        const char* vb = hbp + vt_elem(a.bt, kHD, t0, 0) * 2 + wave * 4096;  // the 16-token sub-block: 16 KB contiguous
+        load_to_lds16_x4(kb, (kl ^ kx) << 4, (kl ^ (kx + 1)) << 4, (kl ^ (kx + 2)) << 4, (kl ^ (kx + 3)) << 4, kdst);
+        load_to_lds16_x4(vb, voff, voff, voff, voff, vdst);
       } else if (sidx < n_sb) {
         const int g = a0 + (sidx - n_c);
         const int lim = a.n_rows - 1 - 16 * g;  // batch rows past the pass's last row do not exist: repeat the last (masked)
-        const char* kb = reinterpret_cast<const char*>(a.Kb + size_t(16 * g) * a.kv_ld + size_t(kvh) * kHD) + lane * 16;
-        const char* vb = reinterpret_cast<const char*>(a.vt_stage + (size_t(kvh) * n_groups + g) * size_t(kHD) * 16) + tid * 16;
+        const char* kb = reinterpret_cast<const char*>(a.Kb + size_t(16 * g) * a.kv_ld + size_t(kvh) * kHD);
+        const char* vb = reinterpret_cast<const char*>(a.vt_stage + (size_t(kvh) * n_groups + g) * size_t(kHD) * 16) + wave * 4096;
 #pragma unroll
         for (int q = 0; q < 4; ++q)
-          kreg[4 * t + q] = *reinterpret_cast<const u32x4*>(kb + size_t(min(4 * q + wave, lim)) * size_t(a.kv_ld) * 2);
+          load_to_lds16(kb + size_t(min(4 * wave + q, lim)) * size_t(a.kv_ld) * 2, (kl ^ (kx + q)) << 4, kdst + q * 1024);
+        load_to_lds16_x4(vb, voff, voff, voff, voff, vdst);
+      } else {  // past the range: K stays whatever it was (S is masked), V^T must be finite
 #pragma unroll
-        for (int q = 0; q < 4; ++q) vreg[4 * t + q] = *reinterpret_cast<const u32x4*>(vb + q * 4096);
-      } else {  // past the range: S is masked, V^T must be finite
-#pragma unroll
-        for (int q = 0; q < 4; ++q) {
-          kreg[4 * t + q] = u32x4{0, 0, 0, 0};
-          vreg[4 * t + q] = u32x4{0, 0, 0, 0};
-        }
+        for (int q = 0; q < 4; ++q)
+          *reinterpret_cast<u32x4*>(lds + stage * kStage + kKStage + t * kVSub + wave * 4096 + q * 1024 + lane * 16) = u32x4{0, 0, 0, 0};
       }
     }
   };
-  auto sstore = [&](int stage) __attribute__((always_inline)) {
-    char* st = lds + stage * kStage;
+  // After this wavefront's loads of `step` have landed: cached keys outside [k0, k1) may be memory
+  // never written; their V must not reach the products.
+  auto fix = [&](int step, int stage) __attribute__((always_inline)) {
 #pragma unroll
-    for (int t = 0; t < 2; ++t)
+    for (int t = 0; t < 2; ++t) {
+      const int sidx = 2 * step + t;
+      if (sidx >= n_c) continue;
+      const int j0 = (c0 + sidx) << 4;
+      if (j0 >= tile.k0 && j0 + 16 <= tile.k1) continue;
+      const int jv = j0 + 8 * ((lane & 1) ^ ((lane >> 4) & 1));  // the half of the piece at this lane's position
+      u32x4 msk;
+#pragma unroll
+      for (int e = 0; e < 4; ++e) {
+        const bool lo = jv + 2 * e >= tile.k0 && jv + 2 * e < tile.k1;
+        const bool hi = jv + 2 * e + 1 >= tile.k0 && jv + 2 * e + 1 < tile.k1;
+        msk[e] = (lo ? 0xffffu : 0u) | (hi ? 0xffff0000u : 0u);
+      }
 #pragma unroll
       for (int q = 0; q < 4; ++q) {
-        *reinterpret_cast<u32x4*>(st + (16 * t + 4 * q + wave) * kRowB + lane * 16) = kreg[4 * t + q];
-        const int c = 256 * q + tid, dim = c >> 1;
-        *reinterpret_cast<u32x4*>(st + kKStage + t * kVSub + dim * 32 + (dim >> 3) * 16 + (c & 1) * 16) = vreg[4 * t + q];
+        u32x4* p = reinterpret_cast<u32x4*>(lds + stage * kStage + kKStage + t * kVSub + wave * 4096 + q * 1024 + lane * 16);
+        *p = *p & msk;
       }
+    }
   };
 
-  // ---- operand reads: per-lane byte offsets inside a stage
-  const int prow = (l32 & 0x13) | ((l32 & 4) << 1) | ((l32 & 8) >> 1);  // pi(l32)
-  const int koff = prow * kRowB + dw * 2 + hb * 16;                     // + 32 ks
-  const int vdim = dw + l32;
-  const int voff = kKStage + vdim * 32 + (vdim >> 3) * 16 + hb * 16;    // + t kVSub + nt (32 * 32 + 4 * 16)
+  // ---- operand reads: LDS byte addresses (base register + immediate)
+  using lds_u32x4 = const __attribute__((address_space(3))) u32x4;
+  auto lds_ptr = [](uint32_t addr) __attribute__((always_inline)) { return reinterpret_cast<lds_u32x4*>(addr); };
+  // K slice ks = 8 g + j of this wavefront's dims is chunk dw / 8 + 16 g + 2 j + hb of key row pi(l32).
+  uint32_t kaddr[8];
+  {
+    const int prow = (l32 & 0x13) | ((l32 & 4) << 1) | ((l32 & 8) >> 1);  // pi(l32)
+#pragma unroll
+    for (int j = 0; j < 8; ++j) kaddr[j] = lds_base + uint32_t(prow * 1024 + dw * 2 + (((2 * j + hb) ^ (l32 & 15)) << 4));
+  }
+  // V^T operand nt of sub-block t: keys 8 hb .. + 7 of dim dw + 32 nt + l32.
+  const uint32_t vaddr = lds_base + uint32_t(kKStage + (dw + l32) * 32 + ((hb ^ ((l32 >> 3) & 1)) << 4));
 
   f32x16 acc[NT];
   float m_run = -INFINITY, l_run = 0.0f;  // l_run: this lane's share (16 of every 32 keys) of the row's sum
@@ -178,15 +201,33 @@ __global__ __launch_bounds__(256, 1) void attn_tiled512_kernel(const KArgs a, in
 #pragma unroll
     for (int i = 0; i < 16; ++i) acc[nt][i] = 0.0f;
 
-  auto compute = [&](int step, int stage) __attribute__((always_inline)) {
-    const char* st = lds + stage * kStage;
+  // A step's matrix work is 32 operand reads from LDS, each feeding one matrix instruction, in 4 groups of 8
+  // through two register buffers: K slices 0..7, K slices 8..15, V^T of sub-block 0, V^T of sub-block 1.
+  // The reads of a group are in flight while the matrix cores consume the group before it; the V^T reads
+  // do not depend on the softmax and cover the exchange of the partial scores.
+  u32x4 ring[2][8];
+  auto compute = [&]<int S>(int step, std::integral_constant<int, S>) __attribute__((always_inline)) {
+#pragma unroll
+    for (int j = 0; j < 8; ++j) ring[0][j] = *lds_ptr(kaddr[j] + uint32_t(S * kStage));
+#pragma unroll
+    for (int j = 0; j < 8; ++j) ring[1][j] = *lds_ptr(kaddr[j] + uint32_t(S * kStage + 256));
+    __builtin_amdgcn_sched_barrier(0);
     // s[4 i + j] is S^T row 8 i + 4 hb + j, which is key 16 (i / 2) + 8 hb + 4 (i % 2) + j of the step:
     // s[8 t + e] is key 8 hb + e of sub-block t.
     f32x16 s;
 #pragma unroll
     for (int i = 0; i < 16; ++i) s[i] = 0.0f;
 #pragma unroll
-    for (int ks = 0; ks < KS; ++ks) s = mfma32x16<DT>(*reinterpret_cast<const u32x4*>(st + koff + 32 * ks), qf[ks], s);
+    for (int j = 0; j < 8; ++j) s = mfma32x16<DT>(ring[0][j], qf[j], s);
+    __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+    for (int j = 0; j < 8; ++j) ring[0][j] = *lds_ptr(vaddr + uint32_t(S * kStage + j * 1024));
+    __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+    for (int j = 0; j < 8; ++j) s = mfma32x16<DT>(ring[1][j], qf[8 + j], s);
+    __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+    for (int j = 0; j < 8; ++j) ring[1][j] = *lds_ptr(vaddr + uint32_t(S * kStage + kVSub + j * 1024));
     // The other half of the dims: through LDS, added in the same order in both wavefronts of the pair.
 #pragma unroll
     for (int v = 0; v < 4; ++v) xch[(wave * 4 + v) * 64 + lane] = f32x4{s[4 * v], s[4 * v + 1], s[4 * v + 2], s[4 * v + 3]};
@@ -227,21 +268,22 @@ __global__ __launch_bounds__(256, 1) void attn_tiled512_kernel(const KArgs a, in
         s[8 * t + e] = vis ? s[8 * t + e] : -INFINITY;
       }
     }
-    // ---- online softmax; the two lanes of a row (hb = 0, 1) agree on the maximum
+    // ---- online softmax; the two lanes of a row (hb = 0, 1) agree on the maximum. The running reference
+    // m_run only moves when some row's maximum exceeds it by more than 8 (log2 units): P stays below
+    // 2^8 and the 128 accumulator registers are rescaled a handful of times per row.
     float mx = -INFINITY;
 #pragma unroll
     for (int i = 0; i < 16; ++i) mx = fmaxf(mx, s[i]);
     mx *= a.scale_log2;  // scale > 0: the max commutes with it
-    mx = fmaxf(mx, __shfl_xor(mx, 32));
-    const float m_new = fmaxf(m_run, mx);
-    const float m_safe = (m_new == -INFINITY) ? 0.0f : m_new;
-    if (__any(m_new > m_run)) {
-      const float corr = fast_exp2(m_run - m_safe);  // -inf -> 0: nothing accumulated yet
+    if (__any(mx > m_run + 8.0f)) {
+      const float m_new = fmaxf(m_run, fmaxf(mx, __shfl_xor(mx, 32)));
+      const float corr = (m_new == -INFINITY) ? 1.0f : fast_exp2(m_run - m_new);  // m_run = -inf -> 0: nothing accumulated yet
       l_run *= corr;
 #pragma unroll
       for (int nt = 0; nt < NT; ++nt) acc[nt] *= corr;
       m_run = m_new;
     }
+    const float m_safe = (m_run == -INFINITY) ? 0.0f : m_run;
     u32x4 pb[2];
     float ps = 0.0f;
 #pragma unroll
@@ -255,27 +297,38 @@ __global__ __launch_bounds__(256, 1) void attn_tiled512_kernel(const KArgs a, in
       pb[t] = u32x4{pack2<DT>(p[0], p[1]), pack2<DT>(p[2], p[3]), pack2<DT>(p[4], p[5]), pack2<DT>(p[6], p[7])};
     }
     l_run += ps;
+    __builtin_amdgcn_sched_barrier(0);
     // ---- O^T += V^T . P^T over this wavefront's dims
 #pragma unroll
-    for (int t = 0; t < 2; ++t)
+    for (int nt = 0; nt < NT; ++nt) acc[nt] = mfma32x16<DT>(ring[0][nt], pb[0], acc[nt]);
 #pragma unroll
-      for (int nt = 0; nt < NT; ++nt)
-        acc[nt] = mfma32x16<DT>(*reinterpret_cast<const u32x4*>(st + voff + t * kVSub + nt * (32 * 32 + 4 * 16)), pb[t], acc[nt]);
+    for (int nt = 0; nt < NT; ++nt) acc[nt] = mfma32x16<DT>(ring[1][nt], pb[1], acc[nt]);
   };
 
-  // At the top of iteration i stage i % 2 holds step i. The loads of step i + 1 are in flight during the
-  // step's matrix work and go into the other stage behind it; one barrier publishes them (and retires
-  // every read of the exchange area), the barrier inside compute() covers the exchange itself.
+  // At the top of iteration i stage i % 2 holds step i and every wavefront has left the other stage: the
+  // loads of step i + 1 go straight into it while step i is in the matrix cores. The barrier at the end
+  // publishes them; the barrier inside compute() covers the exchange of the partial scores.
+  auto iter = [&]<int S>(int i, std::integral_constant<int, S> sc) __attribute__((always_inline)) {
+    if (i + 1 < n_steps) fill(i + 1, S ^ 1);
+    compute(i, sc);
+    wait_loads();
+    if (i + 1 < n_steps) fix(i + 1, S ^ 1);
+    __syncthreads();
+  };
   if (n_steps > 0) {
-    gload(0);
-    sstore(0);
+    fill(0, 0);
+    wait_loads();
+    fix(0, 0);
   }
   __syncthreads();
-  for (int i = 0; i < n_steps; ++i) {
-    if (i + 1 < n_steps) gload(i + 1);
-    compute(i, i & 1);
-    if (i + 1 < n_steps) sstore((i + 1) & 1);
-    __syncthreads();
+  {
+    int i = 0;
+#pragma nounroll
+    for (; i + 2 <= n_steps; i += 2) {
+      iter(i, std::integral_constant<int, 0>{});
+      iter(i + 1, std::integral_constant<int, 1>{});
+    }
+    if (i < n_steps) iter(i, std::integral_constant<int, 0>{});
   }
 
   // ---- output: lane (row l32, half hb) holds dims dw + 32 nt + 8 i + 4 hb + j at acc[nt][4 i + j]
