@@ -355,7 +355,8 @@ int esp_attn_prep(const esp_prep_params* p, const float* X, const float* qn_w, c
                   void* kv_pool, int32_t n_rows, void* stream, char* err, size_t errlen) {
   if (!p) return fail(err, errlen, ESP_EINVAL, "params is NULL");
   if (p->H <= 0 || p->Hkv <= 0) return fail(err, errlen, ESP_EINVAL, "H=%d Hkv=%d", p->H, p->Hkv);
-  if (p->head_dim != 128 && p->head_dim != 256) return fail(err, errlen, ESP_EUNSUPPORTED, "head_dim %d (128 or 256)", p->head_dim);
+  if (p->head_dim != 128 && p->head_dim != 256 && p->head_dim != 512)
+    return fail(err, errlen, ESP_EUNSUPPORTED, "head_dim %d (128, 256 or 512)", p->head_dim);
   if (p->dtype != ESP_F16 && p->dtype != ESP_BF16) return fail(err, errlen, ESP_EINVAL, "dtype %d", p->dtype);
   const int HD = p->head_dim;
   if (p->x_ld % 4 || p->q_off % 4 || p->q_hs % 4 || p->k_off % 4 || p->v_off % 4 || p->q_off < 0 || p->k_off < 0 || p->v_off < 0)
@@ -365,9 +366,10 @@ int esp_attn_prep(const esp_prep_params* p, const float* X, const float* qn_w, c
     return fail(err, errlen, ESP_EINVAL, "x_ld %d does not hold the q / k / v columns", p->x_ld);
   if (p->q_ld < p->H * HD || p->q_ld % 4 || p->kv_ld < p->Hkv * HD || p->kv_ld % 4)
     return fail(err, errlen, ESP_EINVAL, "q_ld %d / kv_ld %d", p->q_ld, p->kv_ld);
-  const int rd = p->rope_dims;
-  if (rd < 0 || rd > HD || (rd != 0 && (rd < 8 || (rd & (rd - 1)))))
-    return fail(err, errlen, ESP_EINVAL, "rope_dims %d: 0 or a power of two in [8, head_dim]", rd);
+  if (HD == 512 && (p->q_ld % 8 || p->kv_ld % 8)) return fail(err, errlen, ESP_EINVAL, "q_ld %d / kv_ld %d: multiples of 8 at head_dim 512", p->q_ld, p->kv_ld);
+  const int rd = p->rope_dims, rd_min = HD == 512 ? 16 : 8;  // a lane holds 4 consecutive dims (8 at head_dim 512): half of rope_dims is a multiple of that
+  if (rd < 0 || rd > HD || (rd != 0 && (rd < rd_min || (rd & (rd - 1)))))
+    return fail(err, errlen, ESP_EINVAL, "rope_dims %d: 0 or a power of two in [%d, head_dim]", rd, rd_min);
   if (n_rows < 0) return fail(err, errlen, ESP_EINVAL, "negative count");
   if (n_rows == 0) return ESP_OK;
   if (!X || !qn_w || !kn_w || !Q || !Kb || !Vb) return fail(err, errlen, ESP_EINVAL, "X, qn_w, kn_w, Q, Kb, Vb must not be NULL");

@@ -24,6 +24,8 @@
 // staged in LDS and leaves as one 16-byte store per (head, dim); any other
 // arrangement (decode rows of different sequences, a row saved into two slots)
 // takes element stores.
+#include <type_traits>
+
 #include "common.hpp"
 
 namespace esp {
@@ -34,9 +36,10 @@ constexpr int kPrepRows = 8;
 template <int DT, int HD>
 __global__ __launch_bounds__(256) void attn_prep_kernel(const PrepArgs a, int n_rows) {
   constexpr int R = kPrepRows;
-  constexpr int LPH = HD / 4;     // lanes per head
-  constexpr int HPP = 256 / LPH;  // heads of the workgroup
-  __shared__ float2 cs[R][128];   // (cos, sin) per row and frequency
+  constexpr int EPL = HD > 256 ? 8 : 4;  // consecutive dims per lane: a head never spans more than one wavefront
+  constexpr int LPH = HD / EPL;          // lanes per head
+  constexpr int HPP = 256 / LPH;         // heads of the workgroup
+  __shared__ float2 cs[R][HD / 2];       // (cos, sin) per row and frequency
   __shared__ int run_ok;
   __shared__ __attribute__((aligned(16))) uint16_t vstage[R][HPP * HD];  // the workgroup's V heads, for the transposed append
   const esp_prep_params& p = a.p;
@@ -64,40 +67,47 @@ __global__ __launch_bounds__(256) void attn_prep_kernel(const PrepArgs a, int n_
   __syncthreads();
   run = run_ok != 0;  // the same value everywhere; through LDS so that the compiler treats it as uniform
 
-  const int li = tid % LPH, d0 = 4 * li;
+  const int li = tid % LPH, d0 = EPL * li;
   const int n_slots = p.H + 2 * p.Hkv;
   const int slot0 = blockIdx.y * HPP;  // the workgroup's first head: queries, then keys, then values
   for (int slot = slot0 + tid / LPH; slot < n_slots; slot += n_slots) {  // at most one head per thread
     const int kind = slot < p.H ? 0 : (slot < p.H + p.Hkv ? 1 : 2);  // q, k, v
     const int h = kind == 0 ? slot : (kind == 1 ? slot - p.H : slot - p.H - p.Hkv);
     const size_t col = size_t(kind == 0 ? p.q_off + h * p.q_hs : (kind == 1 ? p.k_off : p.v_off) + h * HD) + d0;
-    f32x4 xv[R];
+    f32x4 xv[R][EPL / 4];
 #pragma unroll
     for (int r = 0; r < R; ++r)
-      xv[r] = r < rows ? __builtin_nontemporal_load(reinterpret_cast<const f32x4*>(a.X + size_t(row0 + r) * p.x_ld + col))
-                       : f32x4{0, 0, 0, 0};  // read once: no reason to keep it in a cache
-    f32x4 w = {1, 1, 1, 1};
-    if (kind != 2) w = *reinterpret_cast<const f32x4*>((kind == 0 ? a.qn_w : a.kn_w) + d0);
+#pragma unroll
+      for (int v = 0; v < EPL / 4; ++v)
+        xv[r][v] = r < rows ? __builtin_nontemporal_load(reinterpret_cast<const f32x4*>(a.X + size_t(row0 + r) * p.x_ld + col) + v)
+                            : f32x4{0, 0, 0, 0};  // read once: no reason to keep it in a cache
+    float w[EPL];
+#pragma unroll
+    for (int i = 0; i < EPL; ++i) w[i] = kind != 2 ? (kind == 0 ? a.qn_w : a.kn_w)[d0 + i] : 1.0f;
 #pragma unroll
     for (int r = 0; r < R; ++r) {
       if (r >= rows) break;
       const size_t row = size_t(row0 + r);
-      float x[4] = {xv[r][0], xv[r][1], xv[r][2], xv[r][3]};
+      float x[EPL];
+#pragma unroll
+      for (int i = 0; i < EPL; ++i) x[i] = xv[r][i / 4][i % 4];
       if (kind != 2 || p.v_norm) {
-        float ss = x[0] * x[0] + x[1] * x[1] + x[2] * x[2] + x[3] * x[3];
+        float ss = 0.0f;
+#pragma unroll
+        for (int i = 0; i < EPL; ++i) ss += x[i] * x[i];
 #pragma unroll
         for (int o = LPH / 2; o >= 1; o >>= 1) ss += __shfl_xor(ss, o);
         const float inv = rsqrtf(ss / float(HD) + p.eps);
 #pragma unroll
-        for (int i = 0; i < 4; ++i) x[i] = kind == 2 ? x[i] * inv : x[i] * inv * w[i];
+        for (int i = 0; i < EPL; ++i) x[i] = kind == 2 ? x[i] * inv : x[i] * inv * w[i];
       }
       if (kind != 2 && half > 0) {
-        // The partner of dim d < half is d + half: half / 4 lanes away. Every lane of the head takes
+        // The partner of dim d < half is d + half: half / EPL lanes away. Every lane of the head takes
         // part in the exchange; only the rotating dims use it.
         const bool lower = d0 < half;
 #pragma unroll
-        for (int i = 0; i < 4; ++i) {
-          const float partner = __shfl_xor(x[i], half / 4);
+        for (int i = 0; i < EPL; ++i) {
+          const float partner = __shfl_xor(x[i], half / EPL);
           if (d0 < p.rope_dims) {
             const float2 t = cs[r][(lower ? d0 : d0 - half) + i];
             x[i] = lower ? x[i] * t.x - partner * t.y : x[i] * t.x + partner * t.y;
@@ -106,17 +116,20 @@ __global__ __launch_bounds__(256) void attn_prep_kernel(const PrepArgs a, int n_
       }
       if (kind == 0) {
 #pragma unroll
-        for (int i = 0; i < 4; ++i) x[i] *= p.q_scale;
+        for (int i = 0; i < EPL; ++i) x[i] *= p.q_scale;
       }
-      const u32x2 out = {pack2<DT>(x[0], x[1]), pack2<DT>(x[2], x[3])};
+      using out_t = std::conditional_t<EPL == 8, u32x4, u32x2>;  // EPL storage elements
+      out_t out;
+#pragma unroll
+      for (int i = 0; i < EPL / 2; ++i) out[i] = pack2<DT>(x[2 * i], x[2 * i + 1]);
       if (kind == 0) {
-        *reinterpret_cast<u32x2*>(a.Q + row * size_t(p.q_ld) + size_t(h) * HD + d0) = out;
+        *reinterpret_cast<out_t*>(a.Q + row * size_t(p.q_ld) + size_t(h) * HD + d0) = out;
         continue;
       }
-      *reinterpret_cast<u32x2*>((kind == 1 ? a.Kb : a.Vb) + row * size_t(p.kv_ld) + size_t(h) * HD + d0) = out;
+      *reinterpret_cast<out_t*>((kind == 1 ? a.Kb : a.Vb) + row * size_t(p.kv_ld) + size_t(h) * HD + d0) = out;
       // The folded append: the same bits into the row's pool entries (a row saved into two slots has two).
       if (kind == 2 && run) {
-        *reinterpret_cast<u32x2*>(&vstage[r][(slot - slot0) * HD + d0]) = out;
+        *reinterpret_cast<out_t*>(&vstage[r][(slot - slot0) * HD + d0]) = out;
         continue;
       }
 #pragma unroll
@@ -125,13 +138,14 @@ __global__ __launch_bounds__(256) void attn_prep_kernel(const PrepArgs a, int n_
         if (b < 0) continue;
         uint16_t* hb = a.pool + p.kv_base + (size_t(b) * p.Hkv + h) * size_t(2 * p.bt * HD);
         if (kind == 1) {
-          *reinterpret_cast<u32x2*>(hb + size_t(ps) * HD + d0) = out;
+          *reinterpret_cast<out_t*>(hb + size_t(ps) * HD + d0) = out;
         } else {
           uint16_t* vt = hb + vt_elem(p.bt, HD, ps, d0);
-          vt[0] = uint16_t(out[0] & 0xffffu);
-          vt[kVtDim] = uint16_t(out[0] >> 16);
-          vt[2 * kVtDim] = uint16_t(out[1] & 0xffffu);
-          vt[3 * kVtDim] = uint16_t(out[1] >> 16);
+#pragma unroll
+          for (int i = 0; i < EPL / 2; ++i) {
+            vt[(2 * i) * kVtDim] = uint16_t(out[i] & 0xffffu);
+            vt[(2 * i + 1) * kVtDim] = uint16_t(out[i] >> 16);
+          }
         }
       }
     }
@@ -157,12 +171,14 @@ __global__ __launch_bounds__(256) void attn_prep_kernel(const PrepArgs a, int n_
 
 hipError_t launch_attn_prep(const PrepArgs& a, int n_rows, hipStream_t st) {
   const int dt = a.p.dtype, HD = a.p.head_dim;
-  const int hpp = 256 / (HD / 4), n_slots = a.p.H + 2 * a.p.Hkv;
+  const int hpp = 256 / (HD / (HD > 256 ? 8 : 4)), n_slots = a.p.H + 2 * a.p.Hkv;
   const dim3 grid((n_rows + kPrepRows - 1) / kPrepRows, (n_slots + hpp - 1) / hpp), block(256);
   if (dt == ESP_F16 && HD == 128) launch_timed(attn_prep_kernel<ESP_F16, 128>, grid, block, 0, st, a, n_rows);
   else if (dt == ESP_F16 && HD == 256) launch_timed(attn_prep_kernel<ESP_F16, 256>, grid, block, 0, st, a, n_rows);
   else if (dt == ESP_BF16 && HD == 128) launch_timed(attn_prep_kernel<ESP_BF16, 128>, grid, block, 0, st, a, n_rows);
   else if (dt == ESP_BF16 && HD == 256) launch_timed(attn_prep_kernel<ESP_BF16, 256>, grid, block, 0, st, a, n_rows);
+  else if (dt == ESP_F16 && HD == 512) launch_timed(attn_prep_kernel<ESP_F16, 512>, grid, block, 0, st, a, n_rows);
+  else if (dt == ESP_BF16 && HD == 512) launch_timed(attn_prep_kernel<ESP_BF16, 512>, grid, block, 0, st, a, n_rows);
   else return hipErrorInvalidValue;
   return hipGetLastError();
 }

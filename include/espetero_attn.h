@@ -96,7 +96,9 @@ typedef struct esp_kvsave {
 typedef struct esp_attn_params {
   int32_t H;             /* query heads */
   int32_t Hkv;           /* KV heads; H % Hkv == 0, group G = H / Hkv */
-  int32_t head_dim;      /* 128 or 256 */
+  int32_t head_dim;      /* 128, 256 or 512 (512: the g4_attention512_s* / g4_attention_dec512_g* instantiations,
+                            80_:355-358, :561-564; at most 16 packed rows on the streaming kernel, 64-row tiles
+                            on the tiled one: esp_attn_plan_hint's max_rows) */
   int32_t dtype;         /* ESP_F16 | ESP_BF16: element type of Q, Kb, Vb, pool and O */
   int32_t q_ld;          /* Q / O row stride in elements (>= H * head_dim) */
   int32_t kv_ld;         /* Kb / Vb row stride in elements (>= Hkv * head_dim) */
@@ -232,7 +234,8 @@ typedef struct esp_prep_params {
   int32_t v_off;     /* column of value head 0 */
   int32_t q_ld;      /* Q output row stride, elements */
   int32_t kv_ld;     /* Kb / Vb output row stride, elements */
-  int32_t rope_dims; /* 64 in 40_:58-71, head_dim in 80_:99-104 and 82_:75-82, 0: no rotation; a power of two >= 8 */
+  int32_t rope_dims; /* 64 in 40_:58-71, head_dim in 80_:99-104 and 82_:75-82, 0: no rotation; a power of two >= 8
+                        (>= 16 at head_dim 512, g4_attn_prep512, 80_:113) */
   int32_t v_norm;    /* 1: 80_:92-96; 0: 40_:81-83, 82_:58-62 */
   int32_t bt;        /* tokens per KV block, for the folded append */
   float eps;

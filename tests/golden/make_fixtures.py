@@ -41,6 +41,8 @@ ATTENTION = {
     "window_rings": (108, 2, 1, 128, abi.ESP_F16, 16, [(100, 1), (45, 1)], dict(rows_per_tile=1, window=48, ring_layer=True)),
     "bidi_span": (109, 2, 1, 128, abi.ESP_F16, 16, [(20, 12)], dict(rows_per_tile=8, bidi=1, desc_fn=lambda M: synth.image_desc(M, 3, 9))),
     "wide_tree": (110, 2, 1, 128, abi.ESP_F16, 16, [(30, 10)], dict(rows_per_tile=8, desc_fn=lambda M: synth.verify_desc(M, 6))),
+    "decode_hd512_g8": (111, 8, 1, 512, abi.ESP_F16, 16, [(75, 1), (20, 1)], dict(rows_per_tile=1)),
+    "prefill_hd512": (112, 2, 1, 512, abi.ESP_BF16, 16, [(37, 21)], dict(rows_per_tile=64)),
 }
 
 
@@ -57,9 +59,10 @@ def attention_fixtures():
 
 
 def prep_fixtures():
-    for kind, H, Hkv, HD, dtype in (("qwen35", 3, 1, 256, abi.ESP_F16), ("gemma", 2, 1, 128, abi.ESP_BF16), ("omni", 5, 1, 128, abi.ESP_F16)):
+    for kind, H, Hkv, HD, dtype in (("qwen35", 3, 1, 256, abi.ESP_F16), ("gemma", 2, 1, 128, abi.ESP_BF16), ("omni", 5, 1, 128, abi.ESP_F16),
+                                    ("gemma512", 4, 1, 512, abi.ESP_F16)):
         n = 7
-        p, a = synth.make_prep(kind, H, Hkv, HD, dtype, n, seed=120 + H)
+        p, a = synth.make_prep("gemma" if kind == "gemma512" else kind, H, Hkv, HD, dtype, n, seed=120 + H)
         Q, K, V = ob.attn_prep_f64(p, a["X"], a["qn_w"], a["kn_w"], a["pos"], a["inv_freq"], a["rope_sel"], n)
         meta = {f[0]: getattr(p, f[0]) for f in abi.PrepParams._fields_}
         sel = np.zeros(0, np.int32) if a["rope_sel"] is None else a["rope_sel"]

@@ -15,7 +15,7 @@ from helpers import GOLDEN, golden_names, load_golden_attention, tol_for
 
 
 def test_the_fixture_set_is_complete():
-    assert len(golden_names("attention")) == 10 and golden_names("prep") == ["gemma", "omni", "qwen35"]
+    assert len(golden_names("attention")) == 12 and golden_names("prep") == ["gemma", "gemma512", "omni", "qwen35"]
     assert os.path.exists(os.path.join(GOLDEN, "gate.npz")) and os.path.exists(os.path.join(GOLDEN, "planner.json"))
 
 

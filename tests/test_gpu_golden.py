@@ -27,9 +27,10 @@ def test_attention_matches_the_fixture(name):
     print(f"golden attention {name}", flush=True)
     got = ob.to_f32(run_case(c), c.params.dtype)
     assert np.abs(got - want).max() <= tol_for(c.params.dtype)
-    if c.params.rows_per_tile * (c.params.H // c.params.Hkv) <= 32:   # also as 128-row tiles through the tiled kernel
-        c.params.rows_per_tile = 128
-        got = ob.to_f32(run_case(c, host.options_mi355x(128, 8)), c.params.dtype)
+    if c.params.rows_per_tile * (c.params.H // c.params.Hkv) <= 32:   # also as the largest tiles of the tiled kernel
+        rows = device.plan_hint3(c.params)[2]
+        c.params.rows_per_tile = rows
+        got = ob.to_f32(run_case(c, host.options_mi355x(rows, 8)), c.params.dtype)
         assert np.abs(got - want).max() <= tol_for(c.params.dtype)
 
 

@@ -10,7 +10,8 @@ from oracle import binding as ob
 pytestmark = pytest.mark.gpu
 
 
-@pytest.mark.parametrize("HD,Hkv,bt,dtype", [(128, 4, 16, abi.ESP_F16), (256, 2, 16, abi.ESP_F16), (128, 8, 64, abi.ESP_BF16)])
+@pytest.mark.parametrize("HD,Hkv,bt,dtype", [(128, 4, 16, abi.ESP_F16), (256, 2, 16, abi.ESP_F16), (128, 8, 64, abi.ESP_BF16),
+                                             (512, 2, 16, abi.ESP_F16), (512, 1, 64, abi.ESP_BF16)])
 def test_relayout_gather_save_copy_are_bit_exact(HD, Hkv, bt, dtype):
     from gpu_utils import dev_u16, to_host_u16
     device.init(0)

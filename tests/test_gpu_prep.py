@@ -1,7 +1,8 @@
 """esp_attn_prep on the GPU against the CPU checker, through the C ABI. Bar: every output within one
 unit in the last place of the storage type of the checker's (rsqrt / sin / cos differ in their last
-fp32 bits between the two, which can move a rounding); the folded append bit-identical to esp_kv_save
-of the kernel's own outputs."""
+fp32 bits between the two, which can move a rounding), or, where a rotation cancels to a small value,
+within half a unit in the last place at 1.0 in absolute terms; the folded append bit-identical to
+esp_kv_save of the kernel's own outputs."""
 import numpy as np
 import pytest
 import torch
@@ -37,7 +38,8 @@ def _run_gpu(p, a, n_rows, table=None, pool=None):
 
 
 @pytest.mark.parametrize("kind,H,Hkv,HD", [("qwen35", 8, 2, 256), ("gemma", 16, 8, 256), ("gemma", 8, 2, 128),
-                                            ("omni", 40, 8, 128), ("omni", 3, 1, 128)])
+                                            ("omni", 40, 8, 128), ("omni", 3, 1, 128),
+                                            ("gemma", 16, 2, 512), ("omni", 5, 1, 512)])  # 512: g4_attn_prep512, 80_gemma.metal:113
 @pytest.mark.parametrize("dtype", [abi.ESP_F16, abi.ESP_BF16])
 def test_prep_matches_checker(kind, H, Hkv, HD, dtype):
     device.init(0)
@@ -46,9 +48,13 @@ def test_prep_matches_checker(kind, H, Hkv, HD, dtype):
     print(f"prep {kind} H={H} Hkv={Hkv} HD={HD} dtype={dtype}", flush=True)
     want = ob.attn_prep(p, a["X"], a["qn_w"], a["kn_w"], a["pos"], a["inv_freq"], a["rope_sel"], n_rows)
     got = _run_gpu(p, a, n_rows)
+    half_ulp_at_1 = 2.0 ** -11 if dtype == abi.ESP_F16 else 2.0 ** -8
     for g, w, name in zip(got, want, "QKV"):
         u = _ulps(g, w, dtype)
-        assert u.max() <= 1, (name, int(u.max()))
+        # One unit in the last place; where a rotation cancels (x cos - partner sin near 0) the result is small
+        # and its last place is finer than the error of its two terms: there the absolute difference counts.
+        far = (u > 1) & (np.abs(ob.to_f32(g, dtype) - ob.to_f32(w, dtype)) > half_ulp_at_1)
+        assert not far.any(), (name, int(u.max()))
         assert (u > 0).mean() < 0.02, (name, float((u > 0).mean()))       # and almost all bit-identical
     assert np.array_equal(got[2], want[2]) or p.v_norm                    # a plain cast has nothing to differ in
 
@@ -79,7 +85,8 @@ def test_prep_folded_append_is_bitwise_kv_save():
 
 
 @pytest.mark.parametrize("kind,H,Hkv,HD,dtype,first", [("omni", 10, 2, 128, abi.ESP_BF16, 0), ("qwen35", 4, 2, 256, abi.ESP_F16, 0),
-                                                       ("gemma", 4, 4, 256, abi.ESP_F16, 8), ("omni", 6, 2, 128, abi.ESP_F16, 5)])
+                                                       ("gemma", 4, 4, 256, abi.ESP_F16, 8), ("omni", 6, 2, 128, abi.ESP_F16, 5),
+                                                       ("gemma", 8, 2, 512, abi.ESP_F16, 0), ("gemma", 4, 1, 512, abi.ESP_BF16, 3)])
 def test_prep_folded_append_of_a_prefill_chunk(kind, H, Hkv, HD, dtype, first):
     """Rows at consecutive positions of scattered pages, as a prefill chunk appends them: groups of 8 rows
     at 8-aligned positions leave as 16-byte stores of the transposed V plane, the ragged last group and

@@ -9,7 +9,7 @@ import pytest
 from espetero_amd import abi, synth
 from oracle import binding as ob
 
-KINDS = [("qwen35", 256), ("gemma", 256), ("gemma", 128), ("omni", 128)]
+KINDS = [("qwen35", 256), ("gemma", 256), ("gemma", 128), ("omni", 128), ("gemma", 512)]
 
 
 def _run(kind, HD, dtype, n_rows=9, seed=5, **kw):
