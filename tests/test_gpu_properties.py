@@ -241,6 +241,42 @@ def test_c4_prefill_sliding_and_global_sampled_rows():
         assert np.abs(got - want).max() <= 2e-3, name
 
 
+# ---------------------------------------------------------------- head dim 512 (Gemma 4 global layers), full size
+def test_g4_global512_decode_and_prefill_at_full_size():
+    """Float64 brute force on sampled sequences / rows, split-count invariance of the decode, and row 0 of
+    a prefill chunk == the decode step on the same cache (the tiled and the streaming kernel agree)."""
+    wd = _workload("g4_global512_decode")
+    Od = _f32(_run(wd))
+    for seq in (0, 6):
+        K, V = _gather(wd, seq, wd.passes[0].blocks)
+        want = _brute_rows(wd, seq, [0], K, V)
+        b = int(wd.trees[seq]["base"])
+        assert np.abs(Od[b:b + 1] - want).max() <= 2e-3
+    p = wd.params
+    for wgs in (64, 2048):
+        tiles, jobs, n_parts = host.plan_tiles(wd.trees, p.Hkv, 0, None, host.options_mi355x(1, wgs))
+        dp = device.DevicePass(p, wd.trees, tiles, jobs, n_parts, wd.n_rows, wd.tables[0], None, None)
+        assert np.abs(_f32(_run(wd, dp)) - Od).max() <= 1e-3
+    del wd
+    wp = _workload("g4_global512_prefill")
+    Op = _f32(_run(wp))
+    K, V = _gather(wp, 3, wp.passes[0].blocks)
+    rows = [0, 1, 63, 64, 700, 1023]
+    want = _brute_rows(wp, 3, rows, K, V)
+    b = int(wp.trees[3]["base"])
+    assert np.abs(np.stack([Op[b + r] for r in rows]) - want).max() <= 2e-3
+    # row 0 of sequence 3 as a one-row decode pass over the same pool and table
+    pd = synth.make_params(p.H, p.Hkv, p.head_dim, p.dtype, p.bt, rows_per_tile=1)
+    t = wp.trees[3]
+    trees = np.array([(0, int(t["P"]), int(t["table"]), 1)], abi.TREE_DT)
+    tiles, jobs, n_parts = host.plan_tiles(trees, pd.Hkv, 0, None, host.options_mi355x(1, device.plan_hint(pd)[0]))
+    dp = device.DevicePass(pd, trees, tiles, jobs, n_parts, 1, wp.tables[0], None, None)
+    O1 = torch.zeros_like(wp.Q[b:b + 1])
+    dp.run(wp.Q[b:b + 1].contiguous(), wp.Kb[b:b + 1].contiguous(), wp.Vb[b:b + 1].contiguous(), wp.pool, O1)
+    torch.cuda.synchronize()
+    assert np.abs(_f32(O1) - Op[b:b + 1]).max() <= 1e-3
+
+
 def test_c1_single_decode_matches_checker_exactly_sized():
     """The reference's own CPU-runnable shape: small enough for the checker to run whole."""
     from gpu_utils import run_case
