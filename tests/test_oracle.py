@@ -66,6 +66,7 @@ CASES = [
     dict(seqs=((90, 1), (200, 1)), window=64, ring_layer=True),      # sliding window, slot rings
     dict(seqs=((41, 7),), H=10, Hkv=2, dtype=abi.ESP_BF16),          # GQA 5, bf16
     dict(seqs=((33, 2),), H=4, Hkv=2, HD=256),                       # head_dim 256
+    dict(seqs=((40, 3),), H=8, Hkv=1, HD=512),                       # head_dim 512, GQA 8 (Gemma 4 global layers)
     dict(seqs=((64, 9),), bt=64),                                    # the reference's default block size
     dict(seqs=((20, 8),), H=4, Hkv=2, bidi=1, desc_fn=lambda M: synth.image_desc(M, 2, 6)),  # bidirectional span
 ]
