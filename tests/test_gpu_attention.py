@@ -133,9 +133,11 @@ def test_tiled_kernel_matches_checker(kw):
     dict(seqs=((128, 128),), bt=64, H=4, Hkv=2),
     dict(seqs=((100, 140),), H=2, Hkv=1, bidi=1, desc_fn=lambda M: synth.image_desc(M, 10, 90)),   # bidirectional span
     dict(seqs=((1203, 64), (700, 40)), bt=64, H=4, Hkv=2, fill_unused=True),  # long cached ranges, ragged end
+    dict(seqs=((100, 1), (33, 1)), H=32, Hkv=1, rows_per_tile=1),       # G = 32: more packed rows than the streaming kernel takes at 512
+    dict(seqs=((150, 20),), H=4, Hkv=2, rows_per_tile=24),              # tiles smaller than the kernel's 64 rows
 ])
 def test_tiled_kernel_head_dim_512(kw):
-    _check(small_case(seed=44, HD=512, rows_per_tile=64, **kw))
+    _check(small_case(seed=44, HD=512, **{"rows_per_tile": 64, **kw}))
 
 
 def test_tiled_kernel_head_dim_512_split_and_gate():
