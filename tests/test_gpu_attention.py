@@ -57,6 +57,7 @@ def test_stream_kernel_matches_checker(kw):
     dict(seqs=((200, 1),), H=4, Hkv=2, bt=64, rows_per_tile=1),                     # the reference's block size
     dict(seqs=((900, 1), (40, 1)), H=4, Hkv=1, window=128, rows_per_tile=1),        # window (not a Gemma shape; same code)
     dict(seqs=((90, 7),), H=4, Hkv=2, rows_per_tile=8),                             # G = 2, 8-row tiles: batch keys
+    dict(seqs=((700, 4), (33, 4)), H=8, Hkv=1, rows_per_tile=2, desc_fn=lambda M: synth.verify_desc(M, 1)),  # a 4-row verify tree as two 2-row tiles
 ])
 def test_stream_kernel_head_dim_512(kw):
     _check(small_case(seed=37, HD=512, fill_unused=True, **kw))
