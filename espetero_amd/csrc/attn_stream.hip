@@ -298,6 +298,11 @@ __global__ __launch_bounds__(HD >= 512 ? 128 : 256, OCC) void attn_stream_kernel
     }
     f32x4 s[NC][SBU];
     scores(U, s);
+    // The first readers of s sit behind the branches of the visibility rules below.
+#pragma unroll
+    for (int c = 0; c < NC; ++c)
+#pragma unroll
+      for (int sb = 0; sb < SBU; ++sb) mfma_settle(s[c][sb]);
     int kpos[SBU][4];
     if (BATCH && a.window > 0) {
 #pragma unroll

@@ -82,6 +82,22 @@ __device__ __forceinline__ uint16_t pack1(float x) {
 
 __device__ __forceinline__ float fast_exp2(float x) { return __builtin_amdgcn_exp2f(x); }
 
+// Lets the matrix pipeline finish writing `acc` before anything after this point reads it. Matrix
+// instructions are not interlocked against vector instructions that read their result: the compiler
+// pads the distance with wait states, but only sees the instructions of one basic block. Where a branch
+// follows the last matrix instruction and the first reader sits in the branch target, nothing was
+// inserted, and the reader took the accumulator as it was before the last instruction landed
+// (measured: the fourth register of a 16x16x32 result, read 3 instructions after the instruction's
+// issue, lacked the last 32-dim slice of the dot products). Asking for the value in vector registers
+// here, in the block of the matrix instruction, does it: a result the instruction left in vector
+// registers waits out the 32 wait states below (the longest instruction, 16 passes, needs 19); one it
+// left in accumulator registers is copied in front of this statement, in the same block, where the
+// compiler does pad the distance.
+template <typename T>
+__device__ __forceinline__ void mfma_settle(T& acc) {
+  asm volatile("s_nop 15\n\ts_nop 15" : "+v"(acc));
+}
+
 // Everything a kernel of this library reads: the call's device pointers and
 // the per-layer constants, passed by value.
 struct KArgs {

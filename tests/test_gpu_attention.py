@@ -63,6 +63,17 @@ def test_stream_kernel_head_dim_512(kw):
     _check(small_case(seed=37, HD=512, fill_unused=True, **kw))
 
 
+@pytest.mark.parametrize("P,bt", [(10, 32), (15, 32), (74, 32), (26, 64), (15, 16)])
+def test_stream_kernel_partial_unit_at_head_dim_256(P, bt):
+    """A short cache whose keys all sit in one partial 16-key unit: every score counts. (The fourth register of
+    that unit's score tile was once read before the last matrix instruction had written it: keys 3, 7, 11
+    came out with the weight of a dot product short of its last 32 dims, 4e-2 off at P = 10.)"""
+    c = small_case(seed=38, H=2, Hkv=1, HD=256, bt=bt, seqs=((P, 1),), rows_per_tile=1, fill_unused=True)
+    _check(c)
+    c = small_case(seed=39, H=16, Hkv=1, HD=256, bt=bt, seqs=((P, 1), (P + 3, 1)), rows_per_tile=1, dtype=abi.ESP_BF16)
+    _check(c)
+
+
 def test_stream_kernel_reference_planner_records():
     """The kernels accept the reference planner's own records (8-row tiles, 32-key chunks)."""
     c = small_case(seed=32, seqs=((1024, 1),), H=32, Hkv=4, rows_per_tile=8)
