@@ -342,7 +342,7 @@ __global__ __launch_bounds__(256, OCC) void attn_tiled_kernel(const KArgs a, int
         half_full = j0 >= tile.k0 && j0 + 32 <= tile.k1 && (a.window == 0 || qpos_max - j0 < a.window);
       } else if (s0 >= n_c && s0 + 2 <= n_sb) {
         const int j0 = ((a0 + s0 - n_c) << 4) - tree.base;
-        half_full = !batch_window && j0 >= seg_max && j0 + 31 <= rr0 + 32 * wave && j0 >= 0;
+        half_full = !batch_window && j0 >= seg_max && j0 + 31 <= rr0 + 32 * wave && j0 >= tile.b0;
       } else {
         half_full = false;
       }
@@ -360,7 +360,9 @@ __global__ __launch_bounds__(256, OCC) void attn_tiled_kernel(const KArgs a, int
           hi = tile.k1 - 1;
           if (a.window > 0) lo = max(lo, qpos - a.window + 1);
         } else if (batch) {
-          lo = max(d.x, 0);
+          // b0 is the first batch key any row of the tile sees (the window's lower edge; 0 without one). The
+          // first sub-block starts at a multiple of 16 rows at or below it: what lies below b0 is invisible.
+          lo = max(d.x, tile.b0);
           hi = min(k_last, (a.bidi && d.w > 0) ? max(rr, d.w - 1) : rr);
           anc = min(d.z, k_last + 1);
         } else {
@@ -379,7 +381,7 @@ __global__ __launch_bounds__(256, OCC) void attn_tiled_kernel(const KArgs a, int
 #pragma unroll
           for (int e = 0; e < 8; ++e) {
             const int j = jb + e;
-            bool vis = unsigned(e - ea) <= unsigned(ew) || (j >= 0 && j < anc);
+            bool vis = unsigned(e - ea) <= unsigned(ew) || (j >= tile.b0 && j < anc);
             if (batch_window && vis) vis = qpos - a.pos[tree.base + j].x < a.window;
             sv[8 * t + e] = vis ? sv[8 * t + e] : -INFINITY;
           }

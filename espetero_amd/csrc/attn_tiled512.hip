@@ -252,7 +252,7 @@ __global__ __launch_bounds__(256, 1) void attn_tiled512_kernel(const KArgs a, in
         hi = tile.k1 - 1;
         if (a.window > 0) lo = max(lo, qpos - a.window + 1);
       } else if (batch) {
-        lo = max(d.x, 0);
+        lo = max(d.x, tile.b0);  // below b0 (the window's lower edge over the tile's rows) nothing is visible
         hi = min(k_last, (a.bidi && d.w > 0) ? max(rr, d.w - 1) : rr);
         anc = min(d.z, k_last + 1);
       } else {
@@ -263,7 +263,7 @@ __global__ __launch_bounds__(256, 1) void attn_tiled512_kernel(const KArgs a, in
 #pragma unroll
       for (int e = 0; e < 8; ++e) {
         const int j = jb + e;
-        bool vis = (j >= lo && j <= hi) || (j >= 0 && j < anc);
+        bool vis = (j >= lo && j <= hi) || (j >= tile.b0 && j < anc);
         if (batch && a.window > 0 && vis) vis = qpos - a.pos[tree.base + j].x < a.window;
         s[8 * t + e] = vis ? s[8 * t + e] : -INFINITY;
       }

@@ -170,6 +170,16 @@ def test_tiled_kernel_head_dim_512_split_and_gate():
     assert np.abs(whole - want.reshape(c.n_rows, -1)).max() <= 2e-3
 
 
+@pytest.mark.parametrize("HD,rows", [(128, 32), (256, 32), (256, 128), (512, 64)])
+def test_tiled_kernel_one_row_remainder_tile_on_a_windowed_layer(HD, rows):
+    """A chunk of k * rows + 1 rows on a sliding layer: the last tile is one row, its first batch sub-block
+    starts below the window's lower edge, and no other row's position test covers those keys. (They once
+    counted as visible: 0.18 off on that row.)"""
+    for window, ring in ((17, False), (17, True), (40, False)):
+        _check(small_case(seed=46, H=6, Hkv=3, HD=HD, bt=64, seqs=((565, 2 * rows + 3), (300, rows + 1)), rows_per_tile=rows,
+                          window=window, ring_layer=ring, fill_unused=not ring))
+
+
 def test_tiled_kernel_split_tiles_and_combine():
     """A single long-context tile group is split over key ranges and merged."""
     c = small_case(seed=42, seqs=((3000, 100),), H=4, Hkv=2, rows_per_tile=128)
