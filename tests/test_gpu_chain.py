@@ -11,15 +11,19 @@ from oracle import binding as ob
 
 pytestmark = pytest.mark.gpu
 
-H, HKV, HD, BT, K = 8, 2, 128, 16, 10
+K = 10
 P0 = [70, 33, 500, 1030, 16, 0]
+# (query heads, KV heads, head dim, tokens per block, prep arrangement): the benchmark's Qwen shape, a sliding-layer
+# Gemma shape at the reference's block size, and Gemma 4's 512-dim heads (wavefront pairs, open-ended ranges)
+SHAPES = [(8, 2, 128, 16, "omni"), (4, 2, 256, 64, "gemma"), (8, 1, 512, 16, "gemma")]
 
 
-def _setup(seed=12):
+def _setup(shape, seed=12):
+    H, HKV, HD, BT, kind = shape
     rng = np.random.default_rng(seed)
     n = len(P0)
     ap = synth.make_params(H, HKV, HD, abi.ESP_F16, BT, rows_per_tile=1)
-    pp, a = synth.make_prep("omni", H, HKV, HD, abi.ESP_F16, n, seed=seed, bt=BT)
+    pp, a = synth.make_prep(kind, H, HKV, HD, abi.ESP_F16, n, seed=seed, bt=BT)
     nb = [(p + K + BT) // BT for p in P0]                      # room for the K tokens the chain appends
     n_blocks = sum(nb) + 3
     perm = rng.permutation(n_blocks).astype(np.int32)
@@ -41,6 +45,7 @@ def _setup(seed=12):
 
 
 def _host_chain(ap, trees, blocks, pool, Q, Kb, Vb):
+    BT = ap.bt
     """The checker, one step at a time, every record rebuilt on the host. Q / Kb / Vb [K][n][...]: the
     prepared rows of every step (storage bits); each step's K / V row joins the cache after its attention."""
     n = len(trees)
@@ -59,12 +64,15 @@ def _host_chain(ap, trees, blocks, pool, Q, Kb, Vb):
     return np.stack(out), pool
 
 
-def test_device_chain_matches_the_checker_step_by_step_and_replays_identically():
+@pytest.mark.parametrize("shape", SHAPES)
+def test_device_chain_matches_the_checker_step_by_step_and_replays_identically(shape):
     device.init(0)
-    ap, pp, a, trees, blocks, pool_ref, n_blocks, X = _setup()
+    ap, pp, a, trees, blocks, pool_ref, n_blocks, X = _setup(shape)
     n = len(trees)
+    BT = ap.bt
+    print(f"chain shape {shape}", flush=True)
 
-    dev = lambda x: torch.from_numpy(np.ascontiguousarray(x)).cuda()  # noqa: E731
+    dev = lambda x: None if x is None else torch.from_numpy(np.ascontiguousarray(x)).cuda()  # noqa: E731
     ref = dev(pool_ref.view(np.int16))
     pool0 = torch.empty_like(ref)
     device.kv_relayout(ap, ref, abi.ESP_LAYOUT_REFERENCE, pool0, abi.ESP_LAYOUT_NATIVE, n_blocks)
