@@ -241,6 +241,96 @@ def test_fork_shares_blocks_and_copy_on_write_diverges():
     _conservation(e, 16, [a, b])
 
 
+@pytest.mark.parametrize("seed", range(6))
+def test_random_slot_histories_keep_every_slot_readable(seed):
+    """Model-based: random appends (in place, into another slot, after forks), aborted and refused passes, resets.
+    A toy pool holds one token id per (block, position); the pass's own records drive it - copy-on-write pairs
+    first, then the saves - and after every step each slot must read back, through its block list, exactly the
+    tokens it logically holds, the parent's table must read the parent's tokens, and the blocks must add up."""
+    rng = np.random.default_rng(300 + seed)
+    bt = int(rng.choice([16, 32]))
+    n_blocks, n_slots = int(rng.integers(10, 40)), 5
+    e = host.Engine(n_blocks, bt, n_slots)
+    slots = [e.slot_alloc() for _ in range(n_slots)]
+    truth = {s: [] for s in slots}
+    pool = np.full((n_blocks, bt), -1, np.int64)
+    next_tok = [1]
+
+    def read(blocks, n):
+        return [int(x) for x in pool[list(blocks)].reshape(-1)[:n]] if n else []
+
+    def check_all():
+        for s in slots:
+            assert e.slot_len(s) == len(truth[s])
+            assert read(e.slot_blocks(s), len(truth[s])) == truth[s], (seed, s)
+        _conservation(e, n_blocks, slots)
+
+    for step in range(120):
+        op = rng.choice(["pass", "pass", "pass", "fork", "reset"])
+        if op == "fork":
+            a, b = (int(x) for x in rng.choice(slots, 2, replace=False))
+            e.slot_reset(b)
+            e.slot_fork(a, b)
+            truth[b] = list(truth[a])
+        elif op == "reset":
+            a = int(rng.choice(slots))
+            e.slot_reset(a)
+            truth[a] = []
+        else:
+            # up to 3 trees, distinct destinations; a tree extends a parent in place, or into an empty slot, or starts fresh
+            dsts = [int(x) for x in rng.choice(slots, int(rng.integers(1, 4)), replace=False)]
+            specs, plan = [], []
+            for d in dsts:
+                n_new = int(rng.integers(1, 50))
+                kind = rng.choice(["inplace", "from", "fresh"])
+                if kind == "inplace" and truth[d]:
+                    parent = d
+                elif kind == "from":
+                    parent = int(rng.choice(slots))
+                    if not truth[parent] or parent == d or parent in dsts:   # a parent that another tree rewrites is left out
+                        parent = -1
+                else:
+                    parent = -1
+                if parent != d:
+                    e.slot_reset(d)
+                    truth[d] = []
+                specs.append(host.make_spec(parent=parent, save=d, root_len=n_new))
+                plan.append((parent, d, n_new))
+            before = (pool.copy(), {s: list(e.slot_blocks(s)) for s in slots}, e.free_blocks())
+            try:
+                ps = e.pass_begin(specs)
+            except abi.EspError:
+                assert ({s: list(e.slot_blocks(s)) for s in slots}, e.free_blocks()) == before[1:]   # refused: nothing moved
+                check_all()
+                continue
+            rows = {}
+            for t, (parent, d, n_new) in zip(ps["trees"], plan):
+                assert int(t["M"]) == n_new and int(t["P"]) == (len(truth[parent]) if parent >= 0 else 0)
+                toks = list(range(next_tok[0], next_tok[0] + n_new))
+                next_tok[0] += n_new
+                for r, tok in enumerate(toks):
+                    rows[int(t["base"]) + r] = tok
+                plan[plan.index((parent, d, n_new))] = (parent, d, toks)
+                if parent >= 0:   # what the attention of this tree reads through its table: the parent's tokens
+                    nb = (len(truth[parent]) + bt - 1) // bt
+                    tab = ps["table"][int(t["table"]):int(t["table"]) + nb]
+                    cowmap = {int(dst): int(src) for src, dst in ps["cow"].tolist()}
+                    assert [int(x) for x in pool[[cowmap.get(int(b), int(b)) for b in tab]].reshape(-1)[:len(truth[parent])]] == truth[parent]
+            for src, dst in ps["cow"].tolist():
+                pool[dst] = pool[src]
+            for sv in ps["saves"]:
+                pool[int(sv["block"]), int(sv["pos"])] = rows[int(sv["src_row"])]
+            if rng.integers(0, 4) == 0:
+                e.pass_abort()
+                pool[:] = before[0]
+                assert ({s: list(e.slot_blocks(s)) for s in slots}, e.free_blocks()) == before[1:]
+            else:
+                e.pass_commit()
+                new_truth = {d: (list(truth[parent]) if parent >= 0 else []) + toks for parent, d, toks in plan}
+                truth.update(new_truth)
+        check_all()
+
+
 # ---------------------------------------------------------------- rows of verify trees
 def test_leaf_hosting_and_descriptors_match_the_restatement():
     rng = np.random.default_rng(5)
