@@ -16,18 +16,29 @@ P0 = [70, 33, 500, 1030, 16, 0]
 # (query heads, KV heads, head dim, tokens per block, prep arrangement): the benchmark's Qwen shape, a sliding-layer
 # Gemma shape at the reference's block size, and Gemma 4's 512-dim heads (wavefront pairs, open-ended ranges)
 SHAPES = [(8, 2, 128, 16, "omni"), (4, 2, 256, 64, "gemma"), (8, 1, 512, 16, "gemma")]
+# (shape, window): 0 = a layer that keeps every key in listed blocks; > 0 = a sliding layer whose slot holds a ring of
+# ceil(window / block) consecutive blocks, key j in block (j / block) % ring (80_gemma.metal:139), which the chain's
+# appends overwrite as they go
+CASES = [(s, 0) for s in SHAPES] + [((8, 2, 128, 16, "omni"), 100), ((4, 2, 256, 64, "gemma"), 128), ((16, 8, 256, 16, "gemma"), 48)]
 
 
-def _setup(shape, seed=12):
+def _slot_block(ap, blocks, table, j):
+    """Physical block of key j of the slot whose record says `table` (arrays or scalars)."""
+    bi = j // ap.bt
+    return table + bi % ap.ring if ap.ring else blocks[table + bi]
+
+
+def _setup(shape, window, seed=12):
     H, HKV, HD, BT, kind = shape
     rng = np.random.default_rng(seed)
     n = len(P0)
-    ap = synth.make_params(H, HKV, HD, abi.ESP_F16, BT, rows_per_tile=1)
+    ring = (window + BT - 1) // BT if window else 0
+    ap = synth.make_params(H, HKV, HD, abi.ESP_F16, BT, window=window, ring=ring, rows_per_tile=1)
     pp, a = synth.make_prep(kind, H, HKV, HD, abi.ESP_F16, n, seed=seed, bt=BT)
-    nb = [(p + K + BT) // BT for p in P0]                      # room for the K tokens the chain appends
+    nb = [ring if ring else (p + K + BT) // BT for p in P0]    # room for the K tokens the chain appends
     n_blocks = sum(nb) + 3
     perm = rng.permutation(n_blocks).astype(np.int32)
-    blocks = perm[:sum(nb)].copy()
+    blocks = perm[:sum(nb)].copy()                             # a ring's blocks are not listed: its record names the first
     trees = np.zeros(n, abi.TREE_DT)
     kvw = HKV * HD
     pool = np.zeros(n_blocks * 2 * BT * kvw, np.uint16)       # reference layout
@@ -35,8 +46,8 @@ def _setup(shape, seed=12):
     off = 0
     for i, p in enumerate(P0):
         trees[i] = (i, p, off, 1)
-        for j in range(p):
-            b = blocks[off + j // BT]
+        for j in range(max(0, p - ring * BT) if ring else 0, p):   # a ring holds the last ring * block keys
+            b = _slot_block(ap, blocks, off, j)
             pv[b, 0, j % BT] = ob.from_f32(rng.standard_normal(kvw).astype(np.float32) * 0.5, ap.dtype)
             pv[b, 1, j % BT] = ob.from_f32(rng.standard_normal(kvw).astype(np.float32) * 0.5, ap.dtype)
         off += nb[i]
@@ -58,32 +69,32 @@ def _host_chain(ap, trees, blocks, pool, Q, Kb, Vb):
         desc = np.zeros((n, 4), np.int32)
         out.append(ob.attn_direct(ap, Q[s], Kb[s], Vb[s], pool, blocks, desc, pos, trees, n_threads=4))
         e = np.zeros(n, abi.KVSAVE_DT)
-        e["src_row"], e["block"], e["pos"] = np.arange(n), blocks[trees["table"] + trees["P"] // BT], trees["P"] % BT
+        e["src_row"], e["block"], e["pos"] = np.arange(n), _slot_block(ap, blocks, trees["table"], trees["P"]), trees["P"] % BT
         ob.kv_save(ap, Kb[s], Vb[s], pool, e)
         trees["P"] += 1
     return np.stack(out), pool
 
 
-@pytest.mark.parametrize("shape", SHAPES)
-def test_device_chain_matches_the_checker_step_by_step_and_replays_identically(shape):
+@pytest.mark.parametrize("shape,window", CASES)
+def test_device_chain_matches_the_checker_step_by_step_and_replays_identically(shape, window):
     device.init(0)
-    ap, pp, a, trees, blocks, pool_ref, n_blocks, X = _setup(shape)
+    ap, pp, a, trees, blocks, pool_ref, n_blocks, X = _setup(shape, window)
     n = len(trees)
     BT = ap.bt
-    print(f"chain shape {shape}", flush=True)
+    print(f"chain shape {shape} window {window} ring {ap.ring}", flush=True)
 
     dev = lambda x: None if x is None else torch.from_numpy(np.ascontiguousarray(x)).cuda()  # noqa: E731
     ref = dev(pool_ref.view(np.int16))
     pool0 = torch.empty_like(ref)
     device.kv_relayout(ap, ref, abi.ESP_LAYOUT_REFERENCE, pool0, abi.ESP_LAYOUT_NATIVE, n_blocks)
     resident, groups = device.plan_hint(ap)
-    tiles, jobs, n_parts = host.plan_tiles(trees, groups, 0, None, host.options_mi355x(1, resident))
-    tiles = host.open_ended(tiles, trees)
-    assert (tiles["k1"] == 2**31 - 1).sum() == n               # one open range per sequence
     pos0 = np.zeros((n, 4), np.int32)
     pos0[:, :3] = trees["P"][:, None]
+    tiles, jobs, n_parts = host.plan_tiles(trees, groups, window, pos0 if window else None, host.options_mi355x(1, resident))
+    tiles = host.open_ended(tiles, trees)
+    assert (tiles["k1"] == 2**31 - 1).sum() == n               # one open range per sequence
     table0 = np.full((n, 4), -1, np.int32)
-    table0[:, 0] = blocks[trees["table"] + trees["P"] // BT]
+    table0[:, 0] = _slot_block(ap, blocks, trees["table"], trees["P"])
     table0[:, 1] = trees["P"] % BT
     # device-resident state of the chain, and its initial values to go back to before every run
     init = dict(trees=device.to_dev(trees), pos=dev(pos0), table=dev(table0), pool=pool0)
@@ -91,6 +102,8 @@ def test_device_chain_matches_the_checker_step_by_step_and_replays_identically(s
     blocks_d = dev(blocks)
     dp = device.DevicePass(ap, trees, tiles, jobs, n_parts, n, blocks, None, None)
     dp.trees = st["trees"]                                      # the pass reads the records the chain advances
+    if window:
+        dp.pos = st["pos"]                                      # and, for the window rule, the positions it advances
     Xd, qn, kn = dev(X), dev(a["qn_w"]), dev(a["kn_w"])
     inv_freq, sel = dev(a["inv_freq"]), dev(a["rope_sel"])
     Q = torch.zeros(K, n, ap.q_ld, dtype=torch.float16, device="cuda")      # every step's prepared rows are kept
@@ -102,7 +115,7 @@ def test_device_chain_matches_the_checker_step_by_step_and_replays_identically(s
         for s in range(K):
             device.attn_prep(pp, Xd[s], qn, kn, st["pos"], inv_freq, sel, Q[s], Kb[s], Vb[s], st["table"], st["pool"], n)
             dp.run(Q[s], Kb[s], Vb[s], st["pool"], O[s])
-            device.chain_advance(st["trees"], n, st["pos"], st["table"], blocks_d, BT)
+            device.chain_advance(st["trees"], n, st["pos"], st["table"], blocks_d, BT, ap.ring)
 
     def reset():
         for k in st:
@@ -139,9 +152,13 @@ def test_device_chain_matches_the_checker_step_by_step_and_replays_identically(s
         for g_, w_ in ((bits(Q[s_]), qw), (bits(Kb[s_]), kw), (bits(Vb[s_]), vw)):
             assert np.abs(ob.to_f32(g_, ap.dtype).astype(np.float64) - ob.to_f32(w_, ap.dtype)).max() <= 2.0 ** -8
     # every appended token is in the pool where host bookkeeping puts it: bit for bit
+    back = torch.empty_like(ref)
+    device.kv_relayout(ap, st["pool"], abi.ESP_LAYOUT_NATIVE, back, abi.ESP_LAYOUT_REFERENCE, n_blocks)
+    torch.cuda.synchronize()
+    assert np.array_equal(bits(back), ref_out["pool"])
     Kg = torch.zeros((max(P0) + K) * ap.kv_ld, dtype=torch.float16, device="cuda")
     Vg = torch.zeros_like(Kg)
-    for i, p in enumerate(P0):
+    for i, p in enumerate(P0 if not ap.ring else []):           # listed blocks also read back in token order
         device.kv_gather(ap, st["pool"], blocks_d[int(trees[i]["table"]):], p + K, Kg, Vg)
         torch.cuda.synchronize()
         kw, vw = ob.kv_gather(ap, ref_out["pool"], blocks[int(trees[i]["table"]):], p + K)
