@@ -81,7 +81,10 @@ int esp_engine_pass_blocks(const esp_engine* e, const esp_tree_spec* specs, int3
 
 /* Build a pass: validates every tree before touching anything, then plans
  * rows, descriptors, positions, the block table, kv_save entries and
- * copy-on-write pairs. The pass stays pending until committed or aborted. */
+ * copy-on-write pairs. The block table already names the copies: the caller
+ * runs esp_kv_copy_blocks over the pairs before the pass's first attention
+ * (the reference's order, forest.h:2726-2729), the saves after it. The pass
+ * stays pending until committed or aborted. */
 int esp_engine_pass_begin(esp_engine* e, const esp_tree_spec* specs, int32_t n, char* err, size_t errlen);
 int esp_engine_pass_rows(const esp_engine* e);      /* M */
 int esp_engine_pass_counts(const esp_engine* e, int32_t* n_table, int32_t* n_saves, int32_t* n_cow);

@@ -1,8 +1,12 @@
-"""The host engine's own records driving the kernels: a small serving history (prefill of two sequences,
-decode steps, a fork, a verify tree with hosted draft prefixes beside a decode, a further chunk) where every
-pass takes its trees / descriptors / positions / block table / copy-on-write pairs / save entries from
-`KvEngine` and runs on the GPU through the C ABI. The CPU checker follows in a reference-layout pool fed by
-the same records. Bar: attention outputs within the path's tolerance; the pool bit-identical at the end."""
+"""The host engine's own records driving the kernels through serving histories - prefill chunks, decode
+steps, forks, verify trees with hosted draft prefixes, passes that are not committed - where every pass
+takes its trees / descriptors / positions / block table / copy-on-write pairs / save entries from
+`KvEngine` and runs on the GPU through the C ABI, in the reference's order: block copies first
+(src/model/impl/forest.h:2726-2729), attention, then the saves (forest.h:2935-2947). The CPU checker follows
+in a reference-layout pool fed by the same records, and a model that knows no blocks - the list of K / V
+rows every slot logically holds - is checked against both: what a tree's table exposes at attention time is
+its parent's rows, and what a slot's block list reads back after the pass is the slot's rows.
+Bar: attention outputs within the path's tolerance; rows and the pool bit-identical."""
 import numpy as np
 import pytest
 import torch
@@ -15,69 +19,187 @@ from helpers import f32
 pytestmark = pytest.mark.gpu
 
 
-@pytest.mark.parametrize("H,Hkv,HD,bt,dtype", [(8, 2, 128, 16, abi.ESP_F16), (8, 1, 512, 32, abi.ESP_F16), (6, 3, 256, 64, abi.ESP_BF16)])
-def test_engine_records_drive_the_kernels_through_a_serving_history(H, Hkv, HD, bt, dtype):
-    from gpu_utils import dev_u16, to_host_u16
-    device.init(0)
-    rng = np.random.default_rng(H + HD)
-    n_blocks = 96
-    ap = synth.make_params(H, Hkv, HD, dtype, bt)
-    region = n_blocks * 2 * bt * ap.kv_ld
-    pool_ref = np.zeros(region, np.uint16)
-    pool = torch.zeros(region, dtype=torch.int16, device="cuda")
-    e = host.Engine(n_blocks, bt, 4)
-    A, B, Cc, D = (e.slot_alloc() for _ in range(4))
-    tol = 2e-3 if dtype == abi.ESP_F16 else 4e-3
-    tiled_rows = device.plan_hint3(ap)[2]
+class Served:
+    def __init__(self, H, Hkv, HD, bt, dtype, n_blocks, n_slots, seed):
+        device.init(0)
+        self.rng = np.random.default_rng(seed)
+        self.dtype, self.n_blocks = dtype, n_blocks
+        self.ap = synth.make_params(H, Hkv, HD, dtype, bt)
+        self.region = n_blocks * 2 * bt * self.ap.kv_ld
+        self.pool_ref = np.zeros(self.region, np.uint16)
+        self.pool = torch.zeros(self.region, dtype=torch.int16, device="cuda")
+        self.e = host.Engine(n_blocks, bt, n_slots)
+        self.slots = [self.e.slot_alloc() for _ in range(n_slots)]
+        empty = np.zeros((0, self.ap.kv_ld), np.uint16)
+        self.truth = {s: (empty, empty) for s in self.slots}     # slot -> (K rows, V rows) it logically holds
+        self.tol = 2e-3 if dtype == abi.ESP_F16 else 4e-3
+        self.max_rows = device.plan_hint3(self.ap)[2]
 
-    def run(specs, rows_per_tile, commit=True, tag=""):
-        ps = e.pass_begin(specs)
+    def reset(self, s):
+        self.e.slot_reset(s)
+        self.truth[s] = (self.truth[s][0][:0], self.truth[s][1][:0])
+
+    def fork(self, a, b):
+        self.reset(b)
+        self.e.slot_fork(a, b)
+        self.truth[b] = self.truth[a]
+
+    def run(self, specs, rows_per_tile, commit=True, tag=""):
+        """specs: [(parent, save, root_len, leaves, commit_chain)]. False if the engine refused the pass."""
+        from gpu_utils import dev_u16, to_host_u16
+        ap, e, dtype = self.ap, self.e, self.dtype
+        try:
+            ps = e.pass_begin([host.make_spec(parent=p, save=s, root_len=r, leaves=lv, commit_chain=cc) for p, s, r, lv, cc in specs])
+        except abi.EspError as ex:
+            print(f"{tag}: refused ({ex})", flush=True)
+            return False
         M = ps["M"]
-        print(f"{tag}: M={M} trees={[tuple(int(x) for x in t) for t in ps['trees']]} cow={ps['cow'].tolist()} saves={len(ps['saves'])}", flush=True)
-        bits = lambda w: ob.from_f32(rng.standard_normal((M, w)).astype(np.float32) * 0.5, dtype)  # noqa: E731
+        print(f"{tag}: M={M} rows/tile={rows_per_tile} trees={[tuple(int(x) for x in t) for t in ps['trees']]} "
+              f"cow={ps['cow'].tolist()} saves={len(ps['saves'])}", flush=True)
+        bits = lambda w: ob.from_f32(self.rng.standard_normal((M, w)).astype(np.float32) * 0.5, dtype)  # noqa: E731
         Q, Kb, Vb = bits(ap.q_ld), bits(ap.kv_ld), bits(ap.kv_ld)
         blocks = ps["table"] if len(ps["table"]) else np.zeros(1, np.int32)
+        if len(ps["cow"]):
+            device.kv_copy_blocks(ap, self.pool, device.to_dev(np.ascontiguousarray(ps["cow"], np.int32)), len(ps["cow"]), 1, self.region)
+            ob.kv_copy_blocks(ap, self.pool_ref, ps["cow"], 1, self.region)
+        for t, (parent, *_) in zip(ps["trees"], specs):           # the table of every tree exposes its parent's rows
+            P = int(t["P"])
+            assert P == (len(self.truth[parent][0]) if parent >= 0 else 0)
+            if P:
+                kw, vw = ob.kv_gather(ap, self.pool_ref, blocks[int(t["table"]):], P)
+                assert np.array_equal(kw, self.truth[parent][0]) and np.array_equal(vw, self.truth[parent][1]), tag
         ap.rows_per_tile = rows_per_tile
         resident, groups = device.plan_hint(ap)
         tiles, jobs, n_parts = host.plan_tiles(ps["trees"], groups, 0, None, host.options_mi355x(rows_per_tile, resident))
         dp = device.DevicePass(ap, ps["trees"], tiles, jobs, n_parts, M, blocks, ps["desc"], ps["pos"])
         Qd, Kd, Vd = dev_u16(Q), dev_u16(Kb), dev_u16(Vb)
         O = torch.zeros_like(Qd)
-        dp.run(Qd, Kd, Vd, pool, O)
+        dp.run(Qd, Kd, Vd, self.pool, O)
         torch.cuda.synchronize()
-        want = ob.attn_direct(ap, Q, Kb, Vb, pool_ref, blocks, ps["desc"], ps["pos"], ps["trees"], n_threads=8)
+        want = ob.attn_direct(ap, Q, Kb, Vb, self.pool_ref, blocks, ps["desc"], ps["pos"], ps["trees"], n_threads=8)
         err = float(np.abs(f32(to_host_u16(O).reshape(M, -1), dtype) - f32(want, dtype)).max())
-        assert err <= tol, (tag, err)
+        assert err <= self.tol, (tag, err)
         if not commit:
-            e.pass_abort()
-            return
-        if len(ps["cow"]):
-            device.kv_copy_blocks(ap, pool, device.to_dev(np.ascontiguousarray(ps["cow"], np.int32)), len(ps["cow"]), 1, region)
-            ob.kv_copy_blocks(ap, pool_ref, ps["cow"], 1, region)
+            e.pass_abort()     # the copied blocks go back to the free list; nothing a slot lists has changed
+            self.check_slots(tag)
+            return True
         if len(ps["saves"]):
-            device.kv_save(ap, Kd, Vd, pool, device.to_dev(ps["saves"]), len(ps["saves"]))
-            ob.kv_save(ap, Kb, Vb, pool_ref, ps["saves"])
+            device.kv_save(ap, Kd, Vd, self.pool, device.to_dev(ps["saves"]), len(ps["saves"]))
+            ob.kv_save(ap, Kb, Vb, self.pool_ref, ps["saves"])
         torch.cuda.synchronize()
         e.pass_commit()
+        new = {}
+        for t, (parent, save, root_len, *_) in zip(ps["trees"], specs):
+            if save >= 0:                                          # the slot takes its parent's rows and the tree's root
+                pk, pv = self.truth[parent] if parent >= 0 else (Kb[:0], Vb[:0])
+                b = int(t["base"])
+                new[save] = (np.concatenate([pk, Kb[b:b + root_len]]), np.concatenate([pv, Vb[b:b + root_len]]))
+        self.truth.update(new)
+        self.check_slots(tag)
+        return True
 
-    run([host.make_spec(save=A, root_len=100), host.make_spec(save=B, root_len=57)], tiled_rows, tag="prefill A, B")
+    def check_slots(self, tag):
+        for s in self.slots:
+            n = len(self.truth[s][0])
+            assert self.e.slot_len(s) == n, (tag, s)
+            if n:
+                kw, vw = ob.kv_gather(self.ap, self.pool_ref, self.e.slot_blocks(s), n)
+                assert np.array_equal(kw, self.truth[s][0]) and np.array_equal(vw, self.truth[s][1]), (tag, s)
+
+    def finish(self):
+        """The device pool holds what the reference-layout pool holds, block for block, and every slot reads back
+        through the device's gather as its rows."""
+        from gpu_utils import to_host_u16
+        back = torch.zeros_like(self.pool)
+        device.kv_relayout(self.ap, self.pool, abi.ESP_LAYOUT_NATIVE, back, abi.ESP_LAYOUT_REFERENCE, self.n_blocks)
+        torch.cuda.synchronize()
+        assert np.array_equal(to_host_u16(back), self.pool_ref)
+        for s in self.slots:
+            n = len(self.truth[s][0])
+            if not n:
+                continue
+            Kg = torch.zeros(n * self.ap.kv_ld, dtype=torch.int16, device="cuda")
+            Vg = torch.zeros_like(Kg)
+            device.kv_gather(self.ap, self.pool, device.to_dev(np.ascontiguousarray(self.e.slot_blocks(s), np.int32)), n, Kg, Vg)
+            torch.cuda.synchronize()
+            assert np.array_equal(to_host_u16(Kg).reshape(n, -1), self.truth[s][0])
+            assert np.array_equal(to_host_u16(Vg).reshape(n, -1), self.truth[s][1])
+
+
+@pytest.mark.parametrize("H,Hkv,HD,bt,dtype", [(8, 2, 128, 16, abi.ESP_F16), (8, 1, 512, 32, abi.ESP_F16), (6, 3, 256, 64, abi.ESP_BF16)])
+def test_engine_records_drive_the_kernels_through_a_serving_history(H, Hkv, HD, bt, dtype):
+    sv = Served(H, Hkv, HD, bt, dtype, 96, 4, H + HD)
+    A, B, Cc, D = sv.slots
+    e = sv.e
+    G = H // Hkv
+    sv.run([(-1, A, 100, (), 0), (-1, B, 57, (), 0)], sv.max_rows, tag="prefill A, B")
     for s in range(3):
-        run([host.make_spec(parent=A, save=A, root_len=1), host.make_spec(parent=B, save=B, root_len=1)], 1, tag=f"decode {s}")
-    e.slot_fork(A, Cc)
+        sv.run([(A, A, 1, (), 0), (B, B, 1, (), 0)], 1, tag=f"decode {s}")
+    sv.fork(A, Cc)
     drafts = [5, 6, 7]
     leaves = [drafts[:i + 1] for i in range(3)]
-    G = H // Hkv
     rows_verify = 4 if HD < 512 else max(1, 16 // G)       # what the streaming kernel packs at this head dim
-    run([host.make_spec(parent=Cc, save=Cc, root_len=1, leaves=leaves, commit_chain=3), host.make_spec(parent=A, save=A, root_len=1)],
-        rows_verify, tag="verify C (fork of A: copy on write) + decode A")
-    run([host.make_spec(parent=B, root_len=2, leaves=[[1, 2], [1, 3, 4], [9]])], 8 if HD < 512 else max(1, 16 // G), commit=False,
-        tag="wide verify tree on B, not committed")
-    run([host.make_spec(parent=B, save=B, root_len=45), host.make_spec(parent=A, save=D, root_len=20)], tiled_rows,
-        tag="chunk on B + A continued into D")
-    run([host.make_spec(parent=s_, save=s_, root_len=1) for s_ in (A, B, Cc, D)], 1, tag="decode all four")
+    sv.run([(Cc, Cc, 1, leaves, 3), (A, A, 1, (), 0)], rows_verify, tag="verify C (fork of A: copy on write) + decode A")
+    sv.run([(B, -1, 2, [[1, 2], [1, 3, 4], [9]], 0)], 8 if HD < 512 else max(1, 16 // G), commit=False,
+           tag="wide verify tree on B, not committed")
+    sv.run([(B, B, 45, (), 0), (A, D, 20, (), 0)], sv.max_rows, tag="chunk on B + A continued into D")
+    sv.run([(s_, s_, 1, (), 0) for s_ in (A, B, Cc, D)], 1, tag="decode all four")
     assert (e.slot_len(A), e.slot_len(B), e.slot_len(Cc), e.slot_len(D)) == (105, 106, 105, 125)   # the verify pass commits its root token only
-    # the device pool holds what the reference-layout pool holds, block for block
-    back = torch.zeros_like(pool)
-    device.kv_relayout(ap, pool, abi.ESP_LAYOUT_NATIVE, back, abi.ESP_LAYOUT_REFERENCE, n_blocks)
-    torch.cuda.synchronize()
-    assert np.array_equal(to_host_u16(back), pool_ref)
+    sv.finish()
+
+
+def _random_leaves(rng):
+    """A few draft token lists over a small alphabet, so that prefixes are shared and hosted once."""
+    return [[int(x) for x in rng.integers(1, 4, int(rng.integers(1, 5)))] for _ in range(int(rng.integers(1, 5)))]
+
+
+@pytest.mark.parametrize("seed", range(6))
+def test_random_serving_histories(seed):
+    """Random passes of up to three trees (chunks, decode rows, verify trees; in place, into another slot, from
+    nothing), forks and resets in between, one pass in four not committed, a pool small enough that some
+    passes are refused; geometry, block size and tile height drawn per history."""
+    rng = np.random.default_rng(4000 + seed)
+    H, Hkv, HD = [(8, 2, 128), (4, 4, 128), (16, 2, 256), (6, 3, 256), (8, 1, 512), (4, 2, 512)][seed % 6]
+    bt = int(rng.choice([16, 32, 64]))
+    dtype = abi.ESP_F16 if seed % 2 == 0 else abi.ESP_BF16
+    n_slots = 4
+    sv = Served(H, Hkv, HD, bt, dtype, int(rng.integers(24, 64)) * 64 // bt, n_slots, 5000 + seed)
+    heights = [r for r in (1, 2, 4, 8, 16, sv.max_rows) if r <= sv.max_rows]
+    n_passes = 0
+    for step in range(30):
+        op = rng.choice(["pass", "fork", "reset"], p=[0.8, 0.15, 0.05])
+        if op == "fork":
+            a, b = (int(x) for x in rng.choice(sv.slots, 2, replace=False))
+            sv.fork(a, b)
+            continue
+        if op == "reset":
+            sv.reset(int(rng.choice(sv.slots)))
+            continue
+        dsts = [int(x) for x in rng.choice(sv.slots, int(rng.integers(1, 4)), replace=False)]
+        specs = []
+        for d in dsts:
+            kind = rng.choice(["inplace", "from", "fresh"], p=[0.75, 0.2, 0.05])
+            parent = d if len(sv.truth[d][0]) and kind != "fresh" else -1
+            if kind == "from":
+                other = int(rng.choice(sv.slots))
+                if len(sv.truth[other][0]) and other != d and other not in dsts:   # a parent that another tree rewrites is left out
+                    parent = other
+            if parent != d:
+                sv.reset(d)
+            shape = rng.choice(["chunk", "decode", "verify"]) if parent >= 0 else "chunk"
+            if shape == "chunk":
+                specs.append((parent, d, int(rng.integers(2, 90)), (), 0))
+            elif shape == "decode":
+                specs.append((parent, d, 1, (), 0))
+            else:
+                leaves = _random_leaves(rng)
+                chain = int(rng.integers(0, 2))
+                if chain:                                          # leaves [0, k) one chain: prefixes of one draft
+                    draft = [int(x) for x in rng.integers(1, 4, int(rng.integers(1, 4)))]
+                    leaves = [draft[:i + 1] for i in range(len(draft))] + [l for l in leaves if l[0] != draft[0]]
+                    chain = len(draft)
+                specs.append((parent, d, int(rng.integers(1, 3)), leaves, chain))
+        rows = 1 if all(s[2] == 1 and not s[3] for s in specs) else int(rng.choice(heights))
+        n_passes += sv.run(specs, rows, commit=rng.integers(0, 4) != 0, tag=f"seed {seed} step {step}")
+    assert n_passes >= 10
+    sv.finish()
