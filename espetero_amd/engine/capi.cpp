@@ -168,6 +168,24 @@ int esp_engine_pass_cow(const esp_engine* e, int32_t* out) {
   if (!p.cow.empty()) memcpy(out, p.cow.data(), p.cow.size() * 8);
   return int(p.cow.size());
 }
+int esp_engine_pass_rings(const esp_engine* e, int32_t window, int32_t ring_blocks, esp_tree* trees, esp_kvsave* saves,
+                          int32_t saves_cap, int32_t* n_saves, int32_t* copies, int32_t copies_cap, int32_t* n_copies, char* err,
+                          size_t errlen) {
+  try {
+    const auto r = e->e.ring_plan(window, ring_blocks);
+    if (n_saves) *n_saves = int32_t(r.saves.size());
+    if (n_copies) *n_copies = int32_t(r.copies.size());
+    if (int(r.saves.size()) > saves_cap || int(r.copies.size()) > copies_cap || (!r.saves.empty() && !saves) ||
+        (!r.copies.empty() && !copies) || !trees)
+      return put_err(err, errlen, ESP_EWORKSPACE, "pass_rings: output arrays too small (counts written)");
+    memcpy(trees, r.trees.data(), r.trees.size() * sizeof(esp_tree));
+    if (!r.saves.empty()) memcpy(saves, r.saves.data(), r.saves.size() * sizeof(esp_kvsave));
+    if (!r.copies.empty()) memcpy(copies, r.copies.data(), r.copies.size() * 8);
+    return ESP_OK;
+  } catch (const std::exception& ex) {
+    return put_err(err, errlen, ESP_EINVAL, ex.what());
+  }
+}
 int esp_kv_row_table(const esp_kvsave* saves, int32_t n_saves, int32_t rows, int32_t* out, char* err, size_t errlen) {
   try {
     const std::vector<int32_t> t = espetero::engine::row_table(saves, n_saves, rows);

@@ -10,6 +10,7 @@
 //   leaf hosting            src/model/impl/forest.h:2201-2220, commit chains :2223-2234
 //   rows: desc / pos        src/model/impl/forest.h:2374-2443
 //   block table, kv saves   src/model/impl/forest.h:2483-2520
+//   sliding-layer rings     src/model/impl/forest.h:2657-2700 (trees, saves, window copies)
 //   commit / rollback       src/model/impl/forest.h:2468-2482, 4743-4754
 //   slot operations         src/model/model.mm:520-553
 // A pass never changes a slot before commit(): a failure (or abort()) gives
@@ -363,6 +364,42 @@ class KvEngine {
     guard.armed = false;
     ps.pending = true;
     pass_ = std::move(ps);
+  }
+
+  // The pending pass as the sliding layers see it (Gemma: the last `window` positions of slot s live in a second
+  // pool, in the ring of `ring_blocks` consecutive blocks from s * ring_blocks on, position p in block
+  // (p / bt) % ring_blocks; src/model/impl/forest.h:2657-2700):
+  //   trees   read the parent's ring: table = the ring's first block;
+  //   saves   of the rows that are still inside the window when the pass ends, into the ring of every target;
+  //   copies  (ring block of the parent -> same ring block of the target) for a target that is another slot:
+  //           the part of the parent's window the target still needs, each ring block once.
+  // Copies run before the pass's attention and saves after it, like the other pool's.
+  struct RingPlan {
+    std::vector<esp_tree> trees;
+    std::vector<esp_kvsave> saves;
+    std::vector<std::array<int32_t, 2>> copies;
+  };
+  RingPlan ring_plan(int window, int ring_blocks) const {
+    if (!pass_.pending) fail("no pending pass");
+    const int bt = pool_.bt, rb = ring_blocks, W = window;
+    if (W <= 0 || rb <= 0 || int64_t(rb) * bt < W) fail("ring_plan: the ring must hold the window");
+    RingPlan out;
+    for (const TreePlan& T : pass_.trees) {
+      const int parent = T.spec.parent;
+      out.trees.push_back({T.base, T.P, parent >= 0 ? parent * rb : 0, T.M});
+      auto target = [&](int slot, int S) {
+        if (slot != parent && T.P > 0) {
+          std::vector<char> seen(size_t(rb), 0);
+          for (int b = std::max(0, T.P + S - W + 1) / bt; b * bt < T.P; ++b)
+            if (!seen[size_t(b % rb)]++) out.copies.push_back({parent * rb + b % rb, slot * rb + b % rb});
+        }
+        for (int p = std::max(T.P, T.P + S - W + 1); p < T.P + S; ++p)
+          out.saves.push_back({T.base + (p - T.P), slot * rb + (p / bt) % rb, p % bt, 0});
+      };
+      if (T.spec.save >= 0) target(T.spec.save, T.save_len);
+      if (T.spec.work >= 0) target(T.spec.work, T.Tr);
+    }
+    return out;
   }
 
   void pass_commit() {

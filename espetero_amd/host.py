@@ -49,6 +49,7 @@ ENGINE_SYMBOLS = {
     "esp_engine_pass_table": (C.c_int, (_V, _V)),
     "esp_engine_pass_saves": (C.c_int, (_V, _V)),
     "esp_engine_pass_cow": (C.c_int, (_V, _V)),
+    "esp_engine_pass_rings": (C.c_int, (_V, _I, _I, _V, _V, _I, _IP, _V, _I, _IP) + _ERR),
     "esp_slot_file_save": (C.c_int, (C.c_char_p, C.c_int32, C.c_int32, C.c_int32, C.c_int32, C.c_uint64, _V)),
     "esp_slot_file_info": (C.c_int, (C.c_char_p, C.c_int32, _V, _V, _V, _V, _V)),
     "esp_slot_file_load": (C.c_int, (C.c_char_p, C.c_int32, _V, C.c_uint64)),
@@ -235,6 +236,23 @@ class Engine:
         self.lib.esp_engine_pass_cow(self.h, cow.ctypes.data)
         return dict(trees=trees, desc=desc[:M], pos=pos[:M], table=table[:nt.value], saves=saves[:ns.value],
                     cow=cow[:nc.value], M=M)
+
+    def pass_rings(self, window, ring_blocks):
+        """The pending pass on sliding layers: dict(trees, saves, copies)."""
+        n = self.lib.esp_engine_pass_counts(self.h, None, None, None)
+        trees = np.zeros(max(n, 1), abi.TREE_DT)
+        ns, nc = C.c_int32(0), C.c_int32(0)
+        err = C.create_string_buffer(256)
+        rc = self.lib.esp_engine_pass_rings(self.h, window, ring_blocks, trees.ctypes.data, None, 0, C.byref(ns), None, 0,
+                                            C.byref(nc), err, 256)
+        if rc not in (0, 4):
+            abi.check(rc, err)
+        saves = np.zeros(max(ns.value, 1), abi.KVSAVE_DT)
+        copies = np.zeros((max(nc.value, 1), 2), np.int32)
+        rc = self.lib.esp_engine_pass_rings(self.h, window, ring_blocks, trees.ctypes.data, saves.ctypes.data, ns.value,
+                                            C.byref(ns), copies.ctypes.data, nc.value, C.byref(nc), err, 256)
+        abi.check(rc, err)
+        return dict(trees=trees[:n], saves=saves[:ns.value], copies=copies[:nc.value])
 
     def pass_commit(self):
         return self.lib.esp_engine_pass_commit(self.h)

@@ -11,6 +11,7 @@
  *   leaf hosting, row descriptors  src/model/impl/forest.h:2201-2220, 2374-2443
  *   block tables, kv_save entries  src/model/impl/forest.h:2483-2520
  *   slot commit / PassGuard        src/model/impl/forest.h:2468-2482, 4743-4754
+ *   sliding-layer ring planning    src/model/impl/forest.h:2657-2700
  *   slot_alloc/free/reset/fork/len src/model/model.mm:520-553
  * The C++ headers are the interface a C++ engine includes; these functions
  * exist so that other languages (and the tests) can drive the same code.
@@ -94,6 +95,20 @@ int esp_engine_pass_pos(const esp_engine* e, int32_t* out);             /* 4 * M
 int esp_engine_pass_table(const esp_engine* e, int32_t* out);
 int esp_engine_pass_saves(const esp_engine* e, esp_kvsave* out);
 int esp_engine_pass_cow(const esp_engine* e, int32_t* out);             /* 2 * n_cow */
+/* The pending pass on sliding layers (replaces the ring planning of src/model/impl/forest.h:2657-2700):
+ * slot s keeps its last `window` positions in a second pool, in the ring_blocks consecutive blocks from
+ * s * ring_blocks on, position p in block (p / bt) % ring_blocks. Writes the trees as those layers read
+ * them (table = first block of the parent's ring; n trees of the pass), the save entries of the rows that
+ * are still inside the window when the pass ends, and (source, destination) block copies that carry the
+ * parent's window into the ring of a target that is another slot (copies before the attention, saves
+ * after it). A pass whose ring saves have run is committed: an in-place chunk's saves reuse ring cells the
+ * slot would still need if it did not advance. esp_engine_slot_fork has a ring side too, the caller's: copy
+ * the source's whole ring, blocks src * ring_blocks + i -> dst * ring_blocks + i (copy_slot_state,
+ * src/model/impl/forest.h:127-137), with esp_kv_copy_blocks on the ring pool.
+ * ESP_EWORKSPACE when saves_cap / copies_cap are too small: the needed counts are still written. */
+int esp_engine_pass_rings(const esp_engine* e, int32_t window, int32_t ring_blocks, esp_tree* trees, esp_kvsave* saves,
+                          int32_t saves_cap, int32_t* n_saves, int32_t* copies, int32_t copies_cap, int32_t* n_copies,
+                          char* err, size_t errlen);
 /* Slot checkpoint files in the reference's format (src/model/model.mm:600-752), KV section: the
  * 120-byte CkptHeader (magic 0x554b5043, version 4), then n_layers x n_blocks blocks of block_bytes,
  * layer-major, logical block order, each in the reference's block layout (what

@@ -197,3 +197,25 @@ def kv_row_table(saves, rows):
         e[j], e[j + 1] = block, pos
     return t[:rows]
 
+
+
+def ring_plan(trees, window, ring_blocks, bt):
+    """The sliding layers' view of a pass: src/model/impl/forest.h:2657-2659 (trees) and 2679-2700 (saves,
+    copies). Slot s owns ring blocks [s * ring_blocks, (s + 1) * ring_blocks); position p lives in block
+    (p / bt) % ring_blocks. trees: (base, P, M, parent slot or -1, [(target slot, rows saved), ...]).
+    Returns (tree records (base, P, table, M), saves (src_row, block, pos, 0), copies (src, dst))."""
+    recs, saves, copies = [], [], []
+    for base, P, M, parent, targets in trees:
+        recs.append((base, P, parent * ring_blocks if parent >= 0 else 0, M))
+        for slot, S in targets:
+            if slot != parent and P > 0:
+                seen = set()
+                b = max(0, P + S - window + 1) // bt
+                while b * bt < P:
+                    if b % ring_blocks not in seen:
+                        seen.add(b % ring_blocks)
+                        copies.append((parent * ring_blocks + b % ring_blocks, slot * ring_blocks + b % ring_blocks))
+                    b += 1
+            for p in range(max(P, P + S - window + 1), P + S):
+                saves.append((base + (p - P), slot * ring_blocks + (p // bt) % ring_blocks, p % bt, 0))
+    return recs, saves, copies

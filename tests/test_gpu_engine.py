@@ -20,7 +20,7 @@ pytestmark = pytest.mark.gpu
 
 
 class Served:
-    def __init__(self, H, Hkv, HD, bt, dtype, n_blocks, n_slots, seed):
+    def __init__(self, H, Hkv, HD, bt, dtype, n_blocks, n_slots, seed, window=0):
         device.init(0)
         self.rng = np.random.default_rng(seed)
         self.dtype, self.n_blocks = dtype, n_blocks
@@ -34,6 +34,20 @@ class Served:
         self.truth = {s: (empty, empty) for s in self.slots}     # slot -> (K rows, V rows) it logically holds
         self.tol = 2e-3 if dtype == abi.ESP_F16 else 4e-3
         self.max_rows = device.plan_hint3(self.ap)[2]
+        # a sliding layer beside it: one ring of rb blocks per slot in a pool of its own (forest.h:2657-2700)
+        self.W = window
+        if window:
+            self.rb = (window + bt - 1) // bt
+            self.ap_s = synth.make_params(H, Hkv, HD, dtype, bt, window=window, ring=self.rb)
+            self.ring_region = n_slots * self.rb * 2 * bt * self.ap.kv_ld
+            self.ring_ref = np.zeros(self.ring_region, np.uint16)
+            self.ring = torch.zeros(self.ring_region, dtype=torch.int16, device="cuda")
+
+    def ring_copy(self, pairs):
+        pairs = np.ascontiguousarray(pairs, np.int32)
+        if len(pairs):
+            device.kv_copy_blocks(self.ap_s, self.ring, device.to_dev(pairs), len(pairs), 1, self.ring_region)
+            ob.kv_copy_blocks(self.ap_s, self.ring_ref, pairs, 1, self.ring_region)
 
     def reset(self, s):
         self.e.slot_reset(s)
@@ -43,6 +57,8 @@ class Served:
         self.reset(b)
         self.e.slot_fork(a, b)
         self.truth[b] = self.truth[a]
+        if self.W:                                                 # a fork copies the whole ring (forest.h:127-137)
+            self.ring_copy([(a * self.rb + i, b * self.rb + i) for i in range(self.rb)])
 
     def run(self, specs, rows_per_tile, commit=True, tag=""):
         """specs: [(parent, save, root_len, leaves, commit_chain)]. False if the engine refused the pass."""
@@ -79,6 +95,23 @@ class Served:
         want = ob.attn_direct(ap, Q, Kb, Vb, self.pool_ref, blocks, ps["desc"], ps["pos"], ps["trees"], n_threads=8)
         err = float(np.abs(f32(to_host_u16(O).reshape(M, -1), dtype) - f32(want, dtype)).max())
         assert err <= self.tol, (tag, err)
+        if self.W:                                                 # the same rows through the sliding layer
+            rg = e.pass_rings(self.W, self.rb)
+            self.ring_copy(rg["copies"])
+            aps = self.ap_s
+            aps.rows_per_tile = rows_per_tile
+            resident, groups = device.plan_hint(aps)
+            tiles, jobs, n_parts = host.plan_tiles(rg["trees"], groups, self.W, ps["pos"], host.options_mi355x(rows_per_tile, resident))
+            dps = device.DevicePass(aps, rg["trees"], tiles, jobs, n_parts, M, np.zeros(1, np.int32), ps["desc"], ps["pos"])
+            Os = torch.zeros_like(Qd)
+            dps.run(Qd, Kd, Vd, self.ring, Os)
+            torch.cuda.synchronize()
+            want = ob.attn_direct(aps, Q, Kb, Vb, self.ring_ref, np.zeros(1, np.int32), ps["desc"], ps["pos"], rg["trees"], n_threads=8)
+            err = float(np.abs(f32(to_host_u16(Os).reshape(M, -1), dtype) - f32(want, dtype)).max())
+            assert err <= self.tol, (tag, "sliding", err)
+            if commit and len(rg["saves"]):
+                device.kv_save(aps, Kd, Vd, self.ring, device.to_dev(rg["saves"]), len(rg["saves"]))
+                ob.kv_save(aps, Kb, Vb, self.ring_ref, rg["saves"])
         if not commit:
             e.pass_abort()     # the copied blocks go back to the free list; nothing a slot lists has changed
             self.check_slots(tag)
@@ -105,6 +138,11 @@ class Served:
             if n:
                 kw, vw = ob.kv_gather(self.ap, self.pool_ref, self.e.slot_blocks(s), n)
                 assert np.array_equal(kw, self.truth[s][0]) and np.array_equal(vw, self.truth[s][1]), (tag, s)
+            if n and self.W:                                       # the ring reads back what the slot's next row can see
+                lo = max(0, n - self.W + 1)
+                order = [s * self.rb + i % self.rb for i in range((n + self.ap.bt - 1) // self.ap.bt)]
+                kw, vw = ob.kv_gather(self.ap_s, self.ring_ref, np.array(order, np.int32), n)
+                assert np.array_equal(kw[lo:], self.truth[s][0][lo:]) and np.array_equal(vw[lo:], self.truth[s][1][lo:]), (tag, s, "ring")
 
     def finish(self):
         """The device pool holds what the reference-layout pool holds, block for block, and every slot reads back
@@ -114,6 +152,11 @@ class Served:
         device.kv_relayout(self.ap, self.pool, abi.ESP_LAYOUT_NATIVE, back, abi.ESP_LAYOUT_REFERENCE, self.n_blocks)
         torch.cuda.synchronize()
         assert np.array_equal(to_host_u16(back), self.pool_ref)
+        if self.W:
+            back = torch.zeros_like(self.ring)
+            device.kv_relayout(self.ap_s, self.ring, abi.ESP_LAYOUT_NATIVE, back, abi.ESP_LAYOUT_REFERENCE, len(self.slots) * self.rb)
+            torch.cuda.synchronize()
+            assert np.array_equal(to_host_u16(back), self.ring_ref)
         for s in self.slots:
             n = len(self.truth[s][0])
             if not n:
@@ -128,7 +171,7 @@ class Served:
 
 @pytest.mark.parametrize("H,Hkv,HD,bt,dtype", [(8, 2, 128, 16, abi.ESP_F16), (8, 1, 512, 32, abi.ESP_F16), (6, 3, 256, 64, abi.ESP_BF16)])
 def test_engine_records_drive_the_kernels_through_a_serving_history(H, Hkv, HD, bt, dtype):
-    sv = Served(H, Hkv, HD, bt, dtype, 96, 4, H + HD)
+    sv = Served(H, Hkv, HD, bt, dtype, 96, 4, H + HD, window={128: 40, 256: 100, 512: 0}[HD])
     A, B, Cc, D = sv.slots
     e = sv.e
     G = H // Hkv
@@ -157,13 +200,14 @@ def _random_leaves(rng):
 def test_random_serving_histories(seed):
     """Random passes of up to three trees (chunks, decode rows, verify trees; in place, into another slot, from
     nothing), forks and resets in between, one pass in four not committed, a pool small enough that some
-    passes are refused; geometry, block size and tile height drawn per history."""
+    passes are refused; geometry, block size, tile height and the sliding layer's window drawn per history."""
     rng = np.random.default_rng(4000 + seed)
     H, Hkv, HD = [(8, 2, 128), (4, 4, 128), (16, 2, 256), (6, 3, 256), (8, 1, 512), (4, 2, 512)][seed % 6]
     bt = int(rng.choice([16, 32, 64]))
     dtype = abi.ESP_F16 if seed % 2 == 0 else abi.ESP_BF16
     n_slots = 4
-    sv = Served(H, Hkv, HD, bt, dtype, int(rng.integers(24, 64)) * 64 // bt, n_slots, 5000 + seed)
+    window = 0 if HD == 512 else int(rng.integers(20, 200))       # 512-dim heads are the layers without a window
+    sv = Served(H, Hkv, HD, bt, dtype, int(rng.integers(24, 64)) * 64 // bt, n_slots, 5000 + seed, window)
     heights = [r for r in (1, 2, 4, 8, 16, sv.max_rows) if r <= sv.max_rows]
     n_passes = 0
     for step in range(30):

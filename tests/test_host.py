@@ -255,6 +255,11 @@ def test_random_slot_histories_keep_every_slot_readable(seed):
     truth = {s: [] for s in slots}
     pool = np.full((n_blocks, bt), -1, np.int64)
     next_tok = [1]
+    # sliding layers: a second toy pool of one ring per slot (forest.h:2657-2700); what a slot's next row can see
+    # there - its last W - 1 positions - must read back too
+    W = int(rng.integers(5, 120))
+    rb = (W + bt - 1) // bt + int(rng.integers(0, 2))
+    ring = np.full((n_slots * rb, bt), -1, np.int64)
 
     def read(blocks, n):
         return [int(x) for x in pool[list(blocks)].reshape(-1)[:n]] if n else []
@@ -263,6 +268,9 @@ def test_random_slot_histories_keep_every_slot_readable(seed):
         for s in slots:
             assert e.slot_len(s) == len(truth[s])
             assert read(e.slot_blocks(s), len(truth[s])) == truth[s], (seed, s)
+            L = len(truth[s])
+            for p_ in range(max(0, L - W + 1), L):
+                assert ring[s * rb + (p_ // bt) % rb, p_ % bt] == truth[s][p_], (seed, s, p_)
         _conservation(e, n_blocks, slots)
 
     for step in range(120):
@@ -272,6 +280,7 @@ def test_random_slot_histories_keep_every_slot_readable(seed):
             e.slot_reset(b)
             e.slot_fork(a, b)
             truth[b] = list(truth[a])
+            ring[b * rb:(b + 1) * rb] = ring[a * rb:(a + 1) * rb]   # a fork copies the whole ring (forest.h:127-137)
         elif op == "reset":
             a = int(rng.choice(slots))
             e.slot_reset(a)
@@ -316,6 +325,17 @@ def test_random_slot_histories_keep_every_slot_readable(seed):
                     tab = ps["table"][int(t["table"]):int(t["table"]) + nb]
                     cowmap = {int(dst): int(src) for src, dst in ps["cow"].tolist()}
                     assert [int(x) for x in pool[[cowmap.get(int(b), int(b)) for b in tab]].reshape(-1)[:len(truth[parent])]] == truth[parent]
+            rg = e.pass_rings(W, rb)
+            want = ho.ring_plan([(int(t["base"]), int(t["P"]), int(t["M"]), parent, [(d, len(toks))])
+                                 for t, (parent, d, toks) in zip(ps["trees"], plan)], W, rb, bt)
+            assert [tuple(int(x) for x in t) for t in rg["trees"]] == want[0]
+            assert [tuple(int(x) for x in t) for t in rg["saves"]] == want[1]
+            assert [tuple(c) for c in rg["copies"].tolist()] == want[2]
+            ring_before = ring.copy()
+            for src, dst in rg["copies"].tolist():                   # copies, then saves
+                ring[dst] = ring[src]
+            for sv in rg["saves"]:
+                ring[int(sv["block"]), int(sv["pos"])] = rows[int(sv["src_row"])]
             for src, dst in ps["cow"].tolist():
                 pool[dst] = pool[src]
             for sv in ps["saves"]:
@@ -323,6 +343,7 @@ def test_random_slot_histories_keep_every_slot_readable(seed):
             if rng.integers(0, 4) == 0:
                 e.pass_abort()
                 pool[:] = before[0]
+                ring[:] = ring_before      # an in-place chunk's saves reuse ring cells the slot still needs if it does not advance
                 assert ({s: list(e.slot_blocks(s)) for s in slots}, e.free_blocks()) == before[1:]
             else:
                 e.pass_commit()
