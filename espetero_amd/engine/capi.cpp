@@ -218,6 +218,33 @@ int esp_slot_file_load(const char* path, int32_t bt, void* kv, uint64_t kv_bytes
   if (kv_bytes < uint64_t(s.n_layers) * uint64_t(s.n_blocks) * s.block_bytes) return -1;
   return espetero::engine::slot_file_load(path, s, kv);
 }
+int esp_slot_file_save_rings(const char* path, int32_t len, int32_t next_pos, int32_t n_blocks, int32_t n_layers,
+                             uint64_t block_bytes, const void* kv, int32_t r_layers, int32_t r_blocks, uint64_t rblock_bytes,
+                             const void* rings) {
+  if (!path || len < 0 || n_blocks < 0 || n_layers < 0 || (!kv && n_blocks > 0 && n_layers > 0)) return -1;
+  if (r_layers < 0 || r_blocks < 0 || (!rings && r_layers > 0 && r_blocks > 0 && rblock_bytes > 0)) return -1;
+  espetero::engine::SlotInfo s;
+  s.len = len, s.next_pos = next_pos, s.n_blocks = n_blocks, s.n_layers = n_layers, s.block_bytes = block_bytes;
+  s.r_layers = r_layers, s.r_blocks = r_blocks, s.rblock_bytes = rblock_bytes;
+  return espetero::engine::slot_file_save(path, s, kv, rings) ? 0 : -1;
+}
+int esp_slot_file_info_rings(const char* path, int32_t bt, int32_t* len, int32_t* next_pos, int32_t* n_blocks, int32_t* n_layers,
+                             uint64_t* block_bytes, int32_t* r_layers, int32_t* r_blocks, uint64_t* rblock_bytes) {
+  if (!path || bt <= 0) return -1;
+  espetero::engine::SlotInfo s;
+  if (espetero::engine::slot_file_info(path, bt, &s, true) != 0) return -1;
+  *len = s.len, *next_pos = s.next_pos, *n_blocks = s.n_blocks, *n_layers = s.n_layers, *block_bytes = s.block_bytes;
+  *r_layers = s.r_layers, *r_blocks = s.r_blocks, *rblock_bytes = s.rblock_bytes;
+  return 0;
+}
+int esp_slot_file_load_rings(const char* path, int32_t bt, void* kv, uint64_t kv_bytes, void* rings, uint64_t ring_bytes) {
+  if (!path || bt <= 0) return -1;
+  espetero::engine::SlotInfo s;
+  if (espetero::engine::slot_file_info(path, bt, &s, true) != 0) return -1;
+  if (kv_bytes < uint64_t(s.n_layers) * uint64_t(s.n_blocks) * s.block_bytes) return -1;
+  if (ring_bytes < s.ring_bytes() || (s.ring_bytes() && !rings)) return -1;
+  return espetero::engine::slot_file_load(path, s, kv, rings);
+}
 int esp_engine_pass_commit(esp_engine* e) { return guarded([&] { e->e.pass_commit(); }); }
 int esp_engine_pass_abort(esp_engine* e) { return guarded([&] { e->e.pass_abort(); }); }
 

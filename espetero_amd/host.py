@@ -53,6 +53,10 @@ ENGINE_SYMBOLS = {
     "esp_slot_file_save": (C.c_int, (C.c_char_p, C.c_int32, C.c_int32, C.c_int32, C.c_int32, C.c_uint64, _V)),
     "esp_slot_file_info": (C.c_int, (C.c_char_p, C.c_int32, _V, _V, _V, _V, _V)),
     "esp_slot_file_load": (C.c_int, (C.c_char_p, C.c_int32, _V, C.c_uint64)),
+    "esp_slot_file_save_rings": (C.c_int, (C.c_char_p, C.c_int32, C.c_int32, C.c_int32, C.c_int32, C.c_uint64, _V, C.c_int32, C.c_int32,
+                                            C.c_uint64, _V)),
+    "esp_slot_file_info_rings": (C.c_int, (C.c_char_p, C.c_int32, _V, _V, _V, _V, _V, _V, _V, _V)),
+    "esp_slot_file_load_rings": (C.c_int, (C.c_char_p, C.c_int32, _V, C.c_uint64, _V, C.c_uint64)),
     "esp_kv_row_table": (C.c_int, (_V, C.c_int32, C.c_int32, _V, C.c_char_p, C.c_size_t)),
     "esp_engine_pass_commit": (C.c_int, (_V,)),
     "esp_engine_pass_abort": (C.c_int, (_V,)),
@@ -117,6 +121,40 @@ def slot_file_save(path, length, next_pos, n_layers, blocks_kv):
                                          kv.ctypes.data if kv.size else None)
     if rc != 0:
         raise abi.EspError(f"slot_file_save({path}) failed")
+
+
+def slot_file_save_rings(path, length, next_pos, n_layers, blocks_kv, rings):
+    """slot_file_save with the ring section: rings = host array [r_layers][r_blocks][block elements], the slot's ring of
+    every sliding layer in ring order, reference block layout."""
+    kv, rg = np.ascontiguousarray(blocks_kv), np.ascontiguousarray(rings)
+    assert kv.shape[0] == n_layers
+    n_blocks = kv.shape[1]
+    rc = engine_lib().esp_slot_file_save_rings(str(path).encode(), length, next_pos, n_blocks, n_layers,
+                                               kv[0, 0].nbytes if n_blocks else 0, kv.ctypes.data if kv.size else None,
+                                               rg.shape[0], rg.shape[1], rg[0, 0].nbytes if rg.size else 0,
+                                               rg.ctypes.data if rg.size else None)
+    if rc != 0:
+        raise abi.EspError(f"slot_file_save_rings({path}) failed")
+
+
+def slot_file_load_rings(path, bt):
+    """slot_file_load for files with or without a ring section: the same dict plus r_layers, r_blocks, rblock_bytes and
+    rings = uint8 [r_layers][r_blocks][rblock_bytes]; None for a refused file."""
+    v = [C.c_int32(0) for _ in range(4)]
+    r = [C.c_int32(0) for _ in range(2)]
+    bb, rbb = C.c_uint64(0), C.c_uint64(0)
+    lib = engine_lib()
+    if lib.esp_slot_file_info_rings(str(path).encode(), bt, *[C.byref(x) for x in v], C.byref(bb), *[C.byref(x) for x in r],
+                                    C.byref(rbb)) != 0:
+        return None
+    length, next_pos, n_blocks, n_layers = (x.value for x in v)
+    kv = np.zeros((n_layers, n_blocks, bb.value), np.uint8)
+    rings = np.zeros((r[0].value, r[1].value, rbb.value), np.uint8)
+    if lib.esp_slot_file_load_rings(str(path).encode(), bt, kv.ctypes.data if kv.size else None, kv.nbytes,
+                                    rings.ctypes.data if rings.size else None, rings.nbytes) != 0:
+        return None
+    return dict(len=length, next_pos=next_pos, n_blocks=n_blocks, n_layers=n_layers, block_bytes=bb.value, kv=kv,
+                r_layers=r[0].value, r_blocks=r[1].value, rblock_bytes=rbb.value, rings=rings)
 
 
 def slot_file_load(path, bt):

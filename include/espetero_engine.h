@@ -112,7 +112,8 @@ int esp_engine_pass_rings(const esp_engine* e, int32_t window, int32_t ring_bloc
 /* Slot checkpoint files in the reference's format (src/model/model.mm:600-752), KV section: the
  * 120-byte CkptHeader (magic 0x554b5043, version 4), then n_layers x n_blocks blocks of block_bytes,
  * layer-major, logical block order, each in the reference's block layout (what
- * esp_kv_export_blocks produces per layer). The sections of other subsystems are written as absent.
+ * esp_kv_export_blocks produces per layer). The sections of other subsystems are written as absent;
+ * a file with a ring section is refused here (the _rings variants below take it).
  * kv: host memory. save: 0 or -1. info / load: 0, or -1 for a missing, malformed, wrong-version or
  * wrong-size file or one with sections this build does not take (slot_load's -1, model.mm:700-714). */
 int esp_slot_file_save(const char* path, int32_t len, int32_t next_pos, int32_t n_blocks, int32_t n_layers, uint64_t block_bytes,
@@ -120,6 +121,17 @@ int esp_slot_file_save(const char* path, int32_t len, int32_t next_pos, int32_t 
 int esp_slot_file_info(const char* path, int32_t bt, int32_t* len, int32_t* next_pos, int32_t* n_blocks, int32_t* n_layers,
                        uint64_t* block_bytes);
 int esp_slot_file_load(const char* path, int32_t bt, void* kv, uint64_t kv_bytes);
+/* The same with the file's last section, Gemma's sliding rings (model.mm:664-669, 737-742): after the KV
+ * blocks, r_layers x r_blocks ring blocks of rblock_bytes, layer-major, the slot's ring in ring order
+ * (what esp_kv_export_blocks produces from the ring pool for blocks slot * r_blocks + 0 .. r_blocks - 1).
+ * info / load take files with and without rings; a loader must still hold the counts against its own
+ * model (r_layers, r_blocks, rblock_bytes: slot_load's checks, model.mm:703-705). */
+int esp_slot_file_save_rings(const char* path, int32_t len, int32_t next_pos, int32_t n_blocks, int32_t n_layers,
+                             uint64_t block_bytes, const void* kv, int32_t r_layers, int32_t r_blocks, uint64_t rblock_bytes,
+                             const void* rings);
+int esp_slot_file_info_rings(const char* path, int32_t bt, int32_t* len, int32_t* next_pos, int32_t* n_blocks, int32_t* n_layers,
+                             uint64_t* block_bytes, int32_t* r_layers, int32_t* r_blocks, uint64_t* rblock_bytes);
+int esp_slot_file_load_rings(const char* path, int32_t bt, void* kv, uint64_t kv_bytes, void* rings, uint64_t ring_bytes);
 /* kv_row_table (src/model/impl/forest.h:1737-1749): the pass's save records as one int32[4] per row,
  * (block, position, block2, position2), -1 none - the row_table argument of esp_attn_prep.
  * out: 4 * max(rows, 1) ints. Fails on a row saved into more than two slots. Needs no engine. */

@@ -160,3 +160,52 @@ def test_slot_checkpoint_round_trip_through_a_file(tmp_path):
             outs.append(O)
         assert torch.equal(outs[0], outs[1]) and bool(outs[0].any())
     p.kv_base = 0
+
+
+def test_slot_file_ring_section_reloads_a_sliding_layer_bit_identically(tmp_path):
+    """A slot's ring of a sliding layer leaves through esp_kv_export_blocks (its ring blocks in ring order), travels
+    in the slot file's ring section (model.mm:664-669), and comes back into another slot's ring: the sliding
+    layer's attention over the reloaded ring is bit-identical."""
+    from espetero_amd import host
+    from gpu_utils import dev_u16, native_pool, to_host_u16
+    device.init(0)
+    bt, window = 16, 100
+    c = synth.make_case("ringfile", 31, 8, 2, 256, abi.ESP_F16, bt, [(50, 1), (777, 1), (300, 1)], window=window, ring_layer=True,
+                        rows_per_tile=1)
+    p = c.params
+    rb = p.ring
+    blk = 2 * bt * p.kv_ld
+    pool = native_pool(c)
+    slot, new_slot = 1, 2
+    assert int(c.trees[slot]["table"]) == slot * rb
+    mine = np.arange(slot * rb, (slot + 1) * rb, dtype=np.int32)
+    out = torch.zeros(1, rb, blk, dtype=torch.int16, device="cuda")
+    device.kv_export_blocks(p, pool, device.to_dev(mine), rb, out[0])
+    torch.cuda.synchronize()
+    rings = to_host_u16(out)
+    assert np.array_equal(rings[0], c.pool_ref.reshape(c.n_blocks, blk)[mine])      # == the checker's ring blocks
+    P = int(c.trees[slot]["P"])
+    path = tmp_path / "ring.ckpt"
+    full = np.zeros((1, (P + bt - 1) // bt, 64), np.uint16)       # stands for the full-attention layers' blocks: the header's length must fit them
+    host.slot_file_save_rings(path, P, P, 1, full, rings)
+    got = host.slot_file_load_rings(path, bt)
+    assert got is not None and (got["len"], got["r_layers"], got["r_blocks"], got["rblock_bytes"]) == (P, 1, rb, blk * 2)
+    pool2 = torch.zeros_like(pool)
+    theirs = np.arange(new_slot * rb, (new_slot + 1) * rb, dtype=np.int32)
+    device.kv_import_blocks(p, dev_u16(got["rings"].view(np.uint16).reshape(1, rb, blk)[0]), device.to_dev(theirs), rb, pool2)
+    torch.cuda.synchronize()
+    # the sequence alone, from its own ring and from the reloaded one
+    row = int(c.trees[slot]["base"])
+    Q, Kb, Vb = (dev_u16(x[row:row + 1]) for x in (c.Q, c.Kb, c.Vb))
+    pos = np.ascontiguousarray(c.pos.reshape(-1, 4)[row:row + 1])
+    resident, groups = device.plan_hint(p)
+    outs = []
+    for pl, tab in ((pool, slot * rb), (pool2, new_slot * rb)):
+        trees = np.array([(0, P, tab, 1)], abi.TREE_DT)
+        tiles, jobs, n_parts = host.plan_tiles(trees, groups, window, pos, host.options_mi355x(1, resident))
+        dp = device.DevicePass(p, trees, tiles, jobs, n_parts, 1, np.zeros(1, np.int32), None, pos)
+        O = torch.zeros_like(Q)
+        dp.run(Q, Kb, Vb, pl, O)
+        torch.cuda.synchronize()
+        outs.append(O)
+    assert torch.equal(outs[0], outs[1]) and bool(outs[0].any())

@@ -464,3 +464,34 @@ def test_slot_file_round_trip_layout_and_refusals(tmp_path):
     host.slot_file_save(tmp_path / "empty.ckpt", 0, 0, n_layers, np.zeros((n_layers, 0, 2 * bt * kvw), np.uint16))
     e = host.slot_file_load(tmp_path / "empty.ckpt", bt)
     assert e["n_blocks"] == 0 and (tmp_path / "empty.ckpt").stat().st_size == 120
+
+
+def test_slot_file_ring_section(tmp_path):
+    """The file's last section (src/model/model.mm:664-669, 737-742): after the KV blocks, per sliding layer the
+    slot's ring, r_blocks blocks of rblock_bytes; counts in the header's last three fields (:611-612)."""
+    import struct
+    rng = np.random.default_rng(7)
+    n_layers, n_blocks, bt, kvw_g, kvw_s, r_layers, rb = 2, 4, 16, 2 * 512, 8 * 256, 5, 3
+    kv = rng.integers(0, 65536, (n_layers, n_blocks, 2 * bt * kvw_g), dtype=np.uint16)
+    rings = rng.integers(0, 65536, (r_layers, rb, 2 * bt * kvw_s), dtype=np.uint16)
+    path = tmp_path / "g4.ckpt"
+    host.slot_file_save_rings(path, 60, 61, n_layers, kv, rings)
+    raw = path.read_bytes()
+    assert len(raw) == 120 + kv.nbytes + rings.nbytes
+    assert struct.unpack_from("<iiQ", raw, 104) == (r_layers, rb, 2 * bt * kvw_s * 2)
+    assert raw[120:120 + kv.nbytes] == kv.tobytes() and raw[120 + kv.nbytes:] == rings.tobytes()
+    got = host.slot_file_load_rings(path, bt)
+    assert (got["len"], got["next_pos"], got["r_layers"], got["r_blocks"]) == (60, 61, r_layers, rb)
+    assert np.array_equal(got["kv"].view(np.uint16).reshape(kv.shape), kv)
+    assert np.array_equal(got["rings"].view(np.uint16).reshape(rings.shape), rings)
+    assert host.slot_file_load(path, bt) is None                  # a loader without ring pools refuses it
+    (tmp_path / "short.ckpt").write_bytes(raw[:-2])
+    assert host.slot_file_load_rings(tmp_path / "short.ckpt", bt) is None
+    bad = bytearray(raw)
+    struct.pack_into("<i", bad, 104, 0)                           # ring blocks without ring layers
+    (tmp_path / "norl.ckpt").write_bytes(bytes(bad))
+    assert host.slot_file_load_rings(tmp_path / "norl.ckpt", bt) is None
+    # a file without rings loads through either call
+    host.slot_file_save(tmp_path / "plain.ckpt", 60, 61, n_layers, kv)
+    p = host.slot_file_load_rings(tmp_path / "plain.ckpt", bt)
+    assert p["r_layers"] == 0 and p["rings"].size == 0 and np.array_equal(p["kv"].view(np.uint16).reshape(kv.shape), kv)
