@@ -116,6 +116,29 @@ int esp_engine_slot_blocks(const esp_engine* e, int32_t s, int32_t* out, int32_t
     return -1;
   }
 }
+int esp_engine_slot_next_pos(const esp_engine* e, int32_t s) {
+  try {
+    const Slot& sl = e->e.slot(s);
+    return sl.used ? sl.next_pos : -1;
+  } catch (...) {
+    return -1;
+  }
+}
+int esp_engine_slot_chain(const esp_engine* e, int32_t s) {
+  try {
+    return e->e.slot_chain(s);
+  } catch (...) {
+    return -1;
+  }
+}
+int esp_engine_chain_commit(esp_engine* e, int32_t s, int32_t n, char* err, size_t errlen) {
+  try {
+    e->e.chain_commit(s, n);
+    return ESP_OK;
+  } catch (const std::exception& ex) {
+    return put_err(err, errlen, ESP_EINVAL, ex.what());
+  }
+}
 int esp_engine_free_blocks(const esp_engine* e) { return e->e.pool().n_free(); }
 int esp_engine_block_ref(const esp_engine* e, int32_t b) {
   return (b < 0 || b >= e->e.pool().n_blocks) ? -1 : e->e.pool().ref[size_t(b)];

@@ -13,6 +13,7 @@
 //   sliding-layer rings     src/model/impl/forest.h:2657-2700 (trees, saves, window copies)
 //   commit / rollback       src/model/impl/forest.h:2468-2482, 4743-4754
 //   slot operations         src/model/model.mm:520-553
+//   verify-commit           src/model/impl/forest.h:4755-4765, 4846-4861, 5058-5069 (length / position side)
 // A pass never changes a slot before commit(): a failure (or abort()) gives
 // the new blocks back and leaves every slot as it was.
 #pragma once
@@ -38,7 +39,11 @@ struct Slot {
   bool used = false;
   int len = 0;
   int next_pos = 0;
-  std::vector<int> blocks;  // block ids covering positions [0, len)
+  std::vector<int> blocks;  // block ids covering positions [0, len) (and the kept chain rows behind them)
+  // The commit record of the slot's last pass (forest.h:4755-4765): cm_k chain rows whose K / V already sit at
+  // positions len .. len + cm_k - 1, the first at rotary position cm_pos0; valid until another pass begins.
+  int cm_k = 0, cm_pos0 = 0;
+  uint64_t cm_pass = 0;
 };
 
 struct KvPool {
@@ -122,17 +127,40 @@ class KvEngine {
     Slot& sl = checked(s);
     release_blocks(sl);
     sl.len = sl.next_pos = 0;
+    sl.cm_k = 0;
   }
-  // dst becomes a copy of src sharing its blocks by refcount (model.mm:542-553).
+  // dst becomes a copy of src sharing the blocks of its [0, len) by refcount; the chain rows stay the
+  // source's (model.mm:542-553).
   void slot_fork(int src, int dst) {
     Slot& a = checked(src);
     Slot& b = checked(dst);
     if (src == dst) return;
     release_blocks(b);
-    b.blocks = a.blocks;
+    const size_t nb = std::min(size_t((a.len + pool_.bt - 1) / pool_.bt), a.blocks.size());
+    b.blocks.assign(a.blocks.begin(), a.blocks.begin() + long(nb));
     for (int blk : b.blocks) pool_.retain(blk);
     b.len = a.len;
     b.next_pos = a.next_pos;
+    b.cm_k = 0;
+  }
+  // Chain rows of `s` that chain_commit could still take: those its last pass kept, while no other pass has begun.
+  int slot_chain(int s) const {
+    const Slot& sl = slots_.at(size_t(s));
+    return sl.used && sl.cm_pass == pass_seq_ ? sl.cm_k : 0;
+  }
+  // Verify-commit, the block-pool side (run_commit, forest.h:4846-4861, 5058-5069): the first n rows of the
+  // chain the slot's last pass kept (esp_tree_spec::commit_chain) become part of the slot. Their K / V are
+  // already at their positions; length and next position follow, and the rest of the chain is dropped.
+  void chain_commit(int s, int n) {
+    Slot& sl = checked(s);
+    if (pass_.pending) fail("commit: a pass is pending");
+    if (n < 0 || n > sl.cm_k || (n > 0 && sl.cm_pass != pass_seq_))
+      fail("commit: slot " + std::to_string(s) + " holds no such chain rows of the last pass");
+    if (n > 0) {
+      sl.len += n;
+      sl.next_pos = sl.cm_pos0 + n;
+    }
+    sl.cm_k = 0;
   }
 
   // Blocks Forest::target_blocks would allocate for one target (forest.h:1821-1829).
@@ -364,6 +392,7 @@ class KvEngine {
     guard.armed = false;
     ps.pending = true;
     pass_ = std::move(ps);
+    ++pass_seq_;  // the chain rows earlier passes kept are no longer committable
   }
 
   // The pending pass as the sliding layers see it (Gemma: the last `window` positions of slot s live in a second
@@ -385,6 +414,7 @@ class KvEngine {
     if (W <= 0 || rb <= 0 || int64_t(rb) * bt < W) fail("ring_plan: the ring must hold the window");
     RingPlan out;
     for (const TreePlan& T : pass_.trees) {
+      if (T.cm_k) fail("ring_plan: commit_chain is not supported on sliding layers");  // forest.h:2237
       const int parent = T.spec.parent;
       out.trees.push_back({T.base, T.P, parent >= 0 ? parent * rb : 0, T.M});
       auto target = [&](int slot, int S) {
@@ -412,8 +442,17 @@ class KvEngine {
         to.len = len;
         to.next_pos = next;
       };
-      if (T.spec.save >= 0) commit(T.spec.save, T.dst_blocks, T.P + T.save_len, T.save_len == T.Tr ? T.next_root : T.next_save);
-      if (T.spec.work >= 0) commit(T.spec.work, T.work_blocks, T.P + T.Tr, T.next_root);
+      if (T.spec.save >= 0) {
+        commit(T.spec.save, T.dst_blocks, T.P + T.save_len, T.save_len == T.Tr ? T.next_root : T.next_save);
+        Slot& to = slots_[size_t(T.spec.save)];
+        to.cm_k = T.cm_k;
+        to.cm_pos0 = T.next_root;
+        to.cm_pass = pass_seq_;
+      }
+      if (T.spec.work >= 0) {
+        commit(T.spec.work, T.work_blocks, T.P + T.Tr, T.next_root);
+        slots_[size_t(T.spec.work)].cm_k = 0;
+      }
     }
     pass_ = Pass{};
   }
@@ -446,6 +485,7 @@ class KvEngine {
   std::vector<Slot> slots_;
   int max_ctx_;
   Pass pass_;
+  uint64_t pass_seq_ = 0;
 };
 
 }  // namespace espetero::engine

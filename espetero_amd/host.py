@@ -37,6 +37,9 @@ ENGINE_SYMBOLS = {
     "esp_engine_slot_fork": (C.c_int, (_V, _I, _I)),
     "esp_engine_slot_len": (C.c_int, (_V, _I)),
     "esp_engine_slot_blocks": (C.c_int, (_V, _I, _V, _I)),
+    "esp_engine_slot_next_pos": (C.c_int, (_V, _I)),
+    "esp_engine_slot_chain": (C.c_int, (_V, _I)),
+    "esp_engine_chain_commit": (C.c_int, (_V, _I, _I) + _ERR),
     "esp_engine_free_blocks": (C.c_int, (_V,)),
     "esp_engine_block_ref": (C.c_int, (_V, _I)),
     "esp_engine_pass_blocks": (C.c_int, (_V, _TS, _I)),
@@ -234,6 +237,17 @@ class Engine:
 
     def slot_len(self, s):
         return self.lib.esp_engine_slot_len(self.h, s)
+
+    def slot_next_pos(self, s):
+        return self.lib.esp_engine_slot_next_pos(self.h, s)
+
+    def slot_chain(self, s):
+        return self.lib.esp_engine_slot_chain(self.h, s)
+
+    def chain_commit(self, s, n):
+        """The first n chain rows the slot's last pass kept become part of the slot. Raises EspError when refused."""
+        err = C.create_string_buffer(256)
+        abi.check(self.lib.esp_engine_chain_commit(self.h, s, n, err, 256), err)
 
     def slot_blocks(self, s):
         n = self.lib.esp_engine_slot_blocks(self.h, s, None, 0)

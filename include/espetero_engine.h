@@ -13,6 +13,7 @@
  *   slot commit / PassGuard        src/model/impl/forest.h:2468-2482, 4743-4754
  *   sliding-layer ring planning    src/model/impl/forest.h:2657-2700
  *   slot_alloc/free/reset/fork/len src/model/model.mm:520-553
+ *   verify-commit (lengths)        src/model/impl/forest.h:4755-4765, 4846-4861, 5058-5069
  * The C++ headers are the interface a C++ engine includes; these functions
  * exist so that other languages (and the tests) can drive the same code.
  * Errors: 0 / non-zero + message in err, as in espetero_attn.h. Host memory only.
@@ -74,6 +75,14 @@ int esp_engine_slot_free(esp_engine* e, int32_t slot);
 int esp_engine_slot_reset(esp_engine* e, int32_t slot);
 int esp_engine_slot_fork(esp_engine* e, int32_t src, int32_t dst);
 int esp_engine_slot_len(const esp_engine* e, int32_t slot);
+int esp_engine_slot_next_pos(const esp_engine* e, int32_t slot);        /* rotary position of the slot's next token */
+/* Verify-commit, the block-pool side of the reference's run_commit (src/model/impl/forest.h:4846-4861,
+ * 5058-5069): the first n rows of the chain the slot's last pass kept (esp_tree_spec.commit_chain) become
+ * part of the slot - their K / V were saved at their positions by that pass - so its length grows by n and
+ * its next position follows; the rest of the chain is dropped. Refused when n exceeds the kept rows or
+ * another pass has begun since. slot_chain: the rows that could still be committed. */
+int esp_engine_slot_chain(const esp_engine* e, int32_t slot);
+int esp_engine_chain_commit(esp_engine* e, int32_t slot, int32_t n, char* err, size_t errlen);
 int esp_engine_slot_blocks(const esp_engine* e, int32_t slot, int32_t* out, int32_t cap); /* count */
 int esp_engine_free_blocks(const esp_engine* e);
 int esp_engine_block_ref(const esp_engine* e, int32_t block);

@@ -128,8 +128,20 @@ class Served:
                 b = int(t["base"])
                 new[save] = (np.concatenate([pk, Kb[b:b + root_len]]), np.concatenate([pv, Vb[b:b + root_len]]))
         self.truth.update(new)
+        self.last = (ps, specs, Kb, Vb)
         self.check_slots(tag)
         return True
+
+    def accept(self, slot, n):
+        """Verify-commit: the first n chain rows the last pass kept for `slot` join it (forest.h:4846-4861)."""
+        ps, specs, Kb, Vb = self.last
+        (t, spec), = [(t, sp) for t, sp in zip(ps["trees"], specs) if sp[1] == slot]
+        assert self.e.slot_chain(slot) == spec[4] and n <= spec[4]
+        self.e.chain_commit(slot, n)
+        print(f"accept {n} of {spec[4]} chain rows of slot {slot}", flush=True)
+        b = int(t["base"]) + spec[2]                               # the chain's rows follow the root's
+        self.truth[slot] = (np.concatenate([self.truth[slot][0], Kb[b:b + n]]), np.concatenate([self.truth[slot][1], Vb[b:b + n]]))
+        self.check_slots(f"accept {n} of slot {slot}")
 
     def check_slots(self, tag):
         for s in self.slots:
@@ -171,7 +183,7 @@ class Served:
 
 @pytest.mark.parametrize("H,Hkv,HD,bt,dtype", [(8, 2, 128, 16, abi.ESP_F16), (8, 1, 512, 32, abi.ESP_F16), (6, 3, 256, 64, abi.ESP_BF16)])
 def test_engine_records_drive_the_kernels_through_a_serving_history(H, Hkv, HD, bt, dtype):
-    sv = Served(H, Hkv, HD, bt, dtype, 96, 4, H + HD, window={128: 40, 256: 100, 512: 0}[HD])
+    sv = Served(H, Hkv, HD, bt, dtype, 96, 4, H + HD, window={128: 0, 256: 100, 512: 0}[HD])
     A, B, Cc, D = sv.slots
     e = sv.e
     G = H // Hkv
@@ -182,12 +194,16 @@ def test_engine_records_drive_the_kernels_through_a_serving_history(H, Hkv, HD, 
     drafts = [5, 6, 7]
     leaves = [drafts[:i + 1] for i in range(3)]
     rows_verify = 4 if HD < 512 else max(1, 16 // G)       # what the streaming kernel packs at this head dim
-    sv.run([(Cc, Cc, 1, leaves, 3), (A, A, 1, (), 0)], rows_verify, tag="verify C (fork of A: copy on write) + decode A")
+    chain = 0 if sv.W else 3                                # the reference keeps no chain on models with sliding layers (forest.h:2237)
+    sv.run([(Cc, Cc, 1, leaves, chain), (A, A, 1, (), 0)], rows_verify, tag="verify C (fork of A: copy on write) + decode A")
+    if chain:
+        sv.accept(Cc, 2)                                    # two of the three drafts accepted
     sv.run([(B, -1, 2, [[1, 2], [1, 3, 4], [9]], 0)], 8 if HD < 512 else max(1, 16 // G), commit=False,
            tag="wide verify tree on B, not committed")
     sv.run([(B, B, 45, (), 0), (A, D, 20, (), 0)], sv.max_rows, tag="chunk on B + A continued into D")
     sv.run([(s_, s_, 1, (), 0) for s_ in (A, B, Cc, D)], 1, tag="decode all four")
-    assert (e.slot_len(A), e.slot_len(B), e.slot_len(Cc), e.slot_len(D)) == (105, 106, 105, 125)   # the verify pass commits its root token only
+    # the verify pass commits its root token; the accepted drafts come on top
+    assert (e.slot_len(A), e.slot_len(B), e.slot_len(Cc), e.slot_len(D)) == (105, 106, 105 + (2 if chain else 0), 125)
     sv.finish()
 
 
@@ -206,7 +222,7 @@ def test_random_serving_histories(seed):
     bt = int(rng.choice([16, 32, 64]))
     dtype = abi.ESP_F16 if seed % 2 == 0 else abi.ESP_BF16
     n_slots = 4
-    window = 0 if HD == 512 else int(rng.integers(20, 200))       # 512-dim heads are the layers without a window
+    window = 0 if HD == 512 or seed == 0 else int(rng.integers(20, 200))   # 512-dim heads are the layers without a window
     sv = Served(H, Hkv, HD, bt, dtype, int(rng.integers(24, 64)) * 64 // bt, n_slots, 5000 + seed, window)
     heights = [r for r in (1, 2, 4, 8, 16, sv.max_rows) if r <= sv.max_rows]
     n_passes = 0
@@ -237,13 +253,19 @@ def test_random_serving_histories(seed):
                 specs.append((parent, d, 1, (), 0))
             else:
                 leaves = _random_leaves(rng)
-                chain = int(rng.integers(0, 2))
+                chain = int(rng.integers(0, 2)) if parent == d and not sv.W else 0   # kept chains: in place, no sliding layers
                 if chain:                                          # leaves [0, k) one chain: prefixes of one draft
                     draft = [int(x) for x in rng.integers(1, 4, int(rng.integers(1, 4)))]
                     leaves = [draft[:i + 1] for i in range(len(draft))] + [l for l in leaves if l[0] != draft[0]]
                     chain = len(draft)
                 specs.append((parent, d, int(rng.integers(1, 3)), leaves, chain))
         rows = 1 if all(s[2] == 1 and not s[3] for s in specs) else int(rng.choice(heights))
-        n_passes += sv.run(specs, rows, commit=rng.integers(0, 4) != 0, tag=f"seed {seed} step {step}")
+        commit = rng.integers(0, 4) != 0
+        ran = sv.run(specs, rows, commit=commit, tag=f"seed {seed} step {step}")
+        n_passes += ran
+        if ran and commit:
+            for sp in specs:
+                if sp[4] and rng.integers(0, 3):
+                    sv.accept(sp[1], int(rng.integers(0, sp[4] + 1)))
     assert n_passes >= 10
     sv.finish()

@@ -495,3 +495,58 @@ def test_slot_file_ring_section(tmp_path):
     host.slot_file_save(tmp_path / "plain.ckpt", 60, 61, n_layers, kv)
     p = host.slot_file_load_rings(tmp_path / "plain.ckpt", bt)
     assert p["r_layers"] == 0 and p["rings"].size == 0 and np.array_equal(p["kv"].view(np.uint16).reshape(kv.shape), kv)
+
+
+def test_verify_commit_takes_the_kept_chain_rows_into_the_slot():
+    """run_commit's block-pool side (src/model/impl/forest.h:4846-4861, 5058-5069): after a verify pass that kept a
+    chain of k draft rows, the first n of them join the slot - they already sit at positions len .. len + n - 1 -
+    and only while no other pass has begun; a fork does not inherit them (model.mm:551)."""
+    bt = 16
+    e = host.Engine(16, bt, 3)
+    a, b, c = (e.slot_alloc() for _ in range(3))
+    pool = np.full((16, bt), -1, np.int64)
+
+    def run(specs, tokens):
+        ps = e.pass_begin(specs)
+        for src, dst in ps["cow"].tolist():
+            pool[dst] = pool[src]
+        for sv in ps["saves"]:
+            pool[int(sv["block"]), int(sv["pos"])] = tokens[int(sv["src_row"])]
+        e.pass_commit()
+        return ps
+
+    def read(s, n):
+        return [int(x) for x in pool[list(e.slot_blocks(s))].reshape(-1)[:n]]
+
+    run([host.make_spec(save=a, root_len=30)], list(range(100, 130)))
+    assert e.slot_chain(a) == 0
+    drafts = [7, 8, 9]
+    ps = run([host.make_spec(parent=a, save=a, root_len=1, leaves=[drafts[:i + 1] for i in range(3)], commit_chain=3)],
+             [200, 201, 202, 203])                                      # row 0 the pending token, rows 1..3 the chain
+    assert ps["M"] == 4 and e.slot_len(a) == 31 and e.slot_next_pos(a) == 31 and e.slot_chain(a) == 3
+    assert [(int(s_["src_row"]), int(s_["pos"])) for s_ in ps["saves"]] == [(0, 30 % bt), (1, 31 % bt), (2, 0), (3, 1)]
+    with pytest.raises(abi.EspError):
+        e.chain_commit(a, 4)                                            # more than the pass kept
+    assert e.slot_chain(a) == 3                                         # a refused request changes nothing
+    e.slot_fork(a, b)
+    assert e.slot_len(b) == 31 and e.slot_chain(b) == 0 and len(e.slot_blocks(b)) == 2   # the fork: [0, len) only
+    with pytest.raises(abi.EspError):
+        e.chain_commit(b, 1)
+    e.chain_commit(a, 2)
+    assert e.slot_len(a) == 33 and e.slot_next_pos(a) == 33 and e.slot_chain(a) == 0
+    assert read(a, 33) == list(range(100, 130)) + [200, 201, 202]
+    with pytest.raises(abi.EspError):
+        e.chain_commit(a, 1)                                            # the rest of the chain was dropped
+    # the next token goes where the third draft row sat; the fork still reads its own 31
+    run([host.make_spec(parent=a, save=a, root_len=1)], [300])
+    assert read(a, 34) == list(range(100, 130)) + [200, 201, 202, 300] and read(b, 31) == list(range(100, 130)) + [200]
+    # chain rows are only committable until another pass begins, whichever slots it names
+    run([host.make_spec(parent=a, save=a, root_len=1, leaves=[[5]], commit_chain=1)], [301, 302])
+    assert e.slot_chain(a) == 1
+    run([host.make_spec(save=c, root_len=3)], [400, 401, 402])
+    assert e.slot_chain(a) == 0
+    with pytest.raises(abi.EspError):
+        e.chain_commit(a, 1)
+    e.chain_commit(a, 0)                                                # declining is always allowed
+    assert e.slot_len(a) == 35
+    _conservation(e, 16, [a, b, c])
