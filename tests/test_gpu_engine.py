@@ -20,7 +20,8 @@ pytestmark = pytest.mark.gpu
 
 
 class Served:
-    def __init__(self, H, Hkv, HD, bt, dtype, n_blocks, n_slots, seed, window=0):
+    def __init__(self, H, Hkv, HD, bt, dtype, n_blocks, n_slots, seed, window=0, sliding=None):
+        """sliding: (Hkv, head dim) of the sliding layer when they differ from the full layer's (Gemma 4: gemma.h:126-150)."""
         device.init(0)
         self.rng = np.random.default_rng(seed)
         self.dtype, self.n_blocks = dtype, n_blocks
@@ -38,8 +39,11 @@ class Served:
         self.W = window
         if window:
             self.rb = (window + bt - 1) // bt
-            self.ap_s = synth.make_params(H, Hkv, HD, dtype, bt, window=window, ring=self.rb)
-            self.ring_region = n_slots * self.rb * 2 * bt * self.ap.kv_ld
+            Hkv_s, HD_s = sliding or (Hkv, HD)
+            self.ap_s = synth.make_params(H, Hkv_s, HD_s, dtype, bt, window=window, ring=self.rb)
+            self.ring_region = n_slots * self.rb * 2 * bt * self.ap_s.kv_ld
+            empty_s = np.zeros((0, self.ap_s.kv_ld), np.uint16)
+            self.truth_s = {s: (empty_s, empty_s) for s in self.slots}   # the sliding layer has K / V rows of its own
             self.ring_ref = np.zeros(self.ring_region, np.uint16)
             self.ring = torch.zeros(self.ring_region, dtype=torch.int16, device="cuda")
 
@@ -52,12 +56,15 @@ class Served:
     def reset(self, s):
         self.e.slot_reset(s)
         self.truth[s] = (self.truth[s][0][:0], self.truth[s][1][:0])
+        if self.W:
+            self.truth_s[s] = (self.truth_s[s][0][:0], self.truth_s[s][1][:0])
 
     def fork(self, a, b):
         self.reset(b)
         self.e.slot_fork(a, b)
         self.truth[b] = self.truth[a]
         if self.W:                                                 # a fork copies the whole ring (forest.h:127-137)
+            self.truth_s[b] = self.truth_s[a]
             self.ring_copy([(a * self.rb + i, b * self.rb + i) for i in range(self.rb)])
 
     def run(self, specs, rows_per_tile, commit=True, tag=""):
@@ -103,15 +110,17 @@ class Served:
             resident, groups = device.plan_hint(aps)
             tiles, jobs, n_parts = host.plan_tiles(rg["trees"], groups, self.W, ps["pos"], host.options_mi355x(rows_per_tile, resident))
             dps = device.DevicePass(aps, rg["trees"], tiles, jobs, n_parts, M, np.zeros(1, np.int32), ps["desc"], ps["pos"])
-            Os = torch.zeros_like(Qd)
-            dps.run(Qd, Kd, Vd, self.ring, Os)
+            Qs, Kbs, Vbs = bits(aps.q_ld), bits(aps.kv_ld), bits(aps.kv_ld)
+            Qsd, Ksd, Vsd = dev_u16(Qs), dev_u16(Kbs), dev_u16(Vbs)
+            Os = torch.zeros_like(Qsd)
+            dps.run(Qsd, Ksd, Vsd, self.ring, Os)
             torch.cuda.synchronize()
-            want = ob.attn_direct(aps, Q, Kb, Vb, self.ring_ref, np.zeros(1, np.int32), ps["desc"], ps["pos"], rg["trees"], n_threads=8)
+            want = ob.attn_direct(aps, Qs, Kbs, Vbs, self.ring_ref, np.zeros(1, np.int32), ps["desc"], ps["pos"], rg["trees"], n_threads=8)
             err = float(np.abs(f32(to_host_u16(Os).reshape(M, -1), dtype) - f32(want, dtype)).max())
             assert err <= self.tol, (tag, "sliding", err)
             if commit and len(rg["saves"]):
-                device.kv_save(aps, Kd, Vd, self.ring, device.to_dev(rg["saves"]), len(rg["saves"]))
-                ob.kv_save(aps, Kb, Vb, self.ring_ref, rg["saves"])
+                device.kv_save(aps, Ksd, Vsd, self.ring, device.to_dev(rg["saves"]), len(rg["saves"]))
+                ob.kv_save(aps, Kbs, Vbs, self.ring_ref, rg["saves"])
         if not commit:
             e.pass_abort()     # the copied blocks go back to the free list; nothing a slot lists has changed
             self.check_slots(tag)
@@ -121,13 +130,18 @@ class Served:
             ob.kv_save(ap, Kb, Vb, self.pool_ref, ps["saves"])
         torch.cuda.synchronize()
         e.pass_commit()
-        new = {}
+        new, new_s = {}, {}
         for t, (parent, save, root_len, *_) in zip(ps["trees"], specs):
             if save >= 0:                                          # the slot takes its parent's rows and the tree's root
                 pk, pv = self.truth[parent] if parent >= 0 else (Kb[:0], Vb[:0])
                 b = int(t["base"])
                 new[save] = (np.concatenate([pk, Kb[b:b + root_len]]), np.concatenate([pv, Vb[b:b + root_len]]))
+                if self.W:
+                    pk, pv = self.truth_s[parent] if parent >= 0 else (Kbs[:0], Vbs[:0])
+                    new_s[save] = (np.concatenate([pk, Kbs[b:b + root_len]]), np.concatenate([pv, Vbs[b:b + root_len]]))
         self.truth.update(new)
+        if self.W:
+            self.truth_s.update(new_s)
         self.last = (ps, specs, Kb, Vb)
         self.check_slots(tag)
         return True
@@ -154,7 +168,7 @@ class Served:
                 lo = max(0, n - self.W + 1)
                 order = [s * self.rb + i % self.rb for i in range((n + self.ap.bt - 1) // self.ap.bt)]
                 kw, vw = ob.kv_gather(self.ap_s, self.ring_ref, np.array(order, np.int32), n)
-                assert np.array_equal(kw[lo:], self.truth[s][0][lo:]) and np.array_equal(vw[lo:], self.truth[s][1][lo:]), (tag, s, "ring")
+                assert np.array_equal(kw[lo:], self.truth_s[s][0][lo:]) and np.array_equal(vw[lo:], self.truth_s[s][1][lo:]), (tag, s, "ring")
 
     def finish(self):
         """The device pool holds what the reference-layout pool holds, block for block, and every slot reads back
@@ -181,9 +195,13 @@ class Served:
             assert np.array_equal(to_host_u16(Vg).reshape(n, -1), self.truth[s][1])
 
 
-@pytest.mark.parametrize("H,Hkv,HD,bt,dtype", [(8, 2, 128, 16, abi.ESP_F16), (8, 1, 512, 32, abi.ESP_F16), (6, 3, 256, 64, abi.ESP_BF16)])
-def test_engine_records_drive_the_kernels_through_a_serving_history(H, Hkv, HD, bt, dtype):
-    sv = Served(H, Hkv, HD, bt, dtype, 96, 4, H + HD, window={128: 0, 256: 100, 512: 0}[HD])
+# the last: Gemma 4's two layer kinds off the same records - full layers of 512-dim heads on few KV heads, sliding layers
+# of 256-dim heads on more (gemma.h:126-150)
+@pytest.mark.parametrize("H,Hkv,HD,bt,dtype,window,sliding", [(8, 2, 128, 16, abi.ESP_F16, 0, None), (8, 1, 512, 32, abi.ESP_F16, 0, None),
+                                                              (6, 3, 256, 64, abi.ESP_BF16, 100, None),
+                                                              (16, 2, 512, 16, abi.ESP_F16, 72, (8, 256))])
+def test_engine_records_drive_the_kernels_through_a_serving_history(H, Hkv, HD, bt, dtype, window, sliding):
+    sv = Served(H, Hkv, HD, bt, dtype, 96, 4, H + HD, window=window, sliding=sliding)
     A, B, Cc, D = sv.slots
     e = sv.e
     G = H // Hkv
