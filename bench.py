@@ -532,12 +532,338 @@ def graph_replay(w, torch, steps=16, replays=8):
         return {"error": str(e).splitlines()[0][:200]}
 
 
+def spot_check(w, rows=4, threads=8):
+    """Parity of what the timed steps left in O, on a sample: the last `rows` rows of the workload's first and
+    last sequence (whole trees when they carry a verify descriptor), against the CPU checker. The rows before
+    them in the same pass count as cached keys, which the attention's semantics make equivalent
+    (kernels/40_attention.metal:245-249: a batch key and the same key in the cache score alike). Returns
+    (max abs error, rows checked)."""
+    import torch
+    from espetero_amd import abi, device, synth
+    from oracle import binding as ob
+    p = w.params
+    kvw, bt = p.Hkv * p.head_dim, p.bt
+    bits = lambda t: t.contiguous().view(torch.int16).cpu().numpy().view(np.uint16)  # noqa: E731
+    w.step(0)   # rotation set 0's block tables are the ones gathered below
+    torch.cuda.synchronize()
+    worst, checked = 0.0, 0
+    plain = not np.any(w.desc)
+    for i in sorted({0, len(w.seqs) - 1}):
+        P, M = w.seqs[i]
+        t = w.trees[i]
+        b0 = int(t["base"])
+        r = min(rows, M) if plain else M
+        Pc = P + M - r                       # cached keys as the sampled rows see them
+        nb = (Pc + bt - 1) // bt
+        pool_ref = np.zeros((nb + 1) * 2 * bt * kvw, np.uint16)
+        pv = pool_ref.reshape(nb + 1, 2, bt, kvw)
+        Kh, Vh = np.zeros((nb * bt, kvw), np.uint16), np.zeros((nb * bt, kvw), np.uint16)
+        if P:
+            K = torch.zeros(P * kvw, dtype=torch.int16, device="cuda")
+            V = torch.zeros_like(K)
+            device.kv_gather(p, w.pool, w.passes[0].blocks[int(t["table"]):], P, K, V)
+            torch.cuda.synchronize()
+            Kh[:P], Vh[:P] = bits(K).reshape(P, kvw), bits(V).reshape(P, kvw)
+        if M > r:
+            Kh[P:Pc] = bits(w.Kb[b0:b0 + M - r])[:, :kvw]
+            Vh[P:Pc] = bits(w.Vb[b0:b0 + M - r])[:, :kvw]
+        if nb:
+            pv[:nb, 0], pv[:nb, 1] = Kh.reshape(nb, bt, kvw), Vh.reshape(nb, bt, kvw)
+        sl = slice(b0 + M - r, b0 + M)
+        pos = np.zeros((r, 4), np.int32)
+        pos[:, :3] = (Pc + np.arange(r))[:, None]
+        desc = np.zeros((r, 4), np.int32) if plain else w.desc[sl]
+        pr = synth.make_params(p.H, p.Hkv, p.head_dim, p.dtype, bt, window=p.window, rows_per_tile=p.rows_per_tile)
+        want = ob.attn_direct(pr, bits(w.Q[sl]), bits(w.Kb[sl]), bits(w.Vb[sl]), pool_ref, np.arange(max(nb, 1), dtype=np.int32),
+                              desc, pos, np.array([(0, Pc, 0, r)], abi.TREE_DT), n_threads=threads)
+        got = bits(w.O[sl])
+        worst = max(worst, float(np.abs(ob.to_f32(got, p.dtype).astype(np.float64) - ob.to_f32(want, p.dtype)).max()))
+        checked += r
+    return worst, checked
+
+
+def tolerance(dtype):
+    """Max-abs bar of the path against the CPU checker's storage-type output: 2e-3. Both sides round their output
+    to the storage type; on bf16 one unit in the last place of an output below 1 is up to 2^-8, so a result that
+    rounds the other way is allowed on top."""
+    from espetero_amd import abi
+    return 2e-3 if dtype == abi.ESP_F16 else 2e-3 + 2.0 ** -8
+
+
+def timed_run(w, torch, steps, warmup):
+    """warmup untimed steps, then `steps` timed ones between two device synchronisations. The dominant kernel's
+    own begin and end are taken by HIP events handed to its launch (esp_attn_time_next; events recorded between
+    the kernels instead cost the stream about as much as the split-K merge and read microseconds long): on
+    every step when there are at most 50, else on every fourth. Returns wall seconds per step and the per-step
+    kernel milliseconds (all launches of the dominant kernel in a step, each launch's own list beside)."""
+    for i in range(warmup):
+        w.step(i)
+    torch.cuda.synchronize()
+    every = 1 if steps <= 50 else 4
+    nev = getattr(w, "launches_per_step", 1)
+    evs = [[(torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)) for _ in range(nev)]
+           for _ in range(0, steps, every)]
+    for pairs in evs:  # a first record creates the HIP events behind the torch objects
+        for a, b in pairs:
+            a.record()
+            b.record()
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    for i in range(steps):
+        ev = evs[i // every] if i % every == 0 else None
+        w.step(warmup + i, (ev[0] if nev == 1 else ev) if ev else None)
+    torch.cuda.synchronize()
+    wall = (time.perf_counter() - t0) / steps
+    per_launch = np.array([[a.elapsed_time(b) for a, b in pairs] for pairs in evs])  # [samples][launches] ms
+    return wall, per_launch
+
+
+def kernel_name(w):
+    return getattr(w, "kernel", None) or ("attn_stream_kernel" if w.params.rows_per_tile * (w.H // w.Hkv) <= 32
+                                          else "attn_tiled512_kernel" if w.HD == 512 else "attn_tiled_kernel")
+
+
+def roofline(w, per_step_ms, ceilings=None):
+    """achieved = algorithmic bytes (flops) of the pass / the dominant kernel's mean duration per step."""
+    mean, med, mn = float(np.mean(per_step_ms)), float(np.median(per_step_ms)), float(np.min(per_step_ms))
+    if w.bound == "hbm":
+        work, peak, unit, scale = w.alg_bytes, HBM_PEAK_GBS, "GB/s", 1e9
+    else:
+        work, peak, unit, scale = w.alg_flops, MFMA_PEAK_TFLOPS, "TFLOP/s", 1e12
+    achieved = work / (mean * 1e-3) / scale
+    r = {"bound": w.bound, "achieved": round(achieved, 3), "peak": peak, "unit": unit, "frac": round(achieved / peak, 4),
+         "traffic": measured_traffic(w.name), "kernel": kernel_name(w), "kernel_us_avg": round(mean * 1e3, 3),
+         "kernel_us_median": round(med * 1e3, 3), "kernel_us_min": round(mn * 1e3, 3), "samples": int(len(per_step_ms)),
+         "alg_bytes": int(w.alg_bytes), "alg_flops": int(w.alg_flops)}
+    if ceilings:
+        c = ceilings.get("hbm_read_GBs" if w.bound == "hbm" else "mfma_TFLOPs")
+        if c:
+            r["measured_ceiling"] = c
+            r["frac_of_measured_ceiling"] = round(achieved / c, 4)
+    return r
+
+
+def headline(w, wall, per_launch, steps, warmup, ceilings=None):
+    from espetero_amd import abi
+    per_step = per_launch.sum(axis=1)
+    if w.bound == "hbm":
+        metric = ("attn-prep HBM GB/s" if isinstance(w, PrepWorkload) else
+                  "head-gate HBM GB/s" if isinstance(w, GateWorkload) else "decode-attn HBM GB/s")
+        unit, value = "GB/s", w.alg_bytes / wall / 1e9
+    else:
+        metric, unit, value = "prefill-attn TFLOPS", "TFLOP/s", w.alg_flops / wall / 1e12
+    return {
+        "metric": metric, "value": round(value, 3), "unit": unit, "n_gpus": 1, "steps": steps, "warmup": warmup,
+        "ms_per_step": round(wall * 1e3, 6), "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
+        "dtype": "f16" if w.dtype == abi.ESP_F16 else "bf16", "data": "synthetic",
+        "config": {"workload": w.name, "sequences": len(w.seqs), "rows": w.n_rows, "H": w.H, "Hkv": w.Hkv,
+                   "head_dim": w.HD, "page": w.bt, "window": w.window, "context_tokens": int(sum(P for P, _ in w.seqs)),
+                   "tiles": int(len(w.tiles)), "parts": int(w.n_parts), "rotation_sets": w.n_sets,
+                   "pool_pages": w.pool_pages},
+        "roofline": roofline(w, per_step, ceilings),
+    }
+
+
+def cpu_leg(w, torch, budget_s=20.0):
+    w.step(0)   # leave rotation set 0's output in O: the CPU sample is checked against it
+    torch.cuda.synchronize()
+    if isinstance(w, PrepWorkload):
+        return prep_cpu_baseline(w)
+    if isinstance(w, GateWorkload):
+        return gate_cpu_baseline(w)
+    if isinstance(w, ChunkedPrefill):
+        return chunked_cpu_baseline(w)
+    if isinstance(w, LayerMix):
+        return cpu_baseline(w.full, budget_s)   # the full-attention layer of the mix
+    return cpu_baseline(w, budget_s)
+
+
+def compact(w, torch, steps, warmup, ceilings):
+    """One short record of a benchmark configuration: step time, the dominant kernel's duration and roofline
+    fraction, and a parity spot check of the output the timed steps left behind."""
+    from espetero_amd import abi
+    wall, per_launch = timed_run(w, torch, steps, warmup)
+    per_step = per_launch.sum(axis=1)
+    r = roofline(w, per_step, ceilings)
+    rec = {"workload": w.name, "bound": w.bound, "steps": steps, "ms_per_step": round(wall * 1e3, 6),
+           "value": round((w.alg_bytes / 1e9 if w.bound == "hbm" else w.alg_flops / 1e12) / wall, 3), "unit": r["unit"],
+           "kernel": r["kernel"], "kernel_us_median": r["kernel_us_median"], "kernel_us_min": r["kernel_us_min"],
+           "kernel_us_avg": r["kernel_us_avg"], "achieved": r["achieved"], "frac": r["frac"],
+           "dtype": "f16" if w.dtype == abi.ESP_F16 else "bf16", "tolerance": tolerance(w.dtype)}
+    if "frac_of_measured_ceiling" in r:
+        rec["frac_of_measured_ceiling"] = r["frac_of_measured_ceiling"]
+    return rec, per_launch
+
+
+def part_record(name, work, unit_scale, peak, ms):
+    """A launch of a multi-launch step on its own (a chunk of the chunked prefill, a layer kind of the mix)."""
+    mean = float(np.mean(ms))
+    ach = work / (mean * 1e-3) / unit_scale
+    return {"part": name, "kernel_us_median": round(float(np.median(ms)) * 1e3, 3), "kernel_us_min": round(float(np.min(ms)) * 1e3, 3),
+            "kernel_us_avg": round(mean * 1e3, 3), "achieved": round(ach, 3), "frac": round(ach / peak, 4)}
+
+
+class Ceilings:
+    """The machine's own ceilings, measured in this run by libespetero_ceilings.so: a plain non-temporal
+    16-byte-per-lane read of scattered 8 KB pages (and of the same bytes in address order), and the matrix cores
+    under a wavefront that issues the prefill kernel's share of vector arithmetic beside them."""
+
+    def __init__(self):
+        import ctypes as C
+        import torch
+        self.torch, self.C = torch, C
+        path = os.path.join(ROOT, "espetero_amd", "csrc", "libespetero_ceilings.so")
+        if not os.path.exists(path):
+            raise SystemExit(f"{path} is not built (run __graft_entry__.build())")
+        self.lib = C.CDLL(path)
+        V, I = C.c_void_p, C.c_int32
+        self.lib.esp_ceiling_hbm_read.argtypes = [V, V, I, I, I, I, V, V, V, V]
+        self.lib.esp_ceiling_mfma_issue.argtypes = [I, I, I, I, V, V, V, V]
+
+    def _events(self, n):
+        t = self.torch
+        evs = [(t.cuda.Event(enable_timing=True), t.cuda.Event(enable_timing=True)) for _ in range(n)]
+        for a, b in evs:
+            a.record()
+            b.record()
+        t.cuda.synchronize()
+        return evs
+
+    def hbm_read(self, mbytes=(141, 537, 1074), page_bytes=8192, reps=12, workgroups=2 * N_CU):
+        """GB/s of the plain read at each size: scattered pages (a seeded permutation of a 4 GiB buffer) and
+        address order, non-temporal and ordinary loads. Each repetition reads other pages than the one before."""
+        t = self.torch
+        total = 4 << 30
+        buf = t.empty(total, dtype=t.uint8, device="cuda")
+        buf.fill_(1)
+        sink = t.zeros(4, dtype=t.int32, device="cuda")
+        n_all = total // page_bytes
+        perm = t.from_numpy(np.random.default_rng(11).permutation(n_all).astype(np.int32)).cuda()
+        st = self.C.c_void_p(t.cuda.current_stream().cuda_stream)
+        out = []
+        for mb in mbytes:
+            n_pages = mb * 1000000 // page_bytes
+            rec = {"bytes": n_pages * page_bytes, "page_bytes": page_bytes, "workgroups": workgroups}
+            for label, scattered, nt in (("scattered_nt", True, 1), ("scattered", True, 0), ("contiguous_nt", False, 1)):
+                evs = self._events(reps)
+                for k, (a, b) in enumerate(evs):
+                    off = (k * n_pages) % (n_all - n_pages)
+                    pages = self.C.c_void_p(perm.data_ptr() + 4 * off) if scattered else None
+                    base = self.C.c_void_p(buf.data_ptr() + (0 if scattered else off * page_bytes))
+                    rc = self.lib.esp_ceiling_hbm_read(base, pages, n_pages, page_bytes, nt, workgroups,
+                                                       self.C.c_void_p(sink.data_ptr()), st, self.C.c_void_p(a.cuda_event),
+                                                       self.C.c_void_p(b.cuda_event))
+                    assert rc == 0, rc
+                t.cuda.synchronize()
+                ms = np.array([a.elapsed_time(b) for a, b in evs][2:])
+                rec[label] = {"GBs_median": round(rec["bytes"] / float(np.median(ms)) / 1e6, 1),
+                              "GBs_best": round(rec["bytes"] / float(ms.min()) / 1e6, 1), "us_median": round(float(np.median(ms)) * 1e3, 2)}
+            out.append(rec)
+        del buf, perm
+        t.cuda.empty_cache()
+        return out
+
+    def mfma_issue(self, mixes=((0, 0), (2, 0), (4, 0), (0, 1), (1, 1), (2, 1), (3, 1), (4, 1)), iters=2000, workgroups=2 * N_CU):
+        """TFLOP/s of v_mfma_f32_32x32x16_bf16 at two wavefronts per SIMD with (fp32 FMAs, v_exp_f32 + add) per
+        matrix instruction issued beside it; (0, 0) is the matrix cores alone, i.e. the clock they sustain."""
+        t = self.torch
+        outbuf = t.zeros(workgroups * 256, dtype=t.float32, device="cuda")
+        st = self.C.c_void_p(t.cuda.current_stream().cuda_stream)
+        flops = workgroups * 4 * iters * 32 * 32768
+        out = []
+        for nv, ne in mixes:
+            evs = self._events(5)
+            for a, b in evs:
+                rc = self.lib.esp_ceiling_mfma_issue(nv, ne, workgroups, iters, self.C.c_void_p(outbuf.data_ptr()), st,
+                                                     self.C.c_void_p(a.cuda_event), self.C.c_void_p(b.cuda_event))
+                assert rc == 0, rc
+            t.cuda.synchronize()
+            ms = np.array([a.elapsed_time(b) for a, b in evs][1:])
+            out.append({"valu_per_mfma": nv, "exp_per_mfma": ne, "TFLOPs": round(flops / float(np.median(ms)) / 1e9, 1),
+                        "cycles_per_mfma_at_2.4GHz": round(float(np.median(ms)) * 1e-3 * 2.4e9 / (iters * 32 * 2), 2)})
+        return out
+
+
+def run_all(args, torch):
+    """The default run: the batched paged decode as the headline (its K timed steps are the line's steps), the
+    chunked causal prefill as the other half of the metric, one short record per benchmark configuration, and
+    the machine's measured ceilings."""
+    K, W = args.steps, args.warmup
+    ceil = Ceilings()
+    reads = ceil.hbm_read()
+    issue = ceil.mfma_issue()
+    # what the fractions are also stated against: the plain read at the headline's size, the matrix cores alone
+    cz = {"hbm_read_GBs": reads[0]["scattered_nt"]["GBs_median"], "mfma_TFLOPs": issue[0]["TFLOPs"]}
+    w = make_workload("c2_batched_decode", args.workgroups or None, args.tables == "contiguous", args.page)
+    wall, per_launch = timed_run(w, torch, K, W)
+    out = headline(w, wall, per_launch, K, W, cz)
+    out["graph_replay"] = graph_replay(w, torch)
+    err, n = spot_check(w)
+    c2 = {"workload": w.name, "ms_per_step": out["ms_per_step"], "kernel_us_median": out["roofline"]["kernel_us_median"],
+          "kernel_us_min": out["roofline"]["kernel_us_min"], "frac": out["roofline"]["frac"], "max_abs_err_vs_cpu": err,
+          "rows_checked": n, "tolerance": tolerance(w.dtype)}
+    if not args.no_cpu:
+        out["cpu_baseline"] = cpu_leg(w, torch)
+    del w
+    torch.cuda.empty_cache()
+
+    # ---- the prefill half of the metric: config 3 whole (4 x (attention, merge, append)), chunk by chunk beside it
+    steps_p = max(5, min(20, K // 10))
+    w = make_workload("c3_chunked_prefill", args.workgroups or None, False, args.page)
+    rec, pl = compact(w, torch, steps_p, 3, cz)
+    chunk = w.n_rows // pl.shape[1]
+    parts = []
+    for c in range(pl.shape[1]):
+        pairs = chunk * c * chunk + chunk * (chunk + 1) // 2
+        parts.append(part_record(f"chunk P={c * chunk}", 4 * w.HD * w.H * pairs, 1e12, MFMA_PEAK_TFLOPS, pl[:, c]))
+    pre = {"metric": "prefill-attn TFLOPS", "value": rec["value"], "unit": "TFLOP/s", "ms_per_step": rec["ms_per_step"],
+           "steps": steps_p, "dtype": "bf16", "config": {"workload": w.name, "rows": w.n_rows, "chunk": chunk, "H": w.H, "Hkv": w.Hkv,
+                                                        "head_dim": w.HD, "page": w.bt},
+           "roofline": roofline(w, pl.sum(axis=1), cz), "chunks": parts, "tolerance": tolerance(w.dtype)}
+    if not args.no_cpu:
+        w.step(0)
+        torch.cuda.synchronize()
+        pre["cpu_baseline"] = chunked_cpu_baseline(w)
+        pre["max_abs_err_vs_cpu"] = pre["cpu_baseline"]["max_abs_err_vs_gpu"]
+    out["prefill"] = pre
+    del w
+    torch.cuda.empty_cache()
+
+    # ---- one record per benchmark configuration
+    configs = [c2]
+    for name, steps in (("c1_single_decode", 50), ("c5_verify", 30), ("c4_decode_mix", 20), ("c4_prefill_mix", 5)):
+        w = make_workload(name, args.workgroups or None, False, args.page)
+        rec, pl = compact(w, torch, steps, 3, cz)
+        if isinstance(w, LayerMix):
+            hb = w.bound == "hbm"
+            peak, sc = (HBM_PEAK_GBS, 1e9) if hb else (MFMA_PEAK_TFLOPS, 1e12)
+            rec["layers"] = [
+                part_record("sliding layer (each of 5)", w.sliding.alg_bytes if hb else w.sliding.alg_flops, sc, peak, pl[:, :5].reshape(-1)),
+                part_record("global layer", w.full.alg_bytes if hb else w.full.alg_flops, sc, peak, pl[:, 5])]
+            e1, n1 = spot_check(w.sliding)
+            e2, n2 = spot_check(w.full)
+            rec["max_abs_err_vs_cpu"], rec["rows_checked"] = max(e1, e2), n1 + n2
+        else:
+            rec["max_abs_err_vs_cpu"], rec["rows_checked"] = spot_check(w)
+        configs.append(rec)
+        del w
+        torch.cuda.empty_cache()
+    configs.insert(2, {"workload": "c3_chunked_prefill", "ms_per_step": pre["ms_per_step"], "frac": pre["roofline"]["frac"],
+                       "kernel_us_median": pre["roofline"]["kernel_us_median"], "kernel_us_min": pre["roofline"]["kernel_us_min"],
+                       "max_abs_err_vs_cpu": pre.get("max_abs_err_vs_cpu"), "tolerance": pre["tolerance"], "see": "prefill"})
+    out["configs"] = configs
+    out["ceilings"] = {"hbm_read": reads, "mfma_issue": issue}
+    print(json.dumps(out), flush=True)
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
     ap.add_argument("--steps", type=int, default=200)
     ap.add_argument("--warmup", type=int, default=20)
-    ap.add_argument("--workload", default="c2_batched_decode", help="one of: " + ", ".join(WORKLOADS))
+    ap.add_argument("--workload", default="all",
+                    help="all (default): the batched decode as the headline, the chunked prefill, one record per benchmark "
+                         "configuration and the measured ceilings; or one of: hbm_read_ceiling, mfma_issue_ceiling, " + ", ".join(WORKLOADS))
     ap.add_argument("--workgroups", type=int, default=0, help="planner split target (0: ask esp_attn_plan_hint)")
     ap.add_argument("--tables", default="scattered", choices=["scattered", "contiguous"],
                     help="block tables: a seeded permutation of the pool (the benchmark's definition) or address order")
@@ -550,10 +876,9 @@ def main():
         raise SystemExit("bench.py measures one GPU: this path has no multi-GPU leg (run with --gpus 1)")
 
     import torch
-    from espetero_amd import abi, device
+    from espetero_amd import device
     assert torch.cuda.is_available(), "bench.py needs a GPU"
     device.init(0)
-    w = make_workload(args.workload, args.workgroups or None, args.tables == "contiguous", args.page)
     if args.copy_calibration:
         src = torch.ones(256 << 20, dtype=torch.uint8, device="cuda")
         dst = torch.empty_like(src)
@@ -561,72 +886,24 @@ def main():
             dst.copy_(src)   # a plain copy kernel of known size: reads 256 MiB, writes 256 MiB
         torch.cuda.synchronize()
         del src, dst
+    if args.workload == "all":
+        return run_all(args, torch)
+    if args.workload == "hbm_read_ceiling":
+        print(json.dumps({"metric": "plain read GB/s", "unit": "GB/s", "peak": HBM_PEAK_GBS, "sizes": Ceilings().hbm_read()}), flush=True)
+        return
+    if args.workload == "mfma_issue_ceiling":
+        print(json.dumps({"metric": "matrix cores under vector issue, TFLOP/s", "unit": "TFLOP/s", "peak": MFMA_PEAK_TFLOPS,
+                          "mixes": Ceilings().mfma_issue()}), flush=True)
+        return
+    w = make_workload(args.workload, args.workgroups or None, args.tables == "contiguous", args.page)
     K, W = args.steps, args.warmup
-    for i in range(W):
-        w.step(i)
-    torch.cuda.synchronize()
-    # HIP events take the dominant kernel's own begin and end on every EVERY-th step of the timed
-    # region, handed to the kernel's launch through esp_attn_time_next (events recorded between the
-    # kernels instead cost the stream about as much as the split-K merge and read microseconds long).
-    EVERY = 4
-    NEV = getattr(w, "launches_per_step", 1)  # launches of the dominant kernel in one step: one event pair each
-    evs = [[(torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)) for _ in range(NEV)]
-           for _ in range(0, K, EVERY)]
-    for pairs in evs:  # a first record creates the HIP events behind the torch objects
-        for a, b in pairs:
-            a.record()
-            b.record()
-    torch.cuda.synchronize()
-    t0 = time.perf_counter()
-    for i in range(K):
-        ev = evs[i // EVERY] if i % EVERY == 0 else None
-        w.step(W + i, (ev[0] if NEV == 1 else ev) if ev else None)
-    torch.cuda.synchronize()
-    wall = (time.perf_counter() - t0) / K
-    per_step = [sum(a.elapsed_time(b) for a, b in pairs) for pairs in evs]  # all launches of the step together
-    kern_ms = float(np.mean(per_step))
-    kern_min_ms = float(np.min(per_step))
-
-    if w.bound == "hbm":
-        metric = ("attn-prep HBM GB/s" if isinstance(w, PrepWorkload) else
-                  "head-gate HBM GB/s" if isinstance(w, GateWorkload) else "decode-attn HBM GB/s")
-        unit = "GB/s"
-        value = w.alg_bytes / wall / 1e9
-        achieved, peak = w.alg_bytes / (kern_ms * 1e-3) / 1e9, HBM_PEAK_GBS
-    else:
-        metric, unit = "prefill-attn TFLOPS", "TFLOP/s"
-        value = w.alg_flops / wall / 1e12
-        achieved, peak = w.alg_flops / (kern_ms * 1e-3) / 1e12, MFMA_PEAK_TFLOPS
-    out = {
-        "metric": metric, "value": round(value, 3), "unit": unit, "n_gpus": 1, "steps": K, "warmup": W,
-        "ms_per_step": round(wall * 1e3, 6), "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
-        "dtype": "f16" if w.dtype == abi.ESP_F16 else "bf16", "data": "synthetic",
-        "config": {"workload": w.name, "sequences": len(w.seqs), "rows": w.n_rows, "H": w.H, "Hkv": w.Hkv,
-                   "head_dim": w.HD, "page": w.bt, "window": w.window, "context_tokens": int(sum(P for P, _ in w.seqs)),
-                   "tiles": int(len(w.tiles)), "parts": int(w.n_parts), "rotation_sets": w.n_sets,
-                   "pool_pages": w.pool_pages},
-        "roofline": {"bound": w.bound, "achieved": round(achieved, 3), "peak": peak, "unit": unit,
-                     "frac": round(achieved / peak, 4), "traffic": measured_traffic(w.name),
-                     "kernel": getattr(w, "kernel", None) or (
-                         "attn_stream_kernel" if w.bound == "hbm" and w.params.rows_per_tile * (w.H // w.Hkv) <= 32
-                         else "attn_tiled_kernel"),
-                     "kernel_us_avg": round(kern_ms * 1e3, 3), "kernel_us_min": round(kern_min_ms * 1e3, 3),
-                     "alg_bytes": int(w.alg_bytes), "alg_flops": int(w.alg_flops)},
-    }
+    wall, per_launch = timed_run(w, torch, K, W)
+    out = headline(w, wall, per_launch, K, W)
+    if per_launch.shape[1] > 1:
+        out["roofline"]["per_launch_us_median"] = [round(float(x) * 1e3, 3) for x in np.median(per_launch, axis=0)]
     out["graph_replay"] = graph_replay(w, torch)
     if not args.no_cpu:
-        w.step(0)   # leave rotation set 0's output in O: the CPU sample is checked against it
-        torch.cuda.synchronize()
-        if isinstance(w, PrepWorkload):
-            out["cpu_baseline"] = prep_cpu_baseline(w)
-        elif isinstance(w, GateWorkload):
-            out["cpu_baseline"] = gate_cpu_baseline(w)
-        elif isinstance(w, ChunkedPrefill):
-            out["cpu_baseline"] = chunked_cpu_baseline(w)
-        elif isinstance(w, LayerMix):
-            out["cpu_baseline"] = cpu_baseline(w.full)   # the full-attention layer of the mix
-        else:
-            out["cpu_baseline"] = cpu_baseline(w)
+        out["cpu_baseline"] = cpu_leg(w, torch)
     print(json.dumps(out), flush=True)
 
 

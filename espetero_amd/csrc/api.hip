@@ -3,6 +3,8 @@
 #include <cstdarg>
 #include <cstdio>
 #include <cstring>
+#include <mutex>
+#include <vector>
 
 #include "common.hpp"
 
@@ -26,6 +28,9 @@ hipError_t launch_head_gate(int dt, const GateArgs& a, hipStream_t st);
 int stream_workgroups_per_cu(int HD, int NC);
 int tiled_workgroups_per_cu(int HD);
 int tiled_max_rows(int HD);
+hipError_t stream_init_attributes();
+hipError_t tiled_init_attributes();
+hipError_t tiled512_init_attributes();
 }  // namespace esp
 
 namespace {
@@ -114,6 +119,32 @@ esp::KArgs make_args(const esp_attn_params* p, const Carve& c, void* workspace, 
   return a;
 }
 
+constexpr int kMaxDevices = 64;
+struct DeviceState {
+  bool ready = false;
+};
+DeviceState g_dev[kMaxDevices];
+std::mutex g_dev_mutex;
+
+// State of the current device; the first call on a device raises the kernels' dynamic LDS limits (a
+// process-wide fact of that device, not stream work).
+int device_state(DeviceState** out, char* err, size_t errlen) {
+  int dev = 0;
+  hipError_t e = hipGetDevice(&dev);
+  if (e != hipSuccess) return hip_fail(err, errlen, "hipGetDevice", e);
+  if (dev < 0 || dev >= kMaxDevices) return fail(err, errlen, ESP_EUNSUPPORTED, "device ordinal %d (at most %d devices)", dev, kMaxDevices);
+  std::lock_guard<std::mutex> lock(g_dev_mutex);
+  DeviceState& d = g_dev[dev];
+  if (!d.ready) {
+    if ((e = esp::stream_init_attributes()) != hipSuccess) return hip_fail(err, errlen, "hipFuncSetAttribute (streaming kernels)", e);
+    if ((e = esp::tiled_init_attributes()) != hipSuccess) return hip_fail(err, errlen, "hipFuncSetAttribute (tiled kernels)", e);
+    if ((e = esp::tiled512_init_attributes()) != hipSuccess) return hip_fail(err, errlen, "hipFuncSetAttribute (tiled kernels, head dim 512)", e);
+    d.ready = true;
+  }
+  *out = &d;
+  return ESP_OK;
+}
+
 }  // namespace
 
 namespace esp {
@@ -135,7 +166,15 @@ int esp_attn_init(int device, char* err, size_t errlen) {
   if (e != hipSuccess) return hip_fail(err, errlen, "hipGetDeviceProperties", e);
   if (strncmp(prop.gcnArchName, "gfx950", 6) != 0)
     return fail(err, errlen, ESP_EUNSUPPORTED, "device %d is %s; this library is built for gfx950 only", device, prop.gcnArchName);
-  return ESP_OK;
+  // Per-device set-up with that device current: the addresses of the library's own device arrays and
+  // the kernels' LDS limits, so that no later call has anything but launches left to do.
+  int prev = 0;
+  if ((e = hipGetDevice(&prev)) != hipSuccess) return hip_fail(err, errlen, "hipGetDevice", e);
+  if (prev != device && (e = hipSetDevice(device)) != hipSuccess) return hip_fail(err, errlen, "hipSetDevice", e);
+  DeviceState* d = nullptr;
+  const int rc = device_state(&d, err, errlen);
+  if (prev != device) (void)hipSetDevice(prev);
+  return rc;
 }
 
 int esp_attn_plan_hint(const esp_attn_params* p, int device, int32_t* workgroups, int32_t* groups_per_tile,
@@ -163,15 +202,21 @@ size_t esp_attn_workspace_bytes(const esp_attn_params* p, int32_t n_rows, int32_
   return carve(p, n_rows, n_parts).total;
 }
 
-int esp_attn_forward(const esp_attn_params* p, const void* Q, const void* Kb, const void* Vb, const void* kv_pool,
-                     const int32_t* blocks, const int32_t* desc, const int32_t* pos, void* O, const esp_tile* tiles,
-                     int32_t n_tiles, const esp_tree* trees, int32_t n_trees, const esp_combine* jobs, int32_t n_jobs,
-                     int32_t n_parts, int32_t n_rows, void* workspace, size_t workspace_bytes, void* stream, char* err,
-                     size_t errlen) {
+static int forward_impl(const esp_attn_params* p, const void* Q, const void* Kb, const void* Vb, const void* kv_pool,
+                        const int32_t* blocks, const int32_t* desc, const int32_t* pos, void* O, const esp_tile* tiles,
+                        int32_t n_tiles, const esp_tree* trees, int32_t n_trees, const esp_combine* jobs, int32_t n_jobs,
+                        int32_t n_parts, int32_t n_rows, void* workspace, size_t workspace_bytes, void* stream, char* err,
+                        size_t errlen) {
+  // A pending event pair belongs to this call whatever becomes of it: a call that launches nothing
+  // must not leave it armed for some later launch.
+  struct DropPair {
+    ~DropPair() { (void)esp::take_time_next(); }
+  } drop_pair;
   if (int rc = check_params(p, err, errlen)) return rc;
   if (n_tiles < 0 || n_trees < 0 || n_jobs < 0 || n_parts < 0 || n_rows < 0) return fail(err, errlen, ESP_EINVAL, "negative count");
   if (n_tiles == 0) return ESP_OK;
   if (!Q || !Kb || !Vb || !O || !tiles || !trees) return fail(err, errlen, ESP_EINVAL, "Q, Kb, Vb, O, tiles, trees must not be NULL");
+  if (n_trees == 0) return fail(err, errlen, ESP_EINVAL, "%d tiles without trees", n_tiles);
   if (!kv_pool) return fail(err, errlen, ESP_EINVAL, "kv_pool is NULL");
   if (!p->ring && !blocks) return fail(err, errlen, ESP_EINVAL, "blocks is NULL on a layer without rings");
   if (p->window > 0 && !pos) return fail(err, errlen, ESP_EINVAL, "pos is NULL on a sliding-window layer");
@@ -185,6 +230,8 @@ int esp_attn_forward(const esp_attn_params* p, const void* Q, const void* Kb, co
                 p->rows_per_tile, esp::tiled_max_rows(p->head_dim), p->head_dim);
   if (fam > 0 && n_tiles > 65535)
     return fail(err, errlen, ESP_EUNSUPPORTED, "%d tiles in one pass: the streaming kernel's grid takes at most 65535", n_tiles);
+  DeviceState* dev = nullptr;
+  if (int rc = device_state(&dev, err, errlen)) return rc;
   const Carve c = carve(p, n_rows, n_parts);
   if (!workspace || workspace_bytes < c.total)
     return fail(err, errlen, ESP_EWORKSPACE, "workspace %zu bytes, %zu needed", workspace_bytes, c.total);
@@ -222,6 +269,92 @@ int esp_attn_forward(const esp_attn_params* p, const void* Q, const void* Kb, co
   return ESP_OK;
 }
 
+int esp_attn_forward(const esp_attn_params* p, const void* Q, const void* Kb, const void* Vb, const void* kv_pool,
+                     const int32_t* blocks, const int32_t* desc, const int32_t* pos, void* O, const esp_tile* tiles,
+                     int32_t n_tiles, const esp_tree* trees, int32_t n_trees, const esp_combine* jobs, int32_t n_jobs,
+                     int32_t n_parts, int32_t n_rows, void* workspace, size_t workspace_bytes, void* stream, char* err,
+                     size_t errlen) {
+  return forward_impl(p, Q, Kb, Vb, kv_pool, blocks, desc, pos, O, tiles, n_tiles, trees, n_trees, jobs, n_jobs, n_parts, n_rows,
+                      workspace, workspace_bytes, stream, err, errlen);
+}
+
+int esp_attn_validate(const esp_attn_params* p, const esp_tile* tiles, int32_t n_tiles, const esp_tree* trees, int32_t n_trees,
+                      const esp_combine* jobs, int32_t n_jobs, int32_t n_parts, int32_t n_rows, const int32_t* blocks,
+                      int32_t n_block_entries, int32_t pool_blocks, char* err, size_t errlen) {
+  if (int rc = check_params(p, err, errlen)) return rc;
+  if (n_tiles < 0 || n_trees < 0 || n_jobs < 0 || n_parts < 0 || n_rows < 0 || n_block_entries < 0 || pool_blocks < 0)
+    return fail(err, errlen, ESP_EINVAL, "negative count");
+  if (p->rows_per_tile <= 0) return fail(err, errlen, ESP_EINVAL, "rows_per_tile %d", p->rows_per_tile);
+  if ((n_tiles && !tiles) || (n_trees && !trees) || (n_jobs && !jobs)) return fail(err, errlen, ESP_EINVAL, "NULL record array");
+  if (!p->ring && n_block_entries && !blocks) return fail(err, errlen, ESP_EINVAL, "blocks is NULL");
+  const int64_t bt = p->bt;
+  for (int i = 0; i < n_trees; ++i) {
+    const esp_tree& t = trees[i];
+    if (t.base < 0 || t.M < 0 || int64_t(t.base) + t.M > n_rows)
+      return fail(err, errlen, ESP_EINVAL, "tree %d: rows [%d, %d + %d) outside the pass's %d rows", i, t.base, t.base, t.M, n_rows);
+    if (t.P < 0 || t.table < 0) return fail(err, errlen, ESP_EINVAL, "tree %d: P %d, table %d", i, t.P, t.table);
+    if (p->ring) {
+      if (t.P > 0 && int64_t(t.table) + p->ring > pool_blocks)
+        return fail(err, errlen, ESP_EINVAL, "tree %d: ring blocks [%d, %d + %d) outside the pool's %d blocks", i, t.table, t.table, p->ring, pool_blocks);
+    } else {
+      const int64_t nb = (t.P + bt - 1) / bt;
+      if (t.table + nb > n_block_entries)
+        return fail(err, errlen, ESP_EINVAL, "tree %d: block list [%d, %d + %lld) outside the %d entries of blocks", i, t.table, t.table,
+                    (long long)nb, n_block_entries);
+      for (int64_t b = 0; b < nb; ++b)
+        if (blocks[t.table + b] < 0 || blocks[t.table + b] >= pool_blocks)
+          return fail(err, errlen, ESP_EINVAL, "tree %d: block %d (entry %lld of its list) outside the pool's %d blocks", i, blocks[t.table + b],
+                      (long long)b, pool_blocks);
+    }
+  }
+  // every partial record is written by exactly one tile and read by exactly one job
+  std::vector<int32_t> part_job(size_t(n_parts), -1);
+  for (int j = 0; j < n_jobs; ++j) {
+    const esp_combine& c = jobs[j];
+    if (c.r0 < 0 || c.rows <= 0 || c.rows > p->rows_per_tile || int64_t(c.r0) + c.rows > n_rows)
+      return fail(err, errlen, ESP_EINVAL, "job %d: rows [%d, %d + %d), %d rows per tile, %d rows in the pass", j, c.r0, c.r0, c.rows,
+                  p->rows_per_tile, n_rows);
+    if (c.part0 < 0 || c.nparts <= 0 || int64_t(c.part0) + c.nparts > n_parts)
+      return fail(err, errlen, ESP_EINVAL, "job %d: parts [%d, %d + %d) outside the pass's %d records", j, c.part0, c.part0, c.nparts, n_parts);
+    for (int q = c.part0; q < c.part0 + c.nparts; ++q) {
+      if (part_job[size_t(q)] >= 0) return fail(err, errlen, ESP_EINVAL, "partial record %d is merged by jobs %d and %d", q, part_job[size_t(q)], j);
+      part_job[size_t(q)] = j;
+    }
+  }
+  std::vector<char> part_written(size_t(n_parts), 0);
+  for (int i = 0; i < n_tiles; ++i) {
+    const esp_tile& t = tiles[i];
+    if (t.tree < 0 || t.tree >= n_trees) return fail(err, errlen, ESP_EINVAL, "tile %d: tree %d of %d", i, t.tree, n_trees);
+    const esp_tree& tr = trees[t.tree];
+    if (t.r0 < tr.base || t.r0 >= tr.base + tr.M)
+      return fail(err, errlen, ESP_EINVAL, "tile %d: first row %d outside its tree's rows [%d, %d)", i, t.r0, tr.base, tr.base + tr.M);
+    if ((t.r0 - tr.base) % p->rows_per_tile) return fail(err, errlen, ESP_EINVAL, "tile %d: first row %d is no multiple of %d rows into its tree", i, t.r0, p->rows_per_tile);
+    const bool open = t.k1 == INT32_MAX;  // up to the tree's cached length when the kernel runs
+    if (t.k0 < 0 || (!open && (t.k1 < t.k0 || t.k1 > tr.P)) || (open && t.k0 > tr.P))
+      return fail(err, errlen, ESP_EINVAL, "tile %d: cached range [%d, %d) outside its tree's %d cached keys", i, t.k0, t.k1, tr.P);
+    if (t.part < -1 || t.part >= n_parts) return fail(err, errlen, ESP_EINVAL, "tile %d: partial record %d of %d", i, t.part, n_parts);
+    if (t.part >= 0) {
+      if (part_written[size_t(t.part)]) return fail(err, errlen, ESP_EINVAL, "tile %d: partial record %d is written by another tile too", i, t.part);
+      part_written[size_t(t.part)] = 1;
+      if (n_jobs > 0) {
+        const int j = part_job[size_t(t.part)];
+        if (j < 0) return fail(err, errlen, ESP_EINVAL, "tile %d: no job merges its partial record %d", i, t.part);
+        if (jobs[j].r0 != t.r0 || jobs[j].rows != (tr.base + tr.M - t.r0 < p->rows_per_tile ? tr.base + tr.M - t.r0 : p->rows_per_tile))
+          return fail(err, errlen, ESP_EINVAL, "tile %d: job %d merges rows [%d, %d + %d), the tile holds rows from %d", i, j, jobs[j].r0,
+                      jobs[j].r0, jobs[j].rows, t.r0);
+      }
+    }
+    if (t.last != 0 && t.last != 1) return fail(err, errlen, ESP_EINVAL, "tile %d: last %d (0 or 1)", i, t.last);
+    if (t.b0 < 0 || t.b0 > tr.M) return fail(err, errlen, ESP_EINVAL, "tile %d: first batch key %d of %d rows", i, t.b0, tr.M);
+    if (t.pad != 0 && t.pad - 1 != tr.table) return fail(err, errlen, ESP_EINVAL, "tile %d: pad %d is neither 0 nor 1 + its tree's table %d", i, t.pad, tr.table);
+  }
+  if (n_jobs > 0)
+    for (int q = 0; q < n_parts; ++q)
+      if (part_job[size_t(q)] >= 0 && !part_written[size_t(q)])
+        return fail(err, errlen, ESP_EINVAL, "job %d merges partial record %d, which no tile writes", part_job[size_t(q)], q);
+  return ESP_OK;
+}
+
 int esp_attn_time_next(void* start_event, void* stop_event) {
   if ((start_event == nullptr) != (stop_event == nullptr)) return ESP_EINVAL;
   esp::g_time_next.start = static_cast<hipEvent_t>(start_event);
@@ -240,6 +373,7 @@ int esp_attn_combine(const esp_attn_params* p, void* O, const esp_combine* jobs,
   const Carve c = carve(p, n_rows, n_parts);
   if (!workspace || workspace_bytes < c.total)
     return fail(err, errlen, ESP_EWORKSPACE, "workspace %zu bytes, %zu needed", workspace_bytes, c.total);
+  if (reinterpret_cast<uintptr_t>(workspace) % 16) return fail(err, errlen, ESP_EINVAL, "workspace must be 16-byte aligned");
   esp::KArgs a = make_args(p, c, workspace, n_rows);
   a.O = static_cast<uint16_t*>(O);
   hipError_t e = esp::launch_combine(p->dtype, p->head_dim, a, jobs, n_jobs, static_cast<hipStream_t>(stream));

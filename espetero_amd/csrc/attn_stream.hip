@@ -36,6 +36,64 @@
 
 namespace esp {
 
+// Merge of the partial records of one split tile group for 4 dims of one (row, query head), in part
+// order (attention_combine, kernels/40_attention.metal:811-864; kernels/80_gemma.metal:568-597), then
+// the normalised (optionally gated) output.
+template <int DT, int HD>
+__device__ __forceinline__ void merge_records(const KArgs& a, const esp_combine& job, int r, int h, int d) {
+  const int kvh = h / a.G, hg = h - kvh * a.G;
+  const int col = r * a.G + hg;
+  const size_t stride = size_t(a.Hkv) * a.cols;  // records from one part to the next
+  const size_t rec0 = (size_t(job.part0) * a.Hkv + kvh) * a.cols + col;
+  // One pass, 8 records in flight at a time, merged in part order with a running maximum
+  // (a loop that waits for each record's loads in turn is latency bound: the reference
+  // measured 39 us against 11 us for the same change, 40_attention.metal:801-803).
+  float M = -INFINITY, L = 0.0f;
+  f32x4 o = {0, 0, 0, 0};
+  // N records at a time, all their loads issued before the first use. Slots past the last record
+  // repeat record s (a cache hit) with weight 0: loads under a branch would wait for one another.
+  auto merge = [&]<int N>(int s, std::integral_constant<int, N>) __attribute__((always_inline)) {
+    float mN[N], lN[N];
+    f32x4 oN[N];
+#pragma unroll
+    for (int i = 0; i < N; ++i) {
+      const bool in = s + i < job.nparts;
+      const size_t rec = rec0 + size_t(in ? s + i : s) * stride;
+      mN[i] = in ? a.parts_ml[rec * 2] : -INFINITY;
+      lN[i] = a.parts_ml[rec * 2 + 1];
+      oN[i] = *reinterpret_cast<const f32x4*>(a.parts_o + rec * HD + d);
+    }
+    float Mn = M;
+#pragma unroll
+    for (int i = 0; i < N; ++i) Mn = fmaxf(Mn, mN[i]);
+    const float c = (M == -INFINITY) ? 0.0f : fast_exp2(M - Mn);
+    L *= c;
+    o *= c;
+    M = Mn;
+#pragma unroll
+    for (int i = 0; i < N; ++i) {
+      const float w = (mN[i] == -INFINITY) ? 0.0f : fast_exp2(mN[i] - M);
+      L += w * lN[i];
+      o += oN[i] * w;
+    }
+  };
+  if (job.nparts <= 2) {  // the split of a prefill tile: two records, nothing to repeat
+    merge(0, std::integral_constant<int, 2>{});
+  } else {
+    for (int s = 0; s < job.nparts; s += 8) merge(s, std::integral_constant<int, 8>{});
+  }
+  const int row = job.r0 + r;
+  const float inv = L > 0.0f ? 1.0f / L : 0.0f;
+  o *= inv;
+  if (a.gate) {
+    const float* g = a.gate + size_t(row) * a.gate_ld + size_t(h) * a.gate_hs + a.gate_off + d * a.gate_ds;
+#pragma unroll
+    for (int e = 0; e < 4; ++e) o[e] = o[e] / (1.0f + __expf(-g[e * a.gate_ds]));
+  }
+  u32x2 out = {pack2<DT>(o[0], o[1]), pack2<DT>(o[2], o[3])};
+  *reinterpret_cast<u32x2*>(a.O + size_t(row) * a.q_ld + size_t(h) * HD + d) = out;
+}
+
 template <int HD, int SBU>
 struct Unit {  // operands of one unit of SBU 16-key sub-blocks
   u32x4 k[SBU][HD / 32];  // [sub-block][32-dim group]: key = lane % 16, dims 32 kk + 8 (lane / 16) ..
@@ -466,9 +524,7 @@ __global__ __launch_bounds__(HD >= 512 ? 128 : 256, OCC) void attn_stream_kernel
   }
 }
 
-// Merge the split partial records of a tile group in part order
-// (attention_combine, kernels/40_attention.metal:811-864): one thread per
-// (job, row, head, 4 dims).
+// The merge as its own dispatch: one thread per (job, row, head, 4 dims).
 template <int DT, int HD>
 __global__ __launch_bounds__(256) void attn_combine_kernel(const KArgs a, const esp_combine* jobs, int n_jobs) {
   const int per_job = a.R * a.H * (HD / 4);
@@ -481,57 +537,7 @@ __global__ __launch_bounds__(256) void attn_combine_kernel(const KArgs a, const 
   const int h = rem / (HD / 4), d = (rem % (HD / 4)) * 4;
   const esp_combine job = jobs[ji];
   if (r >= job.rows) return;
-  const int kvh = h / a.G, hg = h - kvh * a.G;
-  const int col = r * a.G + hg;
-  const size_t stride = size_t(a.Hkv) * a.cols;  // records from one part to the next
-  const size_t rec0 = (size_t(job.part0) * a.Hkv + kvh) * a.cols + col;
-  // One pass, 8 records in flight at a time, merged in part order with a running maximum
-  // (a loop that waits for each record's loads in turn is latency bound: the reference
-  // measured 39 us against 11 us for the same change, 40_attention.metal:801-803).
-  float M = -INFINITY, L = 0.0f;
-  f32x4 o = {0, 0, 0, 0};
-  // N records at a time, all their loads issued before the first use. Slots past the last record
-  // repeat record s (a cache hit) with weight 0: loads under a branch would wait for one another.
-  auto merge = [&]<int N>(int s, std::integral_constant<int, N>) __attribute__((always_inline)) {
-    float mN[N], lN[N];
-    f32x4 oN[N];
-#pragma unroll
-    for (int i = 0; i < N; ++i) {
-      const bool in = s + i < job.nparts;
-      const size_t rec = rec0 + size_t(in ? s + i : s) * stride;
-      mN[i] = in ? a.parts_ml[rec * 2] : -INFINITY;
-      lN[i] = a.parts_ml[rec * 2 + 1];
-      oN[i] = *reinterpret_cast<const f32x4*>(a.parts_o + rec * HD + d);
-    }
-    float Mn = M;
-#pragma unroll
-    for (int i = 0; i < N; ++i) Mn = fmaxf(Mn, mN[i]);
-    const float c = (M == -INFINITY) ? 0.0f : fast_exp2(M - Mn);
-    L *= c;
-    o *= c;
-    M = Mn;
-#pragma unroll
-    for (int i = 0; i < N; ++i) {
-      const float w = (mN[i] == -INFINITY) ? 0.0f : fast_exp2(mN[i] - M);
-      L += w * lN[i];
-      o += oN[i] * w;
-    }
-  };
-  if (job.nparts <= 2) {  // the split of a prefill tile: two records, nothing to repeat
-    merge(0, std::integral_constant<int, 2>{});
-  } else {
-    for (int s = 0; s < job.nparts; s += 8) merge(s, std::integral_constant<int, 8>{});
-  }
-  const int row = job.r0 + r;
-  const float inv = L > 0.0f ? 1.0f / L : 0.0f;
-  o *= inv;
-  if (a.gate) {
-    const float* g = a.gate + size_t(row) * a.gate_ld + size_t(h) * a.gate_hs + a.gate_off + d * a.gate_ds;
-#pragma unroll
-    for (int e = 0; e < 4; ++e) o[e] = o[e] / (1.0f + __expf(-g[e * a.gate_ds]));
-  }
-  u32x2 out = {pack2<DT>(o[0], o[1]), pack2<DT>(o[2], o[3])};
-  *reinterpret_cast<u32x2*>(a.O + size_t(row) * a.q_ld + size_t(h) * HD + d) = out;
+  merge_records<DT, HD>(a, job, r, h, d);
 }
 
 size_t stream_smem_bytes(int HD, int NC) {
@@ -557,6 +563,30 @@ static hipError_t launch_stream_t(const KArgs& a, int n_tiles, hipStream_t st) {
   if (e != hipSuccess) return e;
   launch_timed(k, dim3(a.Hkv, n_tiles), dim3(HD >= 512 ? 128 : 256), smem, st, a);
   return hipGetLastError();
+}
+
+template <int DT, int HD, int NC>
+static hipError_t stream_attributes_t() {
+  constexpr int SBU = HD == 128 ? 2 : 1;
+  constexpr int OCC = stream_occ(HD, NC);
+  const size_t smem = stream_smem_bytes(HD, NC);
+  hipError_t e = allow_dynamic_lds<attn_stream_kernel<DT, HD, NC, SBU, 16, OCC>>(smem);
+  if (e == hipSuccess) e = allow_dynamic_lds<attn_stream_kernel<DT, HD, NC, SBU, 0, OCC>>(smem);
+  return e;
+}
+
+// The dynamic LDS limit of every variant on the current device, ahead of the first launch (which may
+// happen while a stream is being captured, where a function attribute cannot be set).
+hipError_t stream_init_attributes() {
+  hipError_t e = stream_attributes_t<ESP_F16, 128, 1>();
+  if (e == hipSuccess) e = stream_attributes_t<ESP_F16, 128, 2>();
+  if (e == hipSuccess) e = stream_attributes_t<ESP_F16, 256, 1>();
+  if (e == hipSuccess) e = stream_attributes_t<ESP_F16, 512, 1>();
+  if (e == hipSuccess) e = stream_attributes_t<ESP_BF16, 128, 1>();
+  if (e == hipSuccess) e = stream_attributes_t<ESP_BF16, 128, 2>();
+  if (e == hipSuccess) e = stream_attributes_t<ESP_BF16, 256, 1>();
+  if (e == hipSuccess) e = stream_attributes_t<ESP_BF16, 512, 1>();
+  return e;
 }
 
 // dt, HD, NC are validated by the caller: (HD, NC) in {(128, 1), (128, 2), (256, 1), (512, 1)}.

@@ -614,6 +614,15 @@ static hipError_t launch_tiled_t(const KArgs& a, int n_tiles, hipStream_t st) {
 
 hipError_t launch_tiled512(int dt, const KArgs& a, int n_tiles, hipStream_t st);
 
+// The dynamic LDS limit of every variant on the current device, ahead of the first launch.
+hipError_t tiled_init_attributes() {
+  hipError_t e = allow_dynamic_lds<attn_tiled_kernel<ESP_F16, 128, tiled_occ(128)>>(tiled_smem_bytes(128));
+  if (e == hipSuccess) e = allow_dynamic_lds<attn_tiled_kernel<ESP_F16, 256, tiled_occ(256)>>(tiled_smem_bytes(256));
+  if (e == hipSuccess) e = allow_dynamic_lds<attn_tiled_kernel<ESP_BF16, 128, tiled_occ(128)>>(tiled_smem_bytes(128));
+  if (e == hipSuccess) e = allow_dynamic_lds<attn_tiled_kernel<ESP_BF16, 256, tiled_occ(256)>>(tiled_smem_bytes(256));
+  return e;
+}
+
 hipError_t launch_tiled(int dt, int HD, const KArgs& a, int n_tiles, hipStream_t st) {
   if (HD == 512 && (dt == ESP_F16 || dt == ESP_BF16)) return launch_tiled512(dt, a, n_tiles, st);
   if (dt == ESP_F16 && HD == 128) return launch_tiled_t<ESP_F16, 128>(a, n_tiles, st);

@@ -367,6 +367,12 @@ __global__ __launch_bounds__(256, 1) void attn_tiled512_kernel(const KArgs a, in
     }
 }
 
+// The dynamic LDS limit of both variants on the current device, ahead of the first launch.
+hipError_t tiled512_init_attributes() {
+  const hipError_t e = allow_dynamic_lds<attn_tiled512_kernel<ESP_F16>>(kLds);
+  return e != hipSuccess ? e : allow_dynamic_lds<attn_tiled512_kernel<ESP_BF16>>(kLds);
+}
+
 hipError_t launch_tiled512(int dt, const KArgs& a, int n_tiles, hipStream_t st) {
   constexpr auto kf = attn_tiled512_kernel<ESP_F16>;
   constexpr auto kb = attn_tiled512_kernel<ESP_BF16>;

@@ -1,0 +1,137 @@
+// Measured ceilings of one MI355X for the two bounds the attention kernels are held against, as kernels
+// of their own (include/espetero_ceilings.h): what a plain streaming read reaches at a given size and
+// page scatter, and what the matrix cores reach when the wavefront that feeds them also issues a given
+// amount of vector arithmetic. The reference states its kernels against measured machine limits the
+// same way (docs/kernel-guidelines.md:19-27: a measured stream peak and a measured MMA rate).
+// Measurement only: nothing in the attention path calls these.
+#include <hip/hip_runtime.h>
+#include <hip/hip_ext.h>
+#include <stdint.h>
+
+#include "../../include/espetero_ceilings.h"
+
+namespace {
+
+using u32x4 = uint32_t __attribute__((ext_vector_type(4)));
+using f32x16 = float __attribute__((ext_vector_type(16)));
+using bf16x8 = __bf16 __attribute__((ext_vector_type(8)));
+
+// Every wavefront reads whole pages, 16 bytes per lane per load, DEPTH pages in flight; page p of the
+// launch is pages[p] (a scattered pool) or p itself (address order). The grid is what the streaming
+// attention kernel uses: workgroups of 4 wavefronts, pages dealt round robin over all wavefronts.
+template <int NT, int DEPTH>
+__global__ __launch_bounds__(256, 2) void read_kernel(const char* __restrict__ base, const int32_t* __restrict__ pages, int n_pages,
+                                                       int page_bytes, uint32_t* sink) {
+  const int lane = threadIdx.x & 63;
+  const int gw = blockIdx.x * 4 + (threadIdx.x >> 6), n_waves = gridDim.x * 4;
+  const int per_page = page_bytes / 1024;  // 1 KB per load instruction and wavefront
+  uint32_t acc = 0;
+  for (int p0 = gw; p0 < n_pages; p0 += n_waves * DEPTH) {
+    const char* pg[DEPTH];
+#pragma unroll
+    for (int d = 0; d < DEPTH; ++d) {
+      const int p = p0 + d * n_waves;
+      const int q = p < n_pages ? p : p0;
+      pg[d] = base + size_t(pages ? pages[q] : q) * size_t(page_bytes) + lane * 16;
+    }
+    for (int i = 0; i < per_page; i += 4) {
+      u32x4 v[DEPTH][4];
+#pragma unroll
+      for (int d = 0; d < DEPTH; ++d)
+#pragma unroll
+        for (int j = 0; j < 4; ++j) {
+          const u32x4* src = reinterpret_cast<const u32x4*>(pg[d] + (i + j) * 1024);
+          v[d][j] = NT ? __builtin_nontemporal_load(src) : *src;
+        }
+#pragma unroll
+      for (int d = 0; d < DEPTH; ++d)
+#pragma unroll
+        for (int j = 0; j < 4; ++j) acc ^= v[d][j].x ^ v[d][j].w;
+    }
+  }
+  if (acc == 0x12345678u) sink[0] = acc;  // keeps the loads alive; never true for the bench's data
+}
+
+// One wavefront's instruction stream of a prefill step, nothing else: per matrix instruction
+// (v_mfma_f32_32x32x16_bf16 over four accumulator chains, as Q K^T and P V alternate in the kernel) NV
+// independent fp32 fused multiply-adds and NE v_exp_f32, interleaved by the scheduler one matrix
+// instruction at a time. No memory, no LDS: what is left is the issue port the two kinds share.
+template <int NV, int NE>
+__global__ __launch_bounds__(256, 2) void issue_kernel(float* out, int iters, uint32_t seed) {
+  u32x4 a = {seed + threadIdx.x, seed * 3u, seed * 5u, seed * 7u};
+  u32x4 b = {seed ^ 0x3f803f80u, 0x3f803f80u, 0x3f803f80u, 0x3f803f80u};
+  f32x16 c[4] = {};
+  float v[16], x[8];
+#pragma unroll
+  for (int i = 0; i < 16; ++i) v[i] = float(threadIdx.x + i) * 1e-3f;
+#pragma unroll
+  for (int i = 0; i < 8; ++i) x[i] = -float(threadIdx.x + i) * 1e-2f;
+  for (int it = 0; it < iters; ++it) {
+#pragma unroll
+    for (int j = 0; j < 32; ++j) {
+      c[j & 3] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(bf16x8, a), __builtin_bit_cast(bf16x8, b), c[j & 3], 0, 0, 0);
+#pragma unroll
+      for (int e = 0; e < NV; ++e) v[(j * NV + e) & 15] = __builtin_fmaf(v[(j * NV + e) & 15], 1.0001f, 0.5f);
+#pragma unroll
+      for (int e = 0; e < NE; ++e) x[(j * NE + e) & 7] = __builtin_amdgcn_exp2f(x[(j * NE + e) & 7]) - 1.5f;
+      __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
+      if (NV + 2 * NE > 0) __builtin_amdgcn_sched_group_barrier(0x002, NV + 2 * NE, 0);
+    }
+  }
+  float r = 0;
+#pragma unroll
+  for (int i = 0; i < 16; ++i) r += c[0][i] + c[1][i] + c[2][i] + c[3][i] + v[i];
+#pragma unroll
+  for (int i = 0; i < 8; ++i) r += x[i];
+  out[blockIdx.x * 256 + threadIdx.x] = r;
+}
+
+template <typename K, typename... Args>
+hipError_t launch(K k, dim3 grid, dim3 block, hipStream_t st, hipEvent_t e0, hipEvent_t e1, Args... args) {
+  if (e0 && e1) hipExtLaunchKernelGGL(k, grid, block, 0, st, e0, e1, 0, args...);
+  else hipLaunchKernelGGL(k, grid, block, 0, st, args...);
+  return hipGetLastError();
+}
+
+}  // namespace
+
+extern "C" {
+
+int esp_ceiling_hbm_read(const void* base, const int32_t* pages, int32_t n_pages, int32_t page_bytes, int32_t nontemporal,
+                         int32_t workgroups, uint32_t* sink, void* stream, void* start_event, void* stop_event) {
+  if (!base || !sink || n_pages <= 0 || page_bytes < 4096 || page_bytes % 4096 || workgroups <= 0) return 1;
+  const auto st = static_cast<hipStream_t>(stream);
+  const auto e0 = static_cast<hipEvent_t>(start_event), e1 = static_cast<hipEvent_t>(stop_event);
+  const char* b = static_cast<const char*>(base);
+  const hipError_t e = nontemporal ? launch(read_kernel<1, 2>, dim3(workgroups), dim3(256), st, e0, e1, b, pages, n_pages, page_bytes, sink)
+                                   : launch(read_kernel<0, 2>, dim3(workgroups), dim3(256), st, e0, e1, b, pages, n_pages, page_bytes, sink);
+  return e == hipSuccess ? 0 : 3;
+}
+
+int esp_ceiling_mfma_issue(int32_t valu_per_mfma, int32_t exp_per_mfma, int32_t workgroups, int32_t iters, float* out, void* stream,
+                           void* start_event, void* stop_event) {
+  if (!out || workgroups <= 0 || iters <= 0) return 1;
+  const auto st = static_cast<hipStream_t>(stream);
+  const auto e0 = static_cast<hipEvent_t>(start_event), e1 = static_cast<hipEvent_t>(stop_event);
+  const dim3 g(workgroups), b(256);
+  const int key = valu_per_mfma * 10 + exp_per_mfma;
+  hipError_t e;
+  switch (key) {
+    case 0: e = launch(issue_kernel<0, 0>, g, b, st, e0, e1, out, iters, 1u); break;
+    case 10: e = launch(issue_kernel<1, 0>, g, b, st, e0, e1, out, iters, 1u); break;
+    case 20: e = launch(issue_kernel<2, 0>, g, b, st, e0, e1, out, iters, 1u); break;
+    case 30: e = launch(issue_kernel<3, 0>, g, b, st, e0, e1, out, iters, 1u); break;
+    case 40: e = launch(issue_kernel<4, 0>, g, b, st, e0, e1, out, iters, 1u); break;
+    case 60: e = launch(issue_kernel<6, 0>, g, b, st, e0, e1, out, iters, 1u); break;
+    case 1: e = launch(issue_kernel<0, 1>, g, b, st, e0, e1, out, iters, 1u); break;
+    case 11: e = launch(issue_kernel<1, 1>, g, b, st, e0, e1, out, iters, 1u); break;
+    case 21: e = launch(issue_kernel<2, 1>, g, b, st, e0, e1, out, iters, 1u); break;
+    case 31: e = launch(issue_kernel<3, 1>, g, b, st, e0, e1, out, iters, 1u); break;
+    case 41: e = launch(issue_kernel<4, 1>, g, b, st, e0, e1, out, iters, 1u); break;
+    case 51: e = launch(issue_kernel<5, 1>, g, b, st, e0, e1, out, iters, 1u); break;
+    default: return 2;
+  }
+  return e == hipSuccess ? 0 : 3;
+}
+
+}  // extern "C"

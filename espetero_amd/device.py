@@ -67,6 +67,20 @@ def forward(params, Q, Kb, Vb, pool, blocks, desc, pos, O, tiles, n_tiles, trees
     abi.check(rc, err)
 
 
+def validate(params, tiles, trees, jobs, n_parts, n_rows, blocks, pool_blocks):
+    """Host-side bounds check of a pass's records (numpy arrays) before they are uploaded. Raises EspError."""
+    tiles = np.ascontiguousarray(tiles, dtype=abi.TILE_DT)
+    trees = np.ascontiguousarray(trees, dtype=abi.TREE_DT)
+    jobs = np.ascontiguousarray(jobs, dtype=abi.COMBINE_DT)
+    blocks = None if blocks is None else np.ascontiguousarray(blocks, dtype=np.int32)
+    hp = lambda a: None if a is None or a.size == 0 else a.ctypes.data  # noqa: E731
+    err = C.create_string_buffer(_ERRLEN)
+    rc = abi.attn_lib().esp_attn_validate(C.byref(params), hp(tiles), len(tiles), hp(trees), len(trees), hp(jobs), len(jobs),
+                                          n_parts, n_rows, hp(blocks), 0 if blocks is None else len(blocks), pool_blocks,
+                                          err, _ERRLEN)
+    abi.check(rc, err)
+
+
 def time_next(start, stop):
     """The next forward() records its attention kernel's begin and end into these two torch events
     (created with enable_timing=True and recorded once before, so that their handles exist)."""
@@ -143,7 +157,11 @@ class DevicePass:
     """One planned pass resident on the device: uploads the records once and
     replays esp_attn_forward (what a decode chain does between host syncs)."""
 
-    def __init__(self, params, trees, tiles, jobs, n_parts, n_rows, blocks, desc=None, pos=None, device="cuda"):
+    def __init__(self, params, trees, tiles, jobs, n_parts, n_rows, blocks, desc=None, pos=None, device="cuda",
+                 pool_blocks=None):
+        """pool_blocks: blocks in the pool; when given, the records are checked on the host before the upload."""
+        if pool_blocks is not None:
+            validate(params, tiles, trees, jobs, n_parts, n_rows, blocks, pool_blocks)
         self.params = params
         self.n_trees, self.n_tiles, self.n_jobs = len(trees), len(tiles), len(jobs)
         self.n_parts, self.n_rows = n_parts, n_rows

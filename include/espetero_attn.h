@@ -45,7 +45,7 @@
 extern "C" {
 #endif
 
-#define ESP_ABI_VERSION 1
+#define ESP_ABI_VERSION 2
 
 enum { ESP_OK = 0, ESP_EINVAL = 1, ESP_EUNSUPPORTED = 2, ESP_ELAUNCH = 3, ESP_EWORKSPACE = 4 };
 enum { ESP_F16 = 0, ESP_BF16 = 1 };
@@ -118,7 +118,9 @@ typedef struct esp_attn_params {
                             rounding, its dots computed before the pass by esp_head_gate */
 } esp_attn_params;
 
-/* Library / device check. Safe to call more than once. */
+/* Library / device check and the per-device set-up: raises the dynamic LDS limit of every kernel
+ * variant, so that the first launch of any variant may happen inside a stream capture. Safe to call more than once; a call that was not
+ * preceded by it does the same set-up on first use of a device. */
 int esp_attn_init(int device, char* err, size_t errlen);
 int esp_attn_abi_version(void);
 
@@ -163,6 +165,18 @@ int esp_attn_forward(const esp_attn_params* p, const void* Q, const void* Kb, co
                      int32_t n_parts, int32_t n_rows, void* workspace, size_t workspace_bytes, void* stream, char* err,
                      size_t errlen);
 
+/* Host-side check of a pass's records before they are uploaded; no counterpart in the reference, whose
+ * planner and kernels live in one program (forest.h:2646-2716). The kernels trust every index they
+ * read from device memory, and a bad one is an out-of-bounds access on the GPU. ALL pointers here are
+ * HOST pointers to the same records esp_attn_forward will read: every tree's rows inside [0, n_rows),
+ * its block list inside blocks[0, n_block_entries) with ids below pool_blocks (ring layers: its ring
+ * inside the pool), every tile's tree, rows, cached range, partial record and table hint, every job's
+ * rows and records, each record written by one tile and merged by one job. ESP_EINVAL + message names
+ * the first offender. Touches no device. */
+int esp_attn_validate(const esp_attn_params* p, const esp_tile* tiles, int32_t n_tiles, const esp_tree* trees, int32_t n_trees,
+                      const esp_combine* jobs, int32_t n_jobs, int32_t n_parts, int32_t n_rows, const int32_t* blocks,
+                      int32_t n_block_entries, int32_t pool_blocks, char* err, size_t errlen);
+
 /* Measurement hook; no counterpart in the reference (its bench times command
  * buffers, src/model/impl/bench.h:697-722). The next esp_attn_forward (or
  * esp_attn_prep) hands the two HIP events (hipEvent_t, created with timing
@@ -171,7 +185,9 @@ int esp_attn_forward(const esp_attn_params* p, const void* Q, const void* Kb, co
  * records the kernel's own begin and end
  * into them: hipEventElapsedTime(start, stop) is then that kernel's duration,
  * without marker packets between the kernels of the stream. The pair is used
- * once. Both NULL clears a pending pair. */
+ * once, by the next such call, whether or not that call launches anything (a call
+ * that returns early drops it). One pending pair per process: a single caller
+ * thread arms it and makes the call. Both NULL clears a pending pair. */
 int esp_attn_time_next(void* start_event, void* stop_event);
 
 /* The split-K merge alone: attention_combine (40_:811-864, 80_:568-597) as its

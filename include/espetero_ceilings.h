@@ -1,0 +1,41 @@
+/* espetero_ceilings.h -- measured machine ceilings for the attention path's two rooflines
+ * (libespetero_ceilings.so, built from espetero_amd/csrc/ceilings.hip; gfx950 only).
+ *
+ * No counterpart among the reference's kernels; its documentation holds its kernels against
+ * measured limits of the machine rather than data-sheet figures (docs/kernel-guidelines.md:19-27:
+ * a measured stream bandwidth and a measured MMA rate). These two calls produce the same two
+ * figures on an MI355X; bench.py reports them (--workload hbm_read_ceiling, mfma_issue_ceiling)
+ * and states every roofline fraction against the data-sheet peak and against them.
+ * Conventions as in espetero_attn.h: device pointers, work enqueued on `stream`, 0 or an error
+ * code (1 bad argument, 2 unsupported, 3 launch failure). start_event / stop_event: two
+ * hipEvent_t (or both NULL) that take the kernel's own begin and end.
+ */
+#ifndef ESPETERO_CEILINGS_H
+#define ESPETERO_CEILINGS_H
+
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+/* A plain streaming read: n_pages pages of page_bytes (a multiple of 4096) from `base`, page i of the
+ * launch being pages[i] (device array; NULL: page i itself, i.e. address order), 16 bytes per lane per
+ * load, two pages in flight per wavefront, `workgroups` workgroups of 4 wavefronts. nontemporal: the
+ * loads carry the streaming hint the decode kernel's K / V loads carry. sink: one device word. */
+int esp_ceiling_hbm_read(const void* base, const int32_t* pages, int32_t n_pages, int32_t page_bytes, int32_t nontemporal,
+                         int32_t workgroups, uint32_t* sink, void* stream, void* start_event, void* stop_event);
+
+/* The matrix cores under a wavefront that also issues vector arithmetic: every wavefront runs
+ * iters x 32 v_mfma_f32_32x32x16_bf16 (four accumulator chains), and per matrix instruction
+ * valu_per_mfma fp32 fused multiply-adds plus exp_per_mfma (v_exp_f32 + one add), no memory access.
+ * Supported: exp_per_mfma 0 with valu_per_mfma 0, 1, 2, 3, 4, 6; exp_per_mfma 1 with 0 .. 5.
+ * Workgroups of 4 wavefronts, at most two per compute unit. out: workgroups * 256 floats.
+ * Flops of a launch: workgroups * 4 * iters * 32 * 32768. */
+int esp_ceiling_mfma_issue(int32_t valu_per_mfma, int32_t exp_per_mfma, int32_t workgroups, int32_t iters, float* out, void* stream,
+                           void* start_event, void* stop_event);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* ESPETERO_CEILINGS_H */

@@ -1,0 +1,60 @@
+"""Run as a script in a process of its own (tests/test_gpu_capture.py starts it): after esp_attn_init, the very
+first launch of kernel variants that need more than the default dynamic LDS happens inside a stream capture;
+the replayed graph must give the eager results bit for bit."""
+import os
+import sys
+
+import numpy as np
+import torch
+
+sys.path.insert(0, os.path.dirname(os.path.dirname(os.path.abspath(__file__))))
+sys.path.insert(0, os.path.dirname(os.path.abspath(__file__)))
+
+from espetero_amd import abi, device, host  # noqa: E402
+from gpu_utils import dev_u16, native_pool, plan, to_host_u16  # noqa: E402
+from helpers import small_case  # noqa: E402
+
+
+def main():
+    device.init(0)
+    cases = [small_case(seed=81, seqs=((2500, 1), (700, 1)), H=4, Hkv=2, HD=256, rows_per_tile=1),            # streaming, 67 KB of LDS
+             small_case(seed=82, seqs=((3000, 4),), H=32, Hkv=4, rows_per_tile=4),                             # two column tiles, 68 KB
+             small_case(seed=83, seqs=((300, 130),), H=4, Hkv=2, HD=256, rows_per_tile=128, dtype=abi.ESP_BF16),  # tiled, 128 KB
+             small_case(seed=84, seqs=((200, 70),), H=4, Hkv=2, HD=512, rows_per_tile=64)]                    # tiled, head dim 512
+    runs = []
+    for c in cases:
+        opts = host.options_mi355x(c.params.rows_per_tile, 64)
+        tiles, jobs, n_parts = plan(c, opts)
+        dp = device.DevicePass(c.params, c.trees, tiles, jobs, n_parts, c.n_rows, c.blocks, c.desc, c.pos, pool_blocks=c.n_blocks)
+        Q, Kb, Vb = dev_u16(c.Q), dev_u16(c.Kb), dev_u16(c.Vb)
+        runs.append((dp, Q, Kb, Vb, native_pool(c), torch.zeros_like(Q)))
+    torch.cuda.synchronize()
+    g = torch.cuda.CUDAGraph()
+    side = torch.cuda.Stream()
+    with torch.cuda.stream(side):
+        with torch.cuda.graph(g, stream=side):
+            for dp, Q, Kb, Vb, pool, O in runs:
+                dp.run(Q, Kb, Vb, pool, O)           # the first launch of each of these variants in this process
+    torch.cuda.synchronize()
+    replays = []
+    for _ in range(2):
+        for r in runs:
+            r[5].fill_(0)                            # a fill kernel between the replays
+        torch.cuda.synchronize()
+        g.replay()
+        torch.cuda.synchronize()
+        replays.append([to_host_u16(r[5]).copy() for r in runs])
+    for dp, Q, Kb, Vb, pool, O in runs:
+        O.fill_(0)
+        dp.run(Q, Kb, Vb, pool, O)
+    torch.cuda.synchronize()
+    for i, r in enumerate(runs):
+        eager = to_host_u16(r[5])
+        assert np.abs(eager.astype(np.int64)).max() > 0, f"case {i}: eager output is all zero"
+        for k, rep in enumerate(replays):
+            assert (rep[i] == eager).all(), f"case {i}: replay {k} differs from the eager run"
+    print("capture_first_launch: ok", flush=True)
+
+
+if __name__ == "__main__":
+    main()

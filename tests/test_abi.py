@@ -104,3 +104,68 @@ def test_prep_gate_and_chain_argument_errors():
     a.gate_headwise = 2
     assert lib.esp_attn_forward(C.byref(a), None, None, None, None, None, None, None, None, None, 1, None, 1, None, 0, 0, 1,
                                 None, 0, None, err, 256) == 1 and b"gate_headwise" in err.value
+
+
+def _planned_pass():
+    """A small decode + verify pass planned on the host: records as numpy arrays."""
+    import numpy as np
+    from espetero_amd import synth
+    p = synth.make_params(32, 4, 128, abi.ESP_F16, 16, rows_per_tile=4)
+    trees = np.array([(0, 1000, 0, 4), (4, 70, 63, 1), (5, 0, 68, 2)], abi.TREE_DT)
+    tiles, jobs, n_parts = host.plan_tiles(trees, 4, 0, None, host.options_mi355x(4, 64))
+    blocks = np.arange(63 + 5 + 1, dtype=np.int32)[::-1].copy()
+    assert n_parts > 2 and len(jobs) >= 1
+    return p, trees, tiles, jobs, n_parts, 7, blocks, 80
+
+
+def test_validate_accepts_a_planned_pass_and_names_the_first_bad_record():
+    """esp_attn_validate is host arithmetic over host copies of the records: every index a kernel would
+    dereference, checked before the upload."""
+    import numpy as np
+    import pytest
+    from espetero_amd import device
+    p, trees, tiles, jobs, n_parts, n_rows, blocks, pool_blocks = _planned_pass()
+    device.validate(p, tiles, trees, jobs, n_parts, n_rows, blocks, pool_blocks)
+    device.validate(p, tiles, trees, jobs[:0], n_parts, n_rows, blocks, pool_blocks)   # merge as its own call: no jobs here
+
+    def bad(match, tiles=tiles, trees=trees, jobs=jobs, n_parts=n_parts, n_rows=n_rows, blocks=blocks, pool_blocks=pool_blocks):
+        with pytest.raises(abi.EspError, match=match):
+            device.validate(p, tiles, trees, jobs, n_parts, n_rows, blocks, pool_blocks)
+
+    t = tiles.copy(); t[1]["tree"] = 3
+    bad("tile 1: tree 3 of 3", tiles=t)
+    t = tiles.copy(); t[0]["part"] = n_parts
+    bad("tile 0: partial record", tiles=t)
+    t = tiles.copy(); t[0]["r0"] = 4
+    bad("tile 0: first row 4 outside", tiles=t)
+    t = tiles.copy(); t[0]["pad"] = 7
+    bad("tile 0: pad 7", tiles=t)
+    t = tiles.copy(); t[0]["k1"] = 1001
+    bad("tile 0: cached range", tiles=t)
+    t = tiles.copy(); t[-1]["b0"] = 9
+    bad("first batch key 9", tiles=t)
+    split = [i for i in range(len(tiles)) if tiles[i]["part"] >= 0]
+    t = tiles.copy(); t[split[1]]["part"] = t[split[0]]["part"]
+    bad("written by another tile too", tiles=t)
+    t = np.delete(tiles, split[0])
+    bad("which no tile writes", tiles=t)
+    tr = trees.copy(); tr[2]["M"] = 3
+    bad("tree 2: rows", trees=tr)
+    tr = trees.copy(); tr[0]["table"] = 10
+    bad("tree 0: block list", trees=tr)
+    b = blocks.copy(); b[5] = 80
+    bad("tree 0: block 80", blocks=b)
+    bad("tree 0: block 68", pool_blocks=68)
+    j = jobs.copy(); j[0]["nparts"] += 1
+    bad("job 0: parts|merged by jobs", jobs=j)
+    j = jobs.copy(); j[0]["rows"] = 5
+    bad("job 0: rows", jobs=j)
+    j = np.concatenate([jobs, jobs[:1]])
+    bad("merged by jobs 0 and", jobs=j)
+    # ring layers: the tree's table is the first block of its slot's ring
+    p.ring, p.window = 4, 64
+    tr = np.array([(0, 1000, 8, 1)], abi.TREE_DT)
+    tl, jb, npart = host.plan_tiles(tr, 4, 64, np.full((1, 4), 1000, np.int32), host.options_mi355x(1, 8))
+    device.validate(p, tl, tr, jb, npart, 1, None, 12)
+    with pytest.raises(abi.EspError, match="ring blocks"):
+        device.validate(p, tl, tr, jb, npart, 1, None, 11)

@@ -101,6 +101,29 @@ def test_stream_kernel_is_deterministic():
         assert (run_case(c) == a).all()
 
 
+@pytest.mark.parametrize("kw,wg", [
+    (dict(seqs=((4096, 1), (333, 1), (2000, 1)), H=32, Hkv=4, rows_per_tile=1), 256),          # decode, G = 8
+    (dict(seqs=((3000, 4), (1500, 3)), H=32, Hkv=4, rows_per_tile=4, desc_fn=lambda M: synth.verify_desc(M, 1)), 128),  # two column tiles
+    (dict(seqs=((2500, 1), (700, 1)), H=4, Hkv=2, HD=256, rows_per_tile=1, dtype=abi.ESP_BF16), 64),
+    (dict(seqs=((5000, 1), (900, 1)), H=16, Hkv=2, HD=512, rows_per_tile=1), 64),               # wavefront pairs
+    (dict(seqs=tuple((200 + 37 * i, 1) for i in range(70)), H=8, Hkv=2, rows_per_tile=1), 2048),  # more jobs than one wavefront looks up at once
+    (dict(seqs=((900, 1), (2000, 1)), window=256, ring_layer=True, rows_per_tile=1), 64),
+])
+def test_stream_kernel_merge_as_its_own_call_gives_the_same_bits(kw, wg):
+    """esp_attn_forward with n_jobs = 0 followed by esp_attn_combine gives the bits of the one call that
+    does both, run after run, and both are the checker's result."""
+    from gpu_utils import plan, run_case
+    c = small_case(seed=47, fill_unused=not kw.get("ring_layer", False), **kw)
+    opts = host.options_mi355x(c.params.rows_per_tile, wg)
+    tiles, jobs, n_parts = plan(c, opts)
+    assert len(jobs) >= 2 and n_parts > len(jobs), "the plan must split"
+    print(f"case seqs={c.meta['seqs'][:4]} tiles={len(tiles)} jobs={len(jobs)} parts={n_parts}", flush=True)
+    two = run_case(c, opts, two_step=True)
+    for _ in range(3):
+        assert (run_case(c, opts) == two).all()
+    assert max_abs(two, oracle_direct(c, threads=8), c.params.dtype) <= tol_for(c.params.dtype)
+
+
 def test_gate():
     import torch
     from gpu_utils import run_case
