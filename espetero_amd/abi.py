@@ -12,6 +12,7 @@ import numpy as np
 ESP_F16, ESP_BF16 = 0, 1
 ESP_LAYOUT_REFERENCE, ESP_LAYOUT_NATIVE = 0, 1
 ESP_ABI_VERSION = 2
+ESP_STATIC_SCRATCH_BYTES = 32 << 20
 
 _PKG_DIR = os.path.dirname(os.path.abspath(__file__))
 ATTN_LIB_PATH = os.path.join(_PKG_DIR, "csrc", "libespetero_attn.so")
@@ -81,6 +82,8 @@ ATTN_SYMBOLS = {
     "esp_attn_workspace_bytes": (C.c_size_t, (_P, C.c_int32, C.c_int32)),
     "esp_attn_forward": (C.c_int, (_P, _V, _V, _V, _V, _V, _V, _V, _V, _V, C.c_int32, _V, C.c_int32, _V, C.c_int32,
                                    C.c_int32, C.c_int32, _V, C.c_size_t, _V) + _ERR),
+    "esp_attn_forward_static": (C.c_int, (_P, _V, _V, _V, _V, _V, _V, _V, _V, _V, C.c_int32, _V, C.c_int32, _V, C.c_int32,
+                                          C.c_int32, C.c_int32, _V) + _ERR),
     "esp_attn_validate": (C.c_int, (_P, _V, C.c_int32, _V, C.c_int32, _V, C.c_int32, C.c_int32, C.c_int32, _V, C.c_int32,
                                     C.c_int32) + _ERR),
     "esp_attn_time_next": (C.c_int, (_V, _V)),

@@ -33,6 +33,14 @@ hipError_t tiled_init_attributes();
 hipError_t tiled512_init_attributes();
 }  // namespace esp
 
+// Library-owned device memory, one copy per GPU, held until the process ends: what
+// esp_attn_forward_static uses in place of a caller's workspace (partial records of split tiles, the
+// transposed batch V of the tiled kernels). In host code this name is a stand-in, not a device
+// address: the address comes from hipGetSymbolAddress, once per device (device_state below), and only
+// that is handed to kernels.
+constexpr size_t kScratchBytes = ESP_STATIC_SCRATCH_BYTES;
+static __device__ __align__(256) unsigned char scratch[kScratchBytes];
+
 namespace {
 
 int fail(char* err, size_t errlen, int code, const char* fmt, ...) {
@@ -121,13 +129,14 @@ esp::KArgs make_args(const esp_attn_params* p, const Carve& c, void* workspace, 
 
 constexpr int kMaxDevices = 64;
 struct DeviceState {
+  unsigned char* scratch = nullptr;  // this device's copy of `scratch`
   bool ready = false;
 };
 DeviceState g_dev[kMaxDevices];
 std::mutex g_dev_mutex;
 
-// State of the current device; the first call on a device raises the kernels' dynamic LDS limits (a
-// process-wide fact of that device, not stream work).
+// State of the current device; the first call on a device looks its copy of `scratch` up and raises the
+// kernels' dynamic LDS limits (both are process-wide facts of that device, neither is stream work).
 int device_state(DeviceState** out, char* err, size_t errlen) {
   int dev = 0;
   hipError_t e = hipGetDevice(&dev);
@@ -136,9 +145,12 @@ int device_state(DeviceState** out, char* err, size_t errlen) {
   std::lock_guard<std::mutex> lock(g_dev_mutex);
   DeviceState& d = g_dev[dev];
   if (!d.ready) {
+    void* ps = nullptr;
+    if ((e = hipGetSymbolAddress(&ps, HIP_SYMBOL(scratch))) != hipSuccess) return hip_fail(err, errlen, "hipGetSymbolAddress(scratch)", e);
     if ((e = esp::stream_init_attributes()) != hipSuccess) return hip_fail(err, errlen, "hipFuncSetAttribute (streaming kernels)", e);
     if ((e = esp::tiled_init_attributes()) != hipSuccess) return hip_fail(err, errlen, "hipFuncSetAttribute (tiled kernels)", e);
     if ((e = esp::tiled512_init_attributes()) != hipSuccess) return hip_fail(err, errlen, "hipFuncSetAttribute (tiled kernels, head dim 512)", e);
+    d.scratch = static_cast<unsigned char*>(ps);
     d.ready = true;
   }
   *out = &d;
@@ -202,11 +214,13 @@ size_t esp_attn_workspace_bytes(const esp_attn_params* p, int32_t n_rows, int32_
   return carve(p, n_rows, n_parts).total;
 }
 
+// Attention of one layer over a planned pass. workspace NULL: the library's own scratch array
+// (esp_attn_forward_static), whose size is the limit.
 static int forward_impl(const esp_attn_params* p, const void* Q, const void* Kb, const void* Vb, const void* kv_pool,
                         const int32_t* blocks, const int32_t* desc, const int32_t* pos, void* O, const esp_tile* tiles,
                         int32_t n_tiles, const esp_tree* trees, int32_t n_trees, const esp_combine* jobs, int32_t n_jobs,
-                        int32_t n_parts, int32_t n_rows, void* workspace, size_t workspace_bytes, void* stream, char* err,
-                        size_t errlen) {
+                        int32_t n_parts, int32_t n_rows, void* workspace, size_t workspace_bytes, bool own_scratch,
+                        void* stream, char* err, size_t errlen) {
   // A pending event pair belongs to this call whatever becomes of it: a call that launches nothing
   // must not leave it armed for some later launch.
   struct DropPair {
@@ -233,6 +247,13 @@ static int forward_impl(const esp_attn_params* p, const void* Q, const void* Kb,
   DeviceState* dev = nullptr;
   if (int rc = device_state(&dev, err, errlen)) return rc;
   const Carve c = carve(p, n_rows, n_parts);
+  if (own_scratch) {
+    if (c.total > kScratchBytes)
+      return fail(err, errlen, ESP_EWORKSPACE, "this pass needs %zu bytes of scratch; the library's own array holds %zu "
+                  "(use esp_attn_forward with a workspace)", c.total, kScratchBytes);
+    workspace = dev->scratch;
+    workspace_bytes = kScratchBytes;
+  }
   if (!workspace || workspace_bytes < c.total)
     return fail(err, errlen, ESP_EWORKSPACE, "workspace %zu bytes, %zu needed", workspace_bytes, c.total);
   if (reinterpret_cast<uintptr_t>(workspace) % 16) return fail(err, errlen, ESP_EINVAL, "workspace must be 16-byte aligned");
@@ -275,7 +296,15 @@ int esp_attn_forward(const esp_attn_params* p, const void* Q, const void* Kb, co
                      int32_t n_parts, int32_t n_rows, void* workspace, size_t workspace_bytes, void* stream, char* err,
                      size_t errlen) {
   return forward_impl(p, Q, Kb, Vb, kv_pool, blocks, desc, pos, O, tiles, n_tiles, trees, n_trees, jobs, n_jobs, n_parts, n_rows,
-                      workspace, workspace_bytes, stream, err, errlen);
+                      workspace, workspace_bytes, false, stream, err, errlen);
+}
+
+int esp_attn_forward_static(const esp_attn_params* p, const void* Q, const void* Kb, const void* Vb, const void* kv_pool,
+                            const int32_t* blocks, const int32_t* desc, const int32_t* pos, void* O, const esp_tile* tiles,
+                            int32_t n_tiles, const esp_tree* trees, int32_t n_trees, const esp_combine* jobs, int32_t n_jobs,
+                            int32_t n_parts, int32_t n_rows, void* stream, char* err, size_t errlen) {
+  return forward_impl(p, Q, Kb, Vb, kv_pool, blocks, desc, pos, O, tiles, n_tiles, trees, n_trees, jobs, n_jobs, n_parts, n_rows,
+                      nullptr, 0, true, stream, err, errlen);
 }
 
 int esp_attn_validate(const esp_attn_params* p, const esp_tile* tiles, int32_t n_tiles, const esp_tree* trees, int32_t n_trees,

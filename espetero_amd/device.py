@@ -67,6 +67,16 @@ def forward(params, Q, Kb, Vb, pool, blocks, desc, pos, O, tiles, n_tiles, trees
     abi.check(rc, err)
 
 
+def forward_static(params, Q, Kb, Vb, pool, blocks, desc, pos, O, tiles, n_tiles, trees, n_trees, jobs, n_jobs, n_parts, n_rows,
+                   stream=None):
+    """forward() over the library's own scratch array: no workspace, no allocation."""
+    err = C.create_string_buffer(_ERRLEN)
+    rc = abi.attn_lib().esp_attn_forward_static(
+        C.byref(params), _ptr(Q), _ptr(Kb), _ptr(Vb), _ptr(pool), _ptr(blocks), _ptr(desc), _ptr(pos), _ptr(O),
+        _ptr(tiles), n_tiles, _ptr(trees), n_trees, _ptr(jobs), n_jobs, n_parts, n_rows, _stream(stream), err, _ERRLEN)
+    abi.check(rc, err)
+
+
 def validate(params, tiles, trees, jobs, n_parts, n_rows, blocks, pool_blocks):
     """Host-side bounds check of a pass's records (numpy arrays) before they are uploaded. Raises EspError."""
     tiles = np.ascontiguousarray(tiles, dtype=abi.TILE_DT)
@@ -158,11 +168,13 @@ class DevicePass:
     replays esp_attn_forward (what a decode chain does between host syncs)."""
 
     def __init__(self, params, trees, tiles, jobs, n_parts, n_rows, blocks, desc=None, pos=None, device="cuda",
-                 pool_blocks=None):
-        """pool_blocks: blocks in the pool; when given, the records are checked on the host before the upload."""
+                 pool_blocks=None, static=False):
+        """pool_blocks: blocks in the pool; when given, the records are checked on the host before the upload.
+        static: run over the library's own scratch array (esp_attn_forward_static) instead of a workspace."""
         if pool_blocks is not None:
             validate(params, tiles, trees, jobs, n_parts, n_rows, blocks, pool_blocks)
         self.params = params
+        self.static = static
         self.n_trees, self.n_tiles, self.n_jobs = len(trees), len(tiles), len(jobs)
         self.n_parts, self.n_rows = n_parts, n_rows
         self.trees = to_dev(np.ascontiguousarray(trees, dtype=abi.TREE_DT), device)
@@ -172,9 +184,14 @@ class DevicePass:
         self.desc = to_dev(np.ascontiguousarray(desc, dtype=np.int32), device) if desc is not None else None
         self.pos = to_dev(np.ascontiguousarray(pos, dtype=np.int32), device) if pos is not None else None
         nbytes = workspace_bytes(params, n_rows, n_parts)
-        self.workspace = torch.empty(nbytes, dtype=torch.uint8, device=device)
+        self.workspace = None if static else torch.empty(nbytes, dtype=torch.uint8, device=device)
 
     def run(self, Q, Kb, Vb, pool, O, stream=None, merge=True):
+        if self.static:
+            forward_static(self.params, Q, Kb, Vb, pool, self.blocks, self.desc, self.pos, O, self.tiles, self.n_tiles,
+                           self.trees, self.n_trees, self.jobs if merge else None, self.n_jobs if merge else 0, self.n_parts,
+                           self.n_rows, stream)
+            return
         forward(self.params, Q, Kb, Vb, pool, self.blocks, self.desc, self.pos, O, self.tiles, self.n_tiles, self.trees,
                 self.n_trees, self.jobs if merge else None, self.n_jobs if merge else 0, self.n_parts, self.n_rows,
                 self.workspace, stream)

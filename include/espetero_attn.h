@@ -118,8 +118,9 @@ typedef struct esp_attn_params {
                             rounding, its dots computed before the pass by esp_head_gate */
 } esp_attn_params;
 
-/* Library / device check and the per-device set-up: raises the dynamic LDS limit of every kernel
- * variant, so that the first launch of any variant may happen inside a stream capture. Safe to call more than once; a call that was not
+/* Library / device check and the per-device set-up: looks up this GPU's copy of the library's own
+ * device arrays and raises the dynamic LDS limit of every kernel variant, so that the first launch of
+ * any variant may happen inside a stream capture. Safe to call more than once; a call that was not
  * preceded by it does the same set-up on first use of a device. */
 int esp_attn_init(int device, char* err, size_t errlen);
 int esp_attn_abi_version(void);
@@ -164,6 +165,20 @@ int esp_attn_forward(const esp_attn_params* p, const void* Q, const void* Kb, co
                      int32_t n_tiles, const esp_tree* trees, int32_t n_trees, const esp_combine* jobs, int32_t n_jobs,
                      int32_t n_parts, int32_t n_rows, void* workspace, size_t workspace_bytes, void* stream, char* err,
                      size_t errlen);
+
+/* esp_attn_forward without a workspace and without any allocation: no counterpart in the reference
+ * (its encoder takes every buffer from the model's arena, forest.h:2716); it is for callers that
+ * cannot allocate device memory - code under HIP graph capture, tight serving loops, harnesses that
+ * forbid it. The partial records and the transposed batch V live in a device array of
+ * ESP_STATIC_SCRATCH_BYTES that the library holds on every GPU it runs on until the process ends; a
+ * pass that needs more (esp_attn_workspace_bytes) is refused with ESP_EWORKSPACE. Everything else as
+ * esp_attn_forward, same kernels, same results. Every call on a GPU shares that GPU's array: calls that
+ * overlap on one GPU (two streams, two threads) race; calls on one stream are ordered and safe. */
+#define ESP_STATIC_SCRATCH_BYTES ((size_t)32 << 20)
+int esp_attn_forward_static(const esp_attn_params* p, const void* Q, const void* Kb, const void* Vb, const void* kv_pool,
+                            const int32_t* blocks, const int32_t* desc, const int32_t* pos, void* O, const esp_tile* tiles,
+                            int32_t n_tiles, const esp_tree* trees, int32_t n_trees, const esp_combine* jobs, int32_t n_jobs,
+                            int32_t n_parts, int32_t n_rows, void* stream, char* err, size_t errlen);
 
 /* Host-side check of a pass's records before they are uploaded; no counterpart in the reference, whose
  * planner and kernels live in one program (forest.h:2646-2716). The kernels trust every index they

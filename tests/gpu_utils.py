@@ -32,16 +32,16 @@ def plan(case, options):
     return host.plan_tiles(case.trees, device.plan_hint(p)[1], p.window, case.pos if p.window > 0 else None, options)
 
 
-def run_case(case, options=None, pool=None, with_desc=True, two_step=False):
-    """Returns O as storage bits [n_rows][H * HD]. two_step: attention with the merge left out, then
-    esp_attn_combine as its own call."""
+def run_case(case, options=None, pool=None, with_desc=True, static=False, two_step=False):
+    """Returns O as storage bits [n_rows][H * HD]. static: through esp_attn_forward_static (the library's own
+    scratch array). two_step: attention with the merge left out, then esp_attn_combine as its own call."""
     device.init(0)
     options = options or default_options(case)
     tiles, jobs, n_parts = plan(case, options)
     if pool is None:
         pool = native_pool(case)
     dp = device.DevicePass(case.params, case.trees, tiles, jobs, n_parts, case.n_rows, case.blocks,
-                           case.desc if with_desc else None, case.pos, pool_blocks=case.n_blocks)
+                           case.desc if with_desc else None, case.pos, pool_blocks=case.n_blocks, static=static)
     Q, Kb, Vb = dev_u16(case.Q), dev_u16(case.Kb), dev_u16(case.Vb)
     O = torch.zeros_like(Q)
     dp.run(Q, Kb, Vb, pool, O, merge=not two_step)

@@ -169,3 +169,16 @@ def test_validate_accepts_a_planned_pass_and_names_the_first_bad_record():
     device.validate(p, tl, tr, jb, npart, 1, None, 12)
     with pytest.raises(abi.EspError, match="ring blocks"):
         device.validate(p, tl, tr, jb, npart, 1, None, 11)
+
+
+def test_forward_static_refuses_what_does_not_fit_its_scratch_array():
+    """The entry point without a workspace names its limit; checked on the host before any launch or device call."""
+    from espetero_amd import synth
+    lib = abi.attn_lib()
+    err = C.create_string_buffer(256)
+    p = synth.make_params(32, 5, 128, abi.ESP_F16, 16)
+    rc = lib.esp_attn_forward_static(C.byref(p), None, None, None, None, None, None, None, None, None, 1, None, 1, None, 0, 0, 1,
+                                     None, err, 256)
+    assert rc == 1 and b"multiple of Hkv" in err.value
+    p = synth.make_params(32, 4, 128, abi.ESP_F16, 16, rows_per_tile=4)
+    assert lib.esp_attn_workspace_bytes(C.byref(p), 32, 4096) > abi.ESP_STATIC_SCRATCH_BYTES
