@@ -718,7 +718,7 @@ class Ceilings:
         self.lib = C.CDLL(path)
         V, I = C.c_void_p, C.c_int32
         self.lib.esp_ceiling_hbm_read.argtypes = [V, V, I, I, I, I, V, V, V, V]
-        self.lib.esp_ceiling_mfma_issue.argtypes = [I, I, I, I, V, V, V, V]
+        self.lib.esp_ceiling_mfma_issue.argtypes = [I, I, I, I, I, V, V, V, V]
 
     def _events(self, n):
         t = self.torch
@@ -763,24 +763,27 @@ class Ceilings:
         t.cuda.empty_cache()
         return out
 
-    def mfma_issue(self, mixes=((0, 0), (2, 0), (4, 0), (0, 1), (1, 1), (2, 1), (3, 1), (4, 1)), iters=2000, workgroups=2 * N_CU):
+    def mfma_issue(self, mixes=((0, 0, 1), (0, 0, 0), (2, 1, 1), (4, 1, 1), (4, 1, 0)), iters=2000, workgroups=2 * N_CU):
         """TFLOP/s of v_mfma_f32_32x32x16_bf16 at two wavefronts per SIMD with (fp32 FMAs, v_exp_f32 + add) per
-        matrix instruction issued beside it; (0, 0) is the matrix cores alone, i.e. the clock they sustain."""
+        matrix instruction issued beside it, on random operands (what an attention pass feeds the multipliers) or on
+        constant ones. (0, 0, random) is the matrix cores alone on real data: the ceiling the prefill fractions are
+        also stated against."""
         t = self.torch
         outbuf = t.zeros(workgroups * 256, dtype=t.float32, device="cuda")
         st = self.C.c_void_p(t.cuda.current_stream().cuda_stream)
         flops = workgroups * 4 * iters * 32 * 32768
         out = []
-        for nv, ne in mixes:
+        for nv, ne, rnd in mixes:
             evs = self._events(5)
             for a, b in evs:
-                rc = self.lib.esp_ceiling_mfma_issue(nv, ne, workgroups, iters, self.C.c_void_p(outbuf.data_ptr()), st,
+                rc = self.lib.esp_ceiling_mfma_issue(nv, ne, rnd, workgroups, iters, self.C.c_void_p(outbuf.data_ptr()), st,
                                                      self.C.c_void_p(a.cuda_event), self.C.c_void_p(b.cuda_event))
                 assert rc == 0, rc
             t.cuda.synchronize()
             ms = np.array([a.elapsed_time(b) for a, b in evs][1:])
-            out.append({"valu_per_mfma": nv, "exp_per_mfma": ne, "TFLOPs": round(flops / float(np.median(ms)) / 1e9, 1),
-                        "cycles_per_mfma_at_2.4GHz": round(float(np.median(ms)) * 1e-3 * 2.4e9 / (iters * 32 * 2), 2)})
+            out.append({"valu_per_mfma": nv, "exp_per_mfma": ne, "operands": "random" if rnd else "constant",
+                        "TFLOPs": round(flops / float(np.median(ms)) / 1e9, 1),
+                        "ns_per_mfma_per_simd": round(float(np.median(ms)) * 1e6 / (iters * 32 * 2), 2)})
         return out
 
 

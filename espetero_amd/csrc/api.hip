@@ -198,12 +198,10 @@ int esp_attn_plan_hint(const esp_attn_params* p, int device, int32_t* workgroups
   hipError_t e = hipDeviceGetAttribute(&cus, hipDeviceAttributeMultiprocessorCount, device);
   if (e != hipSuccess) return hip_fail(err, errlen, "hipDeviceGetAttribute", e);
   const int fam = family(p);
-  // Streaming kernel: one resident round (its per-workgroup set-up is what a second round would
-  // pay again). Tiled kernel: two and a half rounds. Measured on 2048-row chunks of 40 heads: at
-  // 6K cached keys one and four rounds cost the same per step and 2.5 is 2 % faster; at 30K cached keys 2.5
-  // rounds are 14 % faster than unsplit tiles and 3 % faster than four rounds (every split tile writes and
-  // re-reads fp32 partial records).
-  *workgroups = fam > 0 ? cus * esp::stream_workgroups_per_cu(p->head_dim, fam) : cus * esp::tiled_workgroups_per_cu(p->head_dim) * 5 / 2;
+  // What is resident at once. The streaming kernel's planner splits a pass up to that many workgroups (a
+  // second round would pay its per-workgroup set-up again); the tiled kernel's planner hands the pass's
+  // workgroups to that many slots and picks the split that finishes earliest.
+  *workgroups = fam > 0 ? cus * esp::stream_workgroups_per_cu(p->head_dim, fam) : cus * esp::tiled_workgroups_per_cu(p->head_dim);
   *groups_per_tile = fam > 0 ? p->Hkv : p->H;
   *max_rows = esp::tiled_max_rows(p->head_dim);
   return ESP_OK;

@@ -45,6 +45,10 @@ namespace esp {
 template <int DT, int HD, int OCC>
 __global__ __launch_bounds__(256, OCC) void attn_tiled_kernel(const KArgs a, int n_tiles) {
   constexpr int KS = HD / 16, NT = HD / 32;
+  // Head dim 128 runs the softmax without a per-step maximum, in slices laid between the matrix instructions by
+  // hand (measured 3 % faster there); at head dim 256, with one wavefront per SIMD and every register taken,
+  // the same code spilled and ran 3 to 8 % slower than the form with a lazily moved maximum, which it keeps.
+  constexpr bool LEAN = HD == 128;
   constexpr int ROWB = HD * 2;     // bytes of one K row
   constexpr int CH = HD / 8;       // 16-byte chunks per K row
   constexpr int RPI = 64 / CH;     // K rows one load instruction covers
@@ -84,11 +88,19 @@ __global__ __launch_bounds__(256, OCC) void attn_tiled_kernel(const KArgs a, int
   const int rr = rr0 + m_row;
   const int4 d = a.desc ? a.desc[row] : make_int4(0, 0, 0, 0);
   const int qpos = a.window > 0 ? a.pos[row].x : 0;
+  // Q fragments; on the lean path multiplied once by scale * log2(e) and rounded back to the storage type:
+  // the matrix instructions then deliver scores in the log2 units the softmax works in, and no vector
+  // instruction per score is spent on the scale.
   u32x4 qf[KS];
   {
     const uint16_t* qp = a.Q + size_t(row) * a.q_ld + size_t(h) * HD + 8 * hb;
 #pragma unroll
-    for (int ks = 0; ks < KS; ++ks) qf[ks] = row_ok ? *reinterpret_cast<const u32x4*>(qp + 16 * ks) : u32x4{0, 0, 0, 0};
+    for (int ks = 0; ks < KS; ++ks) {
+      const u32x4 q = row_ok ? *reinterpret_cast<const u32x4*>(qp + 16 * ks) : u32x4{0, 0, 0, 0};
+#pragma unroll
+      for (int e = 0; e < 4; ++e)
+        qf[ks][e] = LEAN ? pack2<DT>(unpack_lo<DT>(q[e]) * a.scale_log2, unpack_hi<DT>(q[e]) * a.scale_log2) : q[e];
+    }
   }
 
   // ---- tile-wide facts about the rows (for the batch range and the no-mask fast path)
@@ -268,7 +280,13 @@ __global__ __launch_bounds__(256, OCC) void attn_tiled_kernel(const KArgs a, int
   auto lds_ptr = [](uint32_t addr) __attribute__((always_inline)) { return reinterpret_cast<lds_u32x4*>(addr); };
 
   f32x16 acc[NT];
-  float m_run = -INFINITY, l_run = 0.0f;  // l_run: this lane's share (16 of every 32 keys) of the row's sum
+  // The row's running reference m_run (log2 units; -inf: no key seen yet), kept a second time as 16
+  // registers of -m_run (0 while there is none): the block a score tile's first matrix instruction takes
+  // as its addend, so that the scores arrive already relative to the reference.
+  // l_run: this lane's share (16 of every 32 keys) of the row's sum. p_limit: what a half step's share
+  // of the sum may reach before the reference has to move (-1: it has to be set first).
+  // owed: what the reference moved by after the second half step's score tile had been started.
+  float m_run = -INFINITY, l_run = 0.0f, p_limit = -1.0f;
 #pragma unroll
   for (int nt = 0; nt < NT; ++nt)
 #pragma unroll
@@ -326,9 +344,20 @@ __global__ __launch_bounds__(256, OCC) void attn_tiled_kernel(const KArgs a, int
     }
   };
 
-  // Online softmax of half step (step, kt), first part: masks (cold path) and the running
-  // reference. Everything with a branch in it lives here, so that the second part is straight-line
-  // code the scheduler can lay between the matrix instructions of the next group.
+  // Online softmax of half step (step, kt) in three parts.
+  //   softmax_pre     the masks (nothing on the mask-free path); branchy.
+  //   softmax_exp     straight-line: P = exp2(S) - the scores are already relative to the reference - packed
+  //                   to the storage type, and the lane's share of the row sum, taken from the packed P two
+  //                   at a time (v_dot2: the sum is that of the rounded P the products use). No maximum is
+  //                   taken: all P >= 0, so a share <= 2^8 bounds every one of them, P fits its 16 bits and
+  //                   the accumulators need no rescaling. This is the code the scheduler lays between the
+  //                   matrix instructions of the next group: one v_exp and one and a half other vector
+  //                   instructions per score.
+  //   softmax_settle  almost never taken: some lane's share says the reference is too low (or not set: a
+  //                   row without one has p_limit = -1). Then the whole wavefront takes the half step's
+  //                   maximum, moves the reference, rescales what it has accumulated and redoes the half
+  //                   step's P. The two lanes of a row agree on the reference because both take the
+  //                   maximum over the pair.
   float corr_late = 1.0f;
   bool late = false;
   auto softmax_pre = [&](int step, auto kt_c, auto interior) __attribute__((always_inline)) {
@@ -391,33 +420,35 @@ __global__ __launch_bounds__(256, OCC) void attn_tiled_kernel(const KArgs a, int
         }
       }
     }
-    // Lazy rescale: the running reference m_run only moves when some lane's maximum exceeds
-    // it by more than 8 (log2 units), so P stays below 2^8 and the accumulators are rescaled
-    // a handful of times per row instead of once per step. The two lanes of a row agree on
-    // m_run because both take the maximum over the pair whenever either wants to move.
-    float x = -INFINITY;
+    if constexpr (!LEAN) {
+      // Lazy rescale: the running reference m_run only moves when some lane's maximum exceeds
+      // it by more than 8 (log2 units), so P stays below 2^8 and the accumulators are rescaled
+      // a handful of times per row instead of once per step. The two lanes of a row agree on
+      // m_run because both take the maximum over the pair whenever either wants to move.
+      float x = -INFINITY;
 #pragma unroll
-    for (int i = 0; i < 16; ++i) x = fmaxf(x, sv[i]);
-    x *= a.scale_log2;  // scale > 0: the max commutes with it
-    if (__any(x > m_run + 8.0f)) {
-      asm volatile("s_nop 0");  // a real branch: this block must not be speculated into the loop body
-      const float m_new = fmaxf(m_run, fmaxf(x, __shfl_xor(x, 32)));
-      const float corr = (m_new == -INFINITY) ? 1.0f : fast_exp2(m_run - m_new);
-      m_run = m_new;
-      l_run *= corr;
-      if constexpr (kt == 0) {
+      for (int i = 0; i < 16; ++i) x = fmaxf(x, sv[i]);
+      x *= a.scale_log2;  // scale > 0: the max commutes with it
+      if (__any(x > m_run + 8.0f)) {
+        asm volatile("s_nop 0");  // a real branch: this block must not be speculated into the loop body
+        const float m_new = fmaxf(m_run, fmaxf(x, __shfl_xor(x, 32)));
+        const float corr = (m_new == -INFINITY) ? 1.0f : fast_exp2(m_run - m_new);
+        m_run = m_new;
+        l_run *= corr;
+        if constexpr (kt == 0) {
 #pragma unroll
-        for (int nt = 0; nt < NT; ++nt) acc[nt] *= corr;
-      } else {
-        // P V of the first half step is still to be accumulated and its P is relative to the old
-        // reference: the accumulators take this factor once those products are in.
-        corr_late = corr;
-        late = true;
+          for (int nt = 0; nt < NT; ++nt) acc[nt] *= corr;
+        } else {
+          // P V of the first half step is still to be accumulated and its P is relative to the old
+          // reference: the accumulators take this factor once those products are in.
+          corr_late = corr;
+          late = true;
+        }
       }
     }
   };
-  // Second part: s[kt] -> pb[kt], the lane's share of the row sum.
-  auto softmax_exp = [&](auto kt_c) __attribute__((always_inline)) {
+  // Head dim 256: the straight-line part with the scale and the reference in one fused multiply-add per score.
+  auto softmax_exp_fma = [&](auto kt_c) __attribute__((always_inline)) {
     constexpr int kt = decltype(kt_c)::value;
     const float m_safe = (m_run == -INFINITY) ? 0.0f : m_run;
     float ps = 0.0f;
@@ -429,13 +460,72 @@ __global__ __launch_bounds__(256, OCC) void attn_tiled_kernel(const KArgs a, int
         p[e] = fast_exp2(__builtin_fmaf(s[kt][8 * t + e], a.scale_log2, -m_safe));
         ps += p[e];
       }
-      // keys 8 hb .. 8 hb + 7 of sub-block 2 kt + t
       pb[kt][t] = u32x4{pack2<DT>(p[0], p[1]), pack2<DT>(p[2], p[3]), pack2<DT>(p[4], p[5]), pack2<DT>(p[6], p[7])};
     }
     l_run += ps;
     // Pin the results here: without a use in this block the arithmetic above is sunk to the
     // block of its first real use, away from the matrix instructions it should overlap with.
     asm volatile("" : "+v"(pb[kt][0]), "+v"(pb[kt][1]), "+v"(l_run));
+  };
+  // The straight-line part in eight slices, one pair of scores each: slice q subtracts the reference and
+  // takes the exponentials of pair q, and packs and sums pair q - 1, whose exponentials have had a slice's
+  // time to come back. The caller lays the slices between the matrix instructions itself (the
+  // scheduler's grouping hints lumped them behind the first few); finish() packs and sums the last pair.
+  float pv[16], ps0 = 0.0f, ps1 = 0.0f, m_sub = 0.0f;
+  auto slice_pack = [&]<int KT, int Q>() __attribute__((always_inline)) {
+    uint32_t w = pack2<DT>(pv[2 * Q], pv[2 * Q + 1]);
+    asm volatile("" : "+v"(w));  // packed here, not sunk to the block of its first use
+    pb[KT][Q / 4][Q % 4] = w;
+    if constexpr (Q & 1) ps1 += pv[2 * Q] + pv[2 * Q + 1];
+    else ps0 += pv[2 * Q] + pv[2 * Q + 1];
+  };
+  auto slice = [&]<int KT, int Q>() __attribute__((always_inline)) {
+    if constexpr (Q == 0) {
+      ps0 = ps1 = 0.0f;
+      m_sub = (m_run == -INFINITY) ? 0.0f : m_run;
+    }
+    pv[2 * Q] = fast_exp2(s[KT][2 * Q] - m_sub);
+    pv[2 * Q + 1] = fast_exp2(s[KT][2 * Q + 1] - m_sub);
+    if constexpr (Q > 0) slice_pack.template operator()<KT, Q - 1>();
+  };
+  auto softmax_finish = [&]<int KT>() __attribute__((always_inline)) -> float {
+    slice_pack.template operator()<KT, 7>();
+    return ps0 + ps1;
+  };
+  // The whole straight-line part at once (the rare pass that redoes a half step).
+  auto softmax_exp = [&](auto kt_c) __attribute__((always_inline)) -> float {
+    constexpr int kt = decltype(kt_c)::value;
+    [&]<int... Q>(std::integer_sequence<int, Q...>) __attribute__((always_inline)) {
+      (slice.template operator()<kt, Q>(), ...);
+    }(std::make_integer_sequence<int, 8>{});
+    return softmax_finish.template operator()<kt>();
+  };
+  auto softmax_settle = [&](auto kt_c, float ps) __attribute__((always_inline)) {
+    constexpr int kt = decltype(kt_c)::value;
+    if (__any(!(ps <= p_limit))) {
+      asm volatile("s_nop 0");  // a real branch: this block must not be speculated into the loop body
+      f32x16& sv = s[kt];
+      mfma_settle(sv);  // the tile's last matrix instruction was issued in another block
+      float x = -INFINITY;
+#pragma unroll
+      for (int i = 0; i < 16; ++i) x = fmaxf(x, sv[i]);
+      const float m_new = fmaxf(m_run, fmaxf(x, __shfl_xor(x, 32)));
+      const float corr = (m_run == -INFINITY) ? 1.0f : fast_exp2(m_run - m_new);
+      m_run = m_new;
+      p_limit = (m_new == -INFINITY) ? -1.0f : 256.0f;
+      l_run *= corr;
+      if constexpr (kt == 0) {
+#pragma unroll
+        for (int nt = 0; nt < NT; ++nt) acc[nt] *= corr;
+      } else {
+        // P V of the first half step is still to be accumulated and its P is relative to the old
+        // reference: the accumulators take this factor once those products are in.
+        corr_late = late ? corr_late * corr : corr;
+        late = true;
+      }
+      ps = softmax_exp(kt_c);
+    }
+    l_run += ps;
   };
 
   // Phase G of a step: reads of group G + 1, matrix work of group G, and the softmax whose
@@ -447,20 +537,43 @@ __global__ __launch_bounds__(256, OCC) void attn_tiled_kernel(const KArgs a, int
     // issued instruction, a wait included, is time the matrix pipe idles.
     __builtin_amdgcn_s_waitcnt(G + 1 < NG ? kWaitLgkm8 : kWaitLgkm0);
     if constexpr (G == GK || G == 2 * GK) {
-      // The first matrix instructions of the group go out before the branchy part of the softmax,
-      // whose wait for the previous group's results they cover; the rest carry the arithmetic,
-      // one matrix instruction then its share.
-      constexpr int HEAD = 3;
-      mma_group.template operator()<G, 0, HEAD>(ring[G & 1]);
-      __builtin_amdgcn_sched_barrier(0);
-      softmax_pre(step, std::integral_constant<int, G == GK ? 0 : 1>{}, interior);
-      __builtin_amdgcn_sched_barrier(0);
-      mma_group.template operator()<G, HEAD, GP>(ring[G & 1]);
-      softmax_exp(std::integral_constant<int, G == GK ? 0 : 1>{});
+      if constexpr (LEAN) {
+        // On the mask-free path there is no branchy part and the whole group carries the arithmetic.
+        constexpr int HEAD = decltype(interior)::value ? 0 : 3;
+        mma_group.template operator()<G, 0, HEAD>(ring[G & 1]);
+        __builtin_amdgcn_sched_barrier(0);
+        softmax_pre(step, std::integral_constant<int, G == GK ? 0 : 1>{}, interior);
+        __builtin_amdgcn_sched_barrier(0);
+        // One matrix instruction, then its share of the eight slices, fenced so that the order stands.
+        constexpr int NM = GP - HEAD, KT = G == GK ? 0 : 1;
+        [&]<int... M>(std::integer_sequence<int, M...>) __attribute__((always_inline)) {
+          ([&]<int MI>() __attribute__((always_inline)) {
+            mma_group.template operator()<G, HEAD + MI, HEAD + MI + 1>(ring[G & 1]);
+            [&]<int... Q>(std::integer_sequence<int, Q...>) __attribute__((always_inline)) {
+              (slice.template operator()<KT, (8 * MI) / NM + Q>(), ...);
+            }(std::make_integer_sequence<int, (8 * (MI + 1)) / NM - (8 * MI) / NM>{});
+            __builtin_amdgcn_sched_barrier(0);
+          }.template operator()<M>(), ...);
+        }(std::make_integer_sequence<int, NM>{});
+        const float ps = softmax_finish.template operator()<KT>();
+        __builtin_amdgcn_sched_barrier(0);
+        softmax_settle(std::integral_constant<int, G == GK ? 0 : 1>{}, ps);
+      } else {
+        // The first matrix instructions of the group go out before the branchy part of the softmax,
+        // whose wait for the previous group's results they cover; the rest carry the arithmetic,
+        // one matrix instruction then its share.
+        constexpr int HEAD = 3;
+        mma_group.template operator()<G, 0, HEAD>(ring[G & 1]);
+        __builtin_amdgcn_sched_barrier(0);
+        softmax_pre(step, std::integral_constant<int, G == GK ? 0 : 1>{}, interior);
+        __builtin_amdgcn_sched_barrier(0);
+        mma_group.template operator()<G, HEAD, GP>(ring[G & 1]);
+        softmax_exp_fma(std::integral_constant<int, G == GK ? 0 : 1>{});
 #pragma unroll
-      for (int j = HEAD; j < GP; ++j) {
-        __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
-        __builtin_amdgcn_sched_group_barrier(0x002, 13, 0);
+        for (int j = HEAD; j < GP; ++j) {
+          __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
+          __builtin_amdgcn_sched_group_barrier(0x002, 13, 0);
+        }
       }
     } else {
       __builtin_amdgcn_sched_barrier(0);

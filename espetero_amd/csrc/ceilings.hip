@@ -57,9 +57,23 @@ __global__ __launch_bounds__(256, 2) void read_kernel(const char* __restrict__ b
 // independent fp32 fused multiply-adds and NE v_exp_f32, interleaved by the scheduler one matrix
 // instruction at a time. No memory, no LDS: what is left is the issue port the two kinds share.
 template <int NV, int NE>
-__global__ __launch_bounds__(256, 2) void issue_kernel(float* out, int iters, uint32_t seed) {
-  u32x4 a = {seed + threadIdx.x, seed * 3u, seed * 5u, seed * 7u};
-  u32x4 b = {seed ^ 0x3f803f80u, 0x3f803f80u, 0x3f803f80u, 0x3f803f80u};
+__global__ __launch_bounds__(256, 2) void issue_kernel(float* out, int iters, uint32_t seed, int random_data) {
+  // Operands as an attention pass has them: eight different A and four different B fragments of random
+  // 16-bit floats (sign and mantissa random, magnitude 0.25 .. 1), taken in turn. What the matrix cores
+  // reach depends on it: with constant operands the same loop runs at the full 2.4 GHz, with random ones
+  // the clock settles near 1.9 GHz under the power the multipliers then draw.
+  auto rnd = [&](uint32_t x) {
+    x = x * 2654435761u + seed;
+    x ^= x >> 15;
+    x *= 2246822519u;
+    x ^= x >> 13;
+    return random_data ? (x & 0x807f807fu) | 0x3e803e80u | ((x >> 3) & 0x01000100u) : 0x3f803f80u;
+  };
+  u32x4 a[8], b[4];
+#pragma unroll
+  for (int i = 0; i < 8; ++i) a[i] = u32x4{rnd(threadIdx.x + 64 * i), rnd(threadIdx.x + 64 * i + 1), rnd(threadIdx.x + 64 * i + 2), rnd(threadIdx.x + 64 * i + 3)};
+#pragma unroll
+  for (int i = 0; i < 4; ++i) b[i] = u32x4{rnd(threadIdx.x + 999 * i + 7), rnd(threadIdx.x + 999 * i + 8), rnd(threadIdx.x + 999 * i + 9), rnd(threadIdx.x + 999 * i + 10)};
   f32x16 c[4] = {};
   float v[16], x[8];
 #pragma unroll
@@ -69,7 +83,7 @@ __global__ __launch_bounds__(256, 2) void issue_kernel(float* out, int iters, ui
   for (int it = 0; it < iters; ++it) {
 #pragma unroll
     for (int j = 0; j < 32; ++j) {
-      c[j & 3] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(bf16x8, a), __builtin_bit_cast(bf16x8, b), c[j & 3], 0, 0, 0);
+      c[j & 3] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(bf16x8, a[j & 7]), __builtin_bit_cast(bf16x8, b[(j >> 3) & 3]), c[j & 3], 0, 0, 0);
 #pragma unroll
       for (int e = 0; e < NV; ++e) v[(j * NV + e) & 15] = __builtin_fmaf(v[(j * NV + e) & 15], 1.0001f, 0.5f);
 #pragma unroll
@@ -108,7 +122,7 @@ int esp_ceiling_hbm_read(const void* base, const int32_t* pages, int32_t n_pages
   return e == hipSuccess ? 0 : 3;
 }
 
-int esp_ceiling_mfma_issue(int32_t valu_per_mfma, int32_t exp_per_mfma, int32_t workgroups, int32_t iters, float* out, void* stream,
+int esp_ceiling_mfma_issue(int32_t valu_per_mfma, int32_t exp_per_mfma, int32_t random_data, int32_t workgroups, int32_t iters, float* out, void* stream,
                            void* start_event, void* stop_event) {
   if (!out || workgroups <= 0 || iters <= 0) return 1;
   const auto st = static_cast<hipStream_t>(stream);
@@ -117,18 +131,18 @@ int esp_ceiling_mfma_issue(int32_t valu_per_mfma, int32_t exp_per_mfma, int32_t 
   const int key = valu_per_mfma * 10 + exp_per_mfma;
   hipError_t e;
   switch (key) {
-    case 0: e = launch(issue_kernel<0, 0>, g, b, st, e0, e1, out, iters, 1u); break;
-    case 10: e = launch(issue_kernel<1, 0>, g, b, st, e0, e1, out, iters, 1u); break;
-    case 20: e = launch(issue_kernel<2, 0>, g, b, st, e0, e1, out, iters, 1u); break;
-    case 30: e = launch(issue_kernel<3, 0>, g, b, st, e0, e1, out, iters, 1u); break;
-    case 40: e = launch(issue_kernel<4, 0>, g, b, st, e0, e1, out, iters, 1u); break;
-    case 60: e = launch(issue_kernel<6, 0>, g, b, st, e0, e1, out, iters, 1u); break;
-    case 1: e = launch(issue_kernel<0, 1>, g, b, st, e0, e1, out, iters, 1u); break;
-    case 11: e = launch(issue_kernel<1, 1>, g, b, st, e0, e1, out, iters, 1u); break;
-    case 21: e = launch(issue_kernel<2, 1>, g, b, st, e0, e1, out, iters, 1u); break;
-    case 31: e = launch(issue_kernel<3, 1>, g, b, st, e0, e1, out, iters, 1u); break;
-    case 41: e = launch(issue_kernel<4, 1>, g, b, st, e0, e1, out, iters, 1u); break;
-    case 51: e = launch(issue_kernel<5, 1>, g, b, st, e0, e1, out, iters, 1u); break;
+    case 0: e = launch(issue_kernel<0, 0>, g, b, st, e0, e1, out, iters, 1u, random_data); break;
+    case 10: e = launch(issue_kernel<1, 0>, g, b, st, e0, e1, out, iters, 1u, random_data); break;
+    case 20: e = launch(issue_kernel<2, 0>, g, b, st, e0, e1, out, iters, 1u, random_data); break;
+    case 30: e = launch(issue_kernel<3, 0>, g, b, st, e0, e1, out, iters, 1u, random_data); break;
+    case 40: e = launch(issue_kernel<4, 0>, g, b, st, e0, e1, out, iters, 1u, random_data); break;
+    case 60: e = launch(issue_kernel<6, 0>, g, b, st, e0, e1, out, iters, 1u, random_data); break;
+    case 1: e = launch(issue_kernel<0, 1>, g, b, st, e0, e1, out, iters, 1u, random_data); break;
+    case 11: e = launch(issue_kernel<1, 1>, g, b, st, e0, e1, out, iters, 1u, random_data); break;
+    case 21: e = launch(issue_kernel<2, 1>, g, b, st, e0, e1, out, iters, 1u, random_data); break;
+    case 31: e = launch(issue_kernel<3, 1>, g, b, st, e0, e1, out, iters, 1u, random_data); break;
+    case 41: e = launch(issue_kernel<4, 1>, g, b, st, e0, e1, out, iters, 1u, random_data); break;
+    case 51: e = launch(issue_kernel<5, 1>, g, b, st, e0, e1, out, iters, 1u, random_data); break;
     default: return 2;
   }
   return e == hipSuccess ? 0 : 3;

@@ -80,6 +80,25 @@ __device__ __forceinline__ uint16_t pack1(float x) {
   }
 }
 
+// The two storage elements of a dword as fp32.
+template <int DT>
+__device__ __forceinline__ float unpack_lo(uint32_t w) {
+  if constexpr (DT == ESP_F16) return float(__builtin_bit_cast(f16x2, w)[0]);
+  else return __builtin_bit_cast(float, w << 16);
+}
+template <int DT>
+__device__ __forceinline__ float unpack_hi(uint32_t w) {
+  if constexpr (DT == ESP_F16) return float(__builtin_bit_cast(f16x2, w)[1]);
+  else return __builtin_bit_cast(float, w & 0xffff0000u);
+}
+
+// acc + the two storage elements of a dword, in fp32: one v_dot2 against (1, 1).
+template <int DT>
+__device__ __forceinline__ float sum2(uint32_t w, float acc) {
+  if constexpr (DT == ESP_F16) return __builtin_amdgcn_fdot2(__builtin_bit_cast(f16x2, w), __builtin_bit_cast(f16x2, 0x3c003c00u), acc, false);
+  else return __builtin_amdgcn_fdot2_f32_bf16(__builtin_bit_cast(bf16x2, w), __builtin_bit_cast(bf16x2, 0x3f803f80u), acc, false);
+}
+
 __device__ __forceinline__ float fast_exp2(float x) { return __builtin_amdgcn_exp2f(x); }
 
 // Lets the matrix pipeline finish writing `acc` before anything after this point reads it. Matrix

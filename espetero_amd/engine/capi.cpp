@@ -29,6 +29,8 @@ PlanOptions to_cpp(const esp_plan_options& o) {
   p.max_splits = o.max_splits;
   p.min_span = o.min_span;
   p.balanced = o.balanced != 0;
+  p.item_steps = o.item_steps;
+  p.part_steps = o.part_steps;
   return p;
 }
 void to_c(const PlanOptions& p, esp_plan_options* o) {
@@ -40,6 +42,8 @@ void to_c(const PlanOptions& p, esp_plan_options* o) {
   o->max_splits = p.max_splits;
   o->min_span = p.min_span;
   o->balanced = p.balanced ? 1 : 0;
+  o->item_steps = p.item_steps;
+  o->part_steps = p.part_steps;
 }
 template <class F>
 int guarded(F&& f) {

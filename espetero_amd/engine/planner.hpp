@@ -20,6 +20,8 @@
 #include <algorithm>
 #include <climits>
 #include <cstdint>
+#include <functional>
+#include <queue>
 #include <vector>
 
 #include "../../include/espetero_attn.h"
@@ -35,6 +37,12 @@ struct PlanOptions {
   int max_splits = 64;      // parts per tile group
   int min_span = 64;        // shorter cached ranges are not split
   bool balanced = false;    // false: reference rule; true: equal keys per workgroup
+  // Balanced rule on the tiled kernel (rows_per_tile > 32): groups_target is the number of workgroups
+  // resident at once, and the chunk is the one whose workgroups, handed to those slots in the kernel's
+  // dispatch order, finish earliest. item_steps: what a workgroup costs beside its key steps (set-up,
+  // epilogue), in steps of `granule` keys.
+  int item_steps = 0;
+  int part_steps = 0;  // what a split part costs on top: its partial record written, read again and merged
 
   static PlanOptions reference() { return PlanOptions{}; }
   // rows: query rows per tile (decode 1..8 -> 8-row budget is irrelevant; prefill 64/128).
@@ -52,6 +60,8 @@ struct PlanOptions {
       o.granule = 64;
       o.min_chunk = 512;
       o.min_span = 1024;
+      o.item_steps = 6;
+      o.part_steps = 16;
     }
     return o;
   }
@@ -98,16 +108,60 @@ inline void plan_tiles(AttnPlan& A, int groups, int window, const int32_t* pos, 
     }
   }
   const int n_tiles = int(rts.size());
-  const int budget = std::max(1, o.groups_target / std::max(1, groups * n_tiles));
+  int budget = std::max(1, o.groups_target / std::max(1, groups * n_tiles));
   int chunk_all = 0;  // balanced rule: keys per workgroup
-  if (o.balanced && budget > 1) {
+  auto parts_of = [&](const RowTile& rt, long long chunk) {
+    return rt.span >= o.min_span ? std::min<long long>((rt.span + rt.batch + chunk - 1) / chunk, o.max_splits) : 1;
+  };
+  if (o.balanced && o.item_steps > 0) {
+    // Tiled kernel. A pass is tiles x groups workgroups of unequal length (a causal chunk's later tiles
+    // see more keys) on groups_target slots; the hardware hands the next workgroup to the first free slot,
+    // in the kernel's dispatch order (tile records last to first, the groups of a record together). The
+    // time of the pass is when the last slot finishes, so the chunk is chosen by running that hand-out
+    // for every candidate: a few long workgroups leave slots idle at the end, many short ones pay their
+    // set-up, partial records and merge more often.
+    const int slots = std::max(1, o.groups_target);
+    long long max_work = 1;
+    for (const RowTile& rt : rts) max_work = std::max<long long>(max_work, rt.span + rt.batch);
+    const long long c_lo = std::max(1, o.min_chunk / o.granule), c_hi = (max_work + o.granule - 1) / o.granule;
+    auto finish_time = [&](long long chunk) {  // chunk 0: no tile is split
+      std::priority_queue<long long, std::vector<long long>, std::greater<long long>> free_at;
+      for (int i = 0; i < slots; ++i) free_at.push(0);
+      long long end = 0;
+      for (int i = n_tiles - 1; i >= 0; --i) {
+        const RowTile& rt = rts[size_t(i)];
+        const long long work = rt.span + rt.batch;
+        const long long ns = chunk > 0 ? parts_of(rt, chunk) : 1;
+        const long long per = (work + ns - 1) / ns;
+        for (long long p = ns - 1; p >= 0; --p) {  // a record's parts in reverse too
+          const long long keys = std::min(per, work - p * per);
+          const long long cost = o.item_steps + (ns > 1 ? o.part_steps : 0) + (std::max<long long>(keys, 0) + o.granule - 1) / o.granule;
+          for (int g = 0; g < groups; ++g) {
+            const long long t = free_at.top() + cost;
+            free_at.pop();
+            free_at.push(t);
+            end = std::max(end, t);
+          }
+        }
+      }
+      return end;
+    };
+    // Candidates: the chunks that cut the longest tile into 2 .. 8 parts (fewer parts first: ties keep them).
+    long long best = finish_time(0), best_chunk = 0;
+    for (int parts = 2; parts <= 8; ++parts) {
+      const long long c = std::max(c_lo, (c_hi + parts - 1) / parts);
+      const long long t = finish_time(c * o.granule);
+      if (t < best) best = t, best_chunk = c * o.granule;
+    }
+    chunk_all = int(best_chunk);
+    budget = best_chunk > 0 ? 2 : 1;
+  } else if (o.balanced && budget > 1) {
     // The smallest chunk (a granule multiple) whose tile count fits the target: a pass
     // that overshoots the resident workgroup count by a few tiles pays a whole extra round.
     const long long cap = std::max(1, o.groups_target / std::max(1, groups));
     auto tiles_at = [&](long long chunk) {
       long long n = 0;
-      for (const RowTile& rt : rts)
-        n += rt.span >= o.min_span ? std::min<long long>((rt.span + rt.batch + chunk - 1) / chunk, o.max_splits) : 1;
+      for (const RowTile& rt : rts) n += parts_of(rt, chunk);
       return n;
     };
     long long lo = std::max(1, o.min_chunk / o.granule), hi = std::max<long long>(lo, (total_span + o.granule - 1) / o.granule + 1);

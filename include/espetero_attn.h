@@ -127,14 +127,12 @@ int esp_attn_abi_version(void);
 
 /* What the planner needs to know about the kernel that serves these params
  * (rows_per_tile x G packed rows, head_dim, dtype):
- *   workgroups      how many workgroups a pass should be split up to: what is
- *                   resident at once for the streaming kernel (a second round
- *                   pays its per-workgroup set-up again), two and a half
- *                   rounds of that for the tiled kernel: enough to even out
- *                   tiles of unequal length, few enough that the partial
- *                   records of split tiles and their merge cost less than
- *                   the imbalance they remove (the reference aims at a fixed
- *                   256 threadgroups, forest.h:1385);
+ *   workgroups      how many workgroups of the kernel are resident at once: what the
+ *                   streaming kernel's pass is split up to (a second round pays its
+ *                   per-workgroup set-up again), and the slots the tiled kernel's
+ *                   planner hands its workgroups to when it picks the split that
+ *                   finishes earliest (the reference aims at a fixed 256
+ *                   threadgroups, forest.h:1385);
  *   groups_per_tile workgroups one tile becomes: KV heads for the streaming
  *                   kernel (the G heads of a KV head share a workgroup), query
  *                   heads for the tiled kernel (the reference: KV heads x SPLIT,

@@ -29,10 +29,13 @@ int esp_ceiling_hbm_read(const void* base, const int32_t* pages, int32_t n_pages
 /* The matrix cores under a wavefront that also issues vector arithmetic: every wavefront runs
  * iters x 32 v_mfma_f32_32x32x16_bf16 (four accumulator chains), and per matrix instruction
  * valu_per_mfma fp32 fused multiply-adds plus exp_per_mfma (v_exp_f32 + one add), no memory access.
+ * random_data: the matrix operands are random 16-bit floats, as an attention pass has them (1), or the
+ * constant 1.0 (0): the multipliers draw more power on random operands and the clock, and with it the
+ * ceiling, settles lower - the figure a kernel with real data can be held against is the one with 1.
  * Supported: exp_per_mfma 0 with valu_per_mfma 0, 1, 2, 3, 4, 6; exp_per_mfma 1 with 0 .. 5.
  * Workgroups of 4 wavefronts, at most two per compute unit. out: workgroups * 256 floats.
  * Flops of a launch: workgroups * 4 * iters * 32 * 32768. */
-int esp_ceiling_mfma_issue(int32_t valu_per_mfma, int32_t exp_per_mfma, int32_t workgroups, int32_t iters, float* out, void* stream,
+int esp_ceiling_mfma_issue(int32_t valu_per_mfma, int32_t exp_per_mfma, int32_t random_data, int32_t workgroups, int32_t iters, float* out, void* stream,
                            void* start_event, void* stop_event);
 
 #ifdef __cplusplus

@@ -36,11 +36,15 @@ typedef struct esp_plan_options {
   int32_t max_splits;    /* parts per tile group (64) */
   int32_t min_span;      /* shorter cached ranges are not split (64) */
   int32_t balanced;      /* 0: the reference's per-tree budget rule; 1: equal keys per workgroup */
+  int32_t item_steps;    /* balanced rule, tiled kernel (> 0): groups_target is the workgroups resident at once and the
+                            split chunk is the one whose workgroups finish earliest when handed to those slots in
+                            dispatch order; this is a workgroup's fixed cost in steps of `granule` keys */
+  int32_t part_steps;    /* the same rule: what a split part costs on top (its partial record and the merge) */
 } esp_plan_options;
 
 /* The reference's constants. */
 void esp_plan_options_reference(esp_plan_options* o);
-/* Tuned for 256 CUs: rows query rows per tile, workgroups the split target. */
+/* Tuned for 256 CUs: rows query rows per tile, workgroups what esp_attn_plan_hint reports for the kernel. */
 void esp_plan_options_mi355x(esp_plan_options* o, int32_t rows, int32_t workgroups);
 
 /* Plan a pass. trees[n_trees] in; tiles / jobs out (capacities given; on
