@@ -102,6 +102,13 @@ int esp_engine_slot_alloc(esp_engine* e) { return e->e.slot_alloc(); }
 int esp_engine_slot_free(esp_engine* e, int32_t s) { return guarded([&] { e->e.slot_free(s); }); }
 int esp_engine_slot_reset(esp_engine* e, int32_t s) { return guarded([&] { e->e.slot_reset(s); }); }
 int esp_engine_slot_fork(esp_engine* e, int32_t a, int32_t b) { return guarded([&] { e->e.slot_fork(a, b); }); }
+int esp_engine_slot_adopt(esp_engine* e, int32_t len, int32_t next_pos, int32_t n_blocks) {
+  try {
+    return e->e.slot_adopt(len, next_pos, n_blocks);
+  } catch (...) {
+    return -1;
+  }
+}
 int esp_engine_slot_len(const esp_engine* e, int32_t s) {
   try {
     const Slot& sl = e->e.slot(s);

@@ -118,13 +118,37 @@ class KvEngine {
       }
     return -1;
   }
+  // A slot that the pending pass reads or replaces may not be freed, emptied or overwritten under it: the
+  // commit would write the pass's block lists into a slot that is no longer the caller's.
+  bool in_pending_pass(int s) const {
+    if (!pass_.pending) return false;
+    for (const TreePlan& T : pass_.trees)
+      if (T.spec.parent == s || T.spec.save == s || T.spec.work == s) return true;
+    return false;
+  }
   void slot_free(int s) {
     Slot& sl = checked(s);
+    if (in_pending_pass(s)) fail("slot " + std::to_string(s) + " belongs to the pending pass (commit or abort it first)");
     release_blocks(sl);
     sl = Slot{};
   }
+  // A fresh slot holding `len` positions in `n_blocks` new blocks whose contents the caller brings in
+  // afterwards (a loaded checkpoint file: slot_load, src/model/model.mm:694-752). Returns the slot, -1 for
+  // counts that do not fit each other, -2 when the pool or the slot table has no room (the reference's codes).
+  int slot_adopt(int len, int next_pos, int n_blocks) {
+    if (len < 0 || n_blocks < 0 || next_pos < 0 || int64_t(len) > int64_t(n_blocks) * pool_.bt || len > max_ctx_) return -1;
+    if (pool_.n_free() < n_blocks) return -2;
+    const int s = slot_alloc();
+    if (s < 0) return -2;
+    Slot& sl = slots_[size_t(s)];
+    sl.len = len;
+    sl.next_pos = next_pos;
+    for (int i = 0; i < n_blocks; ++i) sl.blocks.push_back(pool_.alloc());
+    return s;
+  }
   void slot_reset(int s) {
     Slot& sl = checked(s);
+    if (in_pending_pass(s)) fail("slot " + std::to_string(s) + " belongs to the pending pass (commit or abort it first)");
     release_blocks(sl);
     sl.len = sl.next_pos = 0;
     sl.cm_k = 0;
@@ -135,6 +159,7 @@ class KvEngine {
     Slot& a = checked(src);
     Slot& b = checked(dst);
     if (src == dst) return;
+    if (in_pending_pass(dst)) fail("slot " + std::to_string(dst) + " belongs to the pending pass (commit or abort it first)");
     release_blocks(b);
     const size_t nb = std::min(size_t((a.len + pool_.bt - 1) / pool_.bt), a.blocks.size());
     b.blocks.assign(a.blocks.begin(), a.blocks.begin() + long(nb));
@@ -163,43 +188,60 @@ class KvEngine {
     sl.cm_k = 0;
   }
 
-  // Blocks Forest::target_blocks would allocate for one target (forest.h:1821-1829).
-  int target_new_blocks(const Slot* parent, int P, int w0, int end, bool in_place) const {
+  // ---- the block list of a slot that continues a parent's cached keys [0, P) and takes positions
+  // [w0, end) of this pass. Behaviour of the reference's Forest::target_blocks / target_new_blocks
+  // (src/model/impl/forest.h:1785-1829), arrived at by classifying every block index of the new list once:
+  //   Shared    lies wholly below w0: the parent's block, one more reference;
+  //   InPlace   holds parent positions and positions of this pass, the parent is the target itself and
+  //             nobody else references the block: kept, the pass appends into it;
+  //   Copied    holds parent positions but may not be written (another slot reads it, or the target is
+  //             another slot): a fresh block that first receives a copy of the parent's;
+  //   Fresh     beyond the parent's keys: a fresh block.
+  enum class BlockUse { Shared, InPlace, Copied, Fresh };
+  BlockUse classify(const std::vector<int>& parent_blocks, int P, int w0, bool in_place, int index) const {
     const int bt = pool_.bt;
-    const int i = w0 / bt;
-    int n = (end + bt - 1) / bt - i;
-    if (n > 0 && in_place && parent && i < int(parent->blocks.size()) && i * bt < P &&
-        pool_.ref[size_t(parent->blocks[size_t(i)])] == 1)
-      --n;
-    return std::max(n, 0);
+    if (index < w0 / bt) {
+      if (index >= int(parent_blocks.size())) fail("a slot's block list is shorter than its length");
+      return BlockUse::Shared;
+    }
+    const bool holds_parent_keys = index < int(parent_blocks.size()) && index * bt < P;
+    if (!holds_parent_keys) return BlockUse::Fresh;
+    return in_place && pool_.ref[size_t(parent_blocks[size_t(index)])] == 1 ? BlockUse::InPlace : BlockUse::Copied;
   }
-
-  // New block list of a target that continues `parent_blocks` (covering [0, P))
-  // and writes positions [w0, end) (forest.h:1785-1811).
+  // How many blocks the list would take from the free list.
+  int target_new_blocks(const Slot* parent, int P, int w0, int end, bool in_place) const {
+    static const std::vector<int> none;
+    const std::vector<int>& pb = parent ? parent->blocks : none;
+    int taken = 0;
+    for (int i = w0 / pool_.bt; i * pool_.bt < end; ++i) {
+      const BlockUse u = classify(pb, P, w0, in_place, i);
+      taken += u == BlockUse::Fresh || u == BlockUse::Copied;
+    }
+    return taken;
+  }
+  // The list itself; copies the pass has to run first are appended to `cow` as (source, destination).
   std::vector<int> target_blocks(const std::vector<int>& parent_blocks, int P, int w0, int end,
                                  std::vector<std::pair<int, int>>& cow, bool in_place) {
-    const int bt = pool_.bt;
-    std::vector<int> out;
-    const int keep = w0 / bt;  // blocks entirely below w0 are shared
-    for (int i = 0; i < keep && i < int(parent_blocks.size()); ++i) {
-      out.push_back(parent_blocks[size_t(i)]);
-      pool_.retain(parent_blocks[size_t(i)]);
-    }
-    const int need = (end + bt - 1) / bt;
-    for (int i = keep; i < need; ++i) {
-      const bool has_parent = i < int(parent_blocks.size()) && i * bt < P;
-      // An in-place append keeps a partial block it owns alone: the pass writes
-      // positions >= w0 there while attention reads positions < P.
-      if (has_parent && in_place && pool_.ref[size_t(parent_blocks[size_t(i)])] == 1) {
-        out.push_back(parent_blocks[size_t(i)]);
-        pool_.retain(parent_blocks[size_t(i)]);
-        continue;
+    std::vector<int> list;
+    for (int i = 0; i * pool_.bt < std::max(end, w0 / pool_.bt * pool_.bt); ++i) {
+      switch (classify(parent_blocks, P, w0, in_place, i)) {
+        case BlockUse::Shared:
+        case BlockUse::InPlace:
+          pool_.retain(parent_blocks[size_t(i)]);
+          list.push_back(parent_blocks[size_t(i)]);
+          break;
+        case BlockUse::Copied: {
+          const int fresh = pool_.alloc();
+          cow.emplace_back(parent_blocks[size_t(i)], fresh);
+          list.push_back(fresh);
+          break;
+        }
+        case BlockUse::Fresh:
+          list.push_back(pool_.alloc());
+          break;
       }
-      const int nb = pool_.alloc();
-      if (has_parent) cow.push_back({parent_blocks[size_t(i)], nb});  // it also holds parent positions
-      out.push_back(nb);
     }
-    return out;
+    return list;
   }
 
   int pass_blocks(const esp_tree_spec* specs, int n) const {
@@ -227,99 +269,138 @@ class KvEngine {
   };
   const Pass& pass() const { return pass_; }
 
+  // ---- what a pass can be refused for. Every check runs before anything is changed: a refused pass leaves the
+  // pool and every slot as they were (the reference's contract, src/model/api.h:283-285).
+  enum class Refusal {
+    PassPending, EmptyPass, BadSlot, BadLength, EmptyTree, SaveBeyondRoot, NothingToSave, WorkSlotClash, SlotTakenTwice,
+    ParentTaken, NoncausalShape, LeafArrays, LeafWithoutToken, ChainShape, ContextTooLong, PoolExhausted
+  };
+  struct PassRefused : EngineError {
+    Refusal why;
+    PassRefused(Refusal w, const std::string& m) : EngineError(m), why(w) {}
+  };
+  [[noreturn]] static void refuse(Refusal why, const std::string& message) { throw PassRefused(why, message); }
+
+  // Which rows the leaves of a verify tree need. A leaf whose tokens open another leaf's token list is not
+  // computed twice: its rows are the first rows of that longer leaf, its host (the reference hosts the same
+  // way, src/model/impl/forest.h:2201-2220: the longest leaf that starts with it, the earliest of equals).
+  // Leaves are visited longest first (earliest first among equals); a leaf is held up against the hosts
+  // found so far, in that order, so the first match is the longest and earliest, and a leaf no host starts
+  // with becomes a host itself. Rows are dealt to the hosts in leaf order.
+  struct LeafLayout {
+    std::vector<int> host, row0;  // per leaf: its host leaf; per host: first row among the tree's leaf rows
+    int rows = 0, longest = 0;
+  };
+  static LeafLayout lay_out_leaves(const esp_tree_spec& spec) {
+    const int n = spec.n_leaves;
+    LeafLayout lay;
+    if (n == 0) return lay;
+    if (!spec.leaf_offsets || !spec.leaf_tokens) refuse(Refusal::LeafArrays, "leaf arrays missing");
+    if (spec.leaf_offsets[0] != 0) refuse(Refusal::LeafArrays, "leaf offsets must start at 0");
+    auto length = [&](int i) { return spec.leaf_offsets[i + 1] - spec.leaf_offsets[i]; };
+    auto tokens = [&](int i) { return spec.leaf_tokens + spec.leaf_offsets[i]; };
+    std::vector<int> order(size_t(n), 0);
+    for (int i = 0; i < n; ++i) {
+      if (length(i) <= 0) refuse(Refusal::LeafWithoutToken, "every leaf needs a token");
+      lay.longest = std::max(lay.longest, length(i));
+      order[size_t(i)] = i;
+    }
+    std::stable_sort(order.begin(), order.end(), [&](int x, int y) { return length(x) > length(y); });
+    lay.host.assign(size_t(n), -1);
+    std::vector<int> hosts;
+    for (int leaf : order) {
+      int found = leaf;
+      for (int h : hosts)
+        if (std::equal(tokens(leaf), tokens(leaf) + length(leaf), tokens(h))) {
+          found = h;
+          break;
+        }
+      lay.host[size_t(leaf)] = found;
+      if (found == leaf) hosts.push_back(leaf);
+    }
+    lay.row0.assign(size_t(n), 0);
+    for (int i = 0; i < n; ++i)
+      if (lay.host[size_t(i)] == i) {
+        lay.row0[size_t(i)] = lay.rows;
+        lay.rows += length(i);
+      }
+    return lay;
+  }
+
+  // One tree of a pass, checked and sized against the slots as they are.
+  TreePlan size_tree(const esp_tree_spec& spec) const {
+    auto slot_or_none = [&](int s, const char* role) {
+      const bool none = s == -1, live = s >= 0 && s < int(slots_.size()) && slots_[size_t(s)].used;
+      if (!none && !live) refuse(Refusal::BadSlot, std::string("invalid ") + role + " slot " + std::to_string(s));
+    };
+    slot_or_none(spec.parent, "parent");
+    slot_or_none(spec.save, "save");
+    slot_or_none(spec.work, "work");
+    if (spec.root_len < 0 || spec.n_leaves < 0) refuse(Refusal::BadLength, "negative root or leaf count");
+    if (spec.root_len + spec.n_leaves == 0) refuse(Refusal::EmptyTree, "empty tree: neither root rows nor leaves");
+    TreePlan T;
+    T.spec = spec;
+    T.Tr = spec.root_len;
+    T.NL = spec.n_leaves;
+    T.save_len = spec.save_len > 0 ? spec.save_len : spec.root_len;
+    T.P = spec.parent >= 0 ? slots_[size_t(spec.parent)].len : 0;
+    if (T.save_len > T.Tr) refuse(Refusal::SaveBeyondRoot, "save_len exceeds root_len");
+    if (T.Tr == 0 && (spec.save >= 0 || spec.work >= 0))
+      refuse(Refusal::NothingToSave, "a tree without root rows has nothing to save (fork the slot instead)");
+    if (spec.work >= 0 && (spec.work == spec.save || spec.work == spec.parent))
+      refuse(Refusal::WorkSlotClash, "the work slot must differ from the save and parent slots");
+    if (spec.noncausal && (spec.parent >= 0 || spec.save >= 0 || spec.work >= 0 || T.NL > 0 || T.Tr == 0))
+      refuse(Refusal::NoncausalShape, "a noncausal tree is a root alone: no parent, save or work slot, no leaves");
+    const LeafLayout lay = lay_out_leaves(spec);
+    T.host = lay.host;
+    T.off = lay.row0;
+    if (spec.commit_chain > 0) {
+      // The rows of leaves 0 .. k-1 are kept as a chain the caller may commit later: leaf i is the first
+      // i + 1 tokens of leaf k-1, whose rows open the tree's leaf rows (forest.h:2223-2234).
+      const int k = spec.commit_chain;
+      if (k > T.NL) refuse(Refusal::ChainShape, "commit_chain names more leaves than the tree has");
+      const bool in_place_whole_root = spec.save >= 0 && spec.save == spec.parent && spec.work < 0 && T.save_len == T.Tr;
+      if (!in_place_whole_root) refuse(Refusal::ChainShape, "commit_chain needs a tree that appends its whole root to its own parent slot");
+      for (int i = 0; i < k; ++i)
+        if (spec.leaf_offsets[i + 1] - spec.leaf_offsets[i] != i + 1 || T.host[size_t(i)] != k - 1)
+          refuse(Refusal::ChainShape, "commit_chain: leaf " + std::to_string(i) + " is not the first " + std::to_string(i + 1) +
+                                          " tokens of leaf " + std::to_string(k - 1));
+      if (T.off[size_t(k - 1)] != 0) refuse(Refusal::ChainShape, "commit_chain: the chain's rows must open the leaf rows");
+      T.cm_k = k;
+    }
+    if (T.P + T.Tr + lay.longest > max_ctx_)
+      refuse(Refusal::ContextTooLong, "context " + std::to_string(T.P + T.Tr + lay.longest) + " exceeds max_ctx " + std::to_string(max_ctx_));
+    T.M = T.Tr + lay.rows;
+    return T;
+  }
+
   void pass_begin(const esp_tree_spec* specs, int n_trees) {
-    if (pass_.pending) fail("a pass is already pending (commit or abort it)");
-    if (n_trees <= 0 || !specs) fail("empty pass");
+    if (pass_.pending) refuse(Refusal::PassPending, "a pass is already pending (commit or abort it)");
+    if (n_trees <= 0 || !specs) refuse(Refusal::EmptyPass, "empty pass");
     Pass ps;
-    ps.trees.resize(size_t(n_trees));
-    const int n_user = int(slots_.size());
-    std::vector<int> saved(size_t(n_user), -1);
+    ps.trees.reserve(size_t(n_trees));
+    // Which tree writes each slot: a slot takes the result of at most one tree, and no tree may read a
+    // slot that another tree of the pass replaces.
+    std::vector<int> writer(slots_.size(), -1);
     int M = 0;
-    // ---- validation and sizes: nothing is modified until every tree passes
     for (int t = 0; t < n_trees; ++t) {
-      const esp_tree_spec& b = specs[t];
-      TreePlan& T = ps.trees[size_t(t)];
-      T.spec = b;
-      auto check_slot = [&](int s, const char* what) {
-        if (s < -1 || s >= n_user || (s >= 0 && !slots_[size_t(s)].used))
-          fail(std::string("invalid ") + what + " slot " + std::to_string(s));
-      };
-      check_slot(b.parent, "parent");
-      check_slot(b.save, "save");
-      check_slot(b.work, "work");
-      if (b.root_len < 0 || b.n_leaves < 0) fail("invalid lengths");
-      if (b.root_len == 0 && b.n_leaves == 0) fail("empty tree");
-      T.Tr = b.root_len;
-      T.save_len = b.save_len > 0 ? b.save_len : T.Tr;
-      if (T.save_len > T.Tr) fail("save_len exceeds root_len");
-      if (b.save >= 0 && T.Tr == 0) fail("nothing to save (use slot_fork)");
-      if (b.work >= 0) {
-        if (T.Tr == 0) fail("nothing to save in the work slot");
-        if (b.work == b.save || b.work == b.parent) fail("work slot must differ from save and parent slots");
-      }
-      T.P = b.parent >= 0 ? slots_[size_t(b.parent)].len : 0;
-      for (int s : {b.save, b.work}) {
-        if (s < 0) continue;
-        if (saved[size_t(s)] >= 0) fail("two trees save into one slot");
-        saved[size_t(s)] = t;
-      }
-      T.NL = b.n_leaves;
-      if (b.noncausal && (b.parent >= 0 || b.save >= 0 || b.work >= 0 || b.n_leaves > 0 || T.Tr == 0))
-        fail("noncausal: a root alone (no parent, save or work slot, leaves)");
-      int leaf_rows = 0, max_leaf = 0;
-      if (T.NL > 0) {
-        if (!b.leaf_offsets || !b.leaf_tokens) fail("leaf arrays missing");
-        if (b.leaf_offsets[0] != 0) fail("offsets must start at 0");
-        auto len_of = [&](int i) { return b.leaf_offsets[i + 1] - b.leaf_offsets[i]; };
-        for (int i = 0; i < T.NL; ++i) {
-          if (len_of(i) <= 0) fail("every leaf needs a token");
-          max_leaf = std::max(max_leaf, len_of(i));
+      TreePlan T = size_tree(specs[t]);
+      for (int s : {specs[t].save, specs[t].work})
+        if (s >= 0) {
+          if (writer[size_t(s)] >= 0) refuse(Refusal::SlotTakenTwice, "two trees save into one slot (" + std::to_string(s) + ")");
+          writer[size_t(s)] = t;
         }
-        // A leaf whose tokens are a prefix of another leaf is read from that leaf's rows.
-        T.host.assign(size_t(T.NL), -1);
-        T.off.assign(size_t(T.NL), 0);
-        for (int i = 0; i < T.NL; ++i) {
-          int h = i;
-          const int32_t* ti = b.leaf_tokens + b.leaf_offsets[i];
-          for (int j = 0; j < T.NL; ++j) {
-            if (j == i || len_of(j) < len_of(i)) continue;
-            if (len_of(j) == len_of(i) && j > i) continue;
-            if (len_of(j) < len_of(h) || (len_of(j) == len_of(h) && j >= h)) continue;
-            if (std::equal(ti, ti + len_of(i), b.leaf_tokens + b.leaf_offsets[j])) h = j;
-          }
-          T.host[size_t(i)] = h;
-        }
-        for (int i = 0; i < T.NL; ++i)
-          if (T.host[size_t(i)] == i) {
-            T.off[size_t(i)] = leaf_rows;
-            leaf_rows += len_of(i);
-          }
-        if (b.commit_chain > 0) {
-          const int kc = b.commit_chain;
-          if (kc > T.NL) fail("commit_chain exceeds the leaves");
-          if (b.save < 0 || b.save != b.parent || b.work >= 0 || T.save_len != T.Tr)
-            fail("commit_chain: in-place trees with a whole root only");
-          for (int i = 0; i < kc; ++i)
-            if (len_of(i) != i + 1 || T.host[size_t(i)] != kc - 1) fail("commit_chain: the leaves are not one chain");
-          if (T.off[size_t(kc - 1)] != 0) fail("commit_chain: the chain must be the first leaf rows");
-          T.cm_k = kc;
-        }
-      }
-      if (b.commit_chain > 0 && T.NL == 0) fail("commit_chain without leaves");
-      if (T.P + T.Tr + max_leaf > max_ctx_) fail("context exceeds max_ctx (" + std::to_string(max_ctx_) + ")");
-      T.M = T.Tr + leaf_rows;
       T.base = M;
       M += T.M;
+      ps.trees.push_back(std::move(T));
     }
     for (int t = 0; t < n_trees; ++t) {
       const int p = specs[t].parent;
-      if (p >= 0 && saved[size_t(p)] >= 0 && saved[size_t(p)] != t) fail("a tree saves into another tree's parent");
+      if (p >= 0 && writer[size_t(p)] >= 0 && writer[size_t(p)] != t)
+        refuse(Refusal::ParentTaken, "tree " + std::to_string(writer[size_t(p)]) + " saves into the parent slot of tree " + std::to_string(t));
     }
-    {
-      const int need = pass_blocks(specs, n_trees);
-      if (need > pool_.n_free())
-        fail("KV cache full: need " + std::to_string(need) + " blocks, " + std::to_string(pool_.n_free()) + " free");
-    }
+    if (const int need = pass_blocks(specs, n_trees); need > pool_.n_free())
+      refuse(Refusal::PoolExhausted, "KV cache full: the pass needs " + std::to_string(need) + " blocks, " + std::to_string(pool_.n_free()) + " are free");
 
     // ---- rows: descriptors and positions
     ps.M = M;

@@ -35,6 +35,7 @@ ENGINE_SYMBOLS = {
     "esp_engine_slot_free": (C.c_int, (_V, _I)),
     "esp_engine_slot_reset": (C.c_int, (_V, _I)),
     "esp_engine_slot_fork": (C.c_int, (_V, _I, _I)),
+    "esp_engine_slot_adopt": (C.c_int, (_V, _I, _I, _I)),
     "esp_engine_slot_len": (C.c_int, (_V, _I)),
     "esp_engine_slot_blocks": (C.c_int, (_V, _I, _V, _I)),
     "esp_engine_slot_next_pos": (C.c_int, (_V, _I)),
@@ -234,6 +235,10 @@ class Engine:
 
     def slot_fork(self, a, b):
         return self.lib.esp_engine_slot_fork(self.h, a, b)
+
+    def slot_adopt(self, length, next_pos, n_blocks):
+        """A fresh slot of `length` positions in n_blocks new blocks (a loaded checkpoint): the slot, -1 or -2."""
+        return self.lib.esp_engine_slot_adopt(self.h, length, next_pos, n_blocks)
 
     def slot_len(self, s):
         return self.lib.esp_engine_slot_len(self.h, s)

@@ -78,6 +78,12 @@ int esp_engine_slot_alloc(esp_engine* e);                 /* slot or -1 */
 int esp_engine_slot_free(esp_engine* e, int32_t slot);
 int esp_engine_slot_reset(esp_engine* e, int32_t slot);
 int esp_engine_slot_fork(esp_engine* e, int32_t src, int32_t dst);
+/* The engine side of slot_load (src/model/model.mm:694-752): a fresh slot of `len` positions (next rotary position
+ * next_pos) in n_blocks newly allocated blocks, for a caller that then brings the blocks' contents in
+ * (esp_slot_file_load + esp_kv_import_blocks into esp_engine_slot_blocks). Returns the slot, -1 when the counts
+ * do not fit each other (len > n_blocks * bt, or beyond max_ctx), -2 when the pool or the slot table has no room:
+ * the reference's return codes. Free, reset and fork of a slot that the pending pass reads or writes are refused. */
+int esp_engine_slot_adopt(esp_engine* e, int32_t len, int32_t next_pos, int32_t n_blocks);
 int esp_engine_slot_len(const esp_engine* e, int32_t slot);
 int esp_engine_slot_next_pos(const esp_engine* e, int32_t slot);        /* rotary position of the slot's next token */
 /* Verify-commit, the block-pool side of the reference's run_commit (src/model/impl/forest.h:4846-4861,

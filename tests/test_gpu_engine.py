@@ -287,3 +287,95 @@ def test_random_serving_histories(seed):
                     sv.accept(sp[1], int(rng.integers(0, sp[4] + 1)))
     assert n_passes >= 10
     sv.finish()
+
+
+@pytest.mark.parametrize("H,Hkv,HD,M,rows_per_tile,dtype", [
+    (4, 2, 128, 4, 4, abi.ESP_F16),      # streaming kernel: the root's rows packed into one column tile
+    (8, 1, 128, 3, 4, abi.ESP_BF16),     # 24 packed rows: two column tiles
+    (4, 2, 128, 150, 128, abi.ESP_BF16),  # tiled kernel, two row tiles
+    (4, 2, 256, 70, 128, abi.ESP_F16),
+    (2, 1, 512, 40, 64, abi.ESP_F16),
+])
+def test_noncausal_root_through_the_engine(H, Hkv, HD, M, rows_per_tile, dtype):
+    """A noncausal root (src/model/impl/forest.h:2402-2403; mask rule kernels/40_attention.metal:104-113, :220): the
+    engine describes every row as seeing the whole root, and both kernel families then give dense bidirectional
+    attention - held against the checker and against a float64 softmax that knows no mask."""
+    from gpu_utils import dev_u16, to_host_u16
+    device.init(0)
+    rng = np.random.default_rng(5)
+    e = host.Engine(8, 16, 2)
+    ps = e.pass_begin([host.make_spec(root_len=M, noncausal=1)])
+    assert ps["M"] == M and (ps["desc"][:, 2] == M).all()
+    ap = synth.make_params(H, Hkv, HD, dtype, 16, rows_per_tile=rows_per_tile)
+    bits = lambda w: ob.from_f32(rng.standard_normal((M, w)).astype(np.float32) * 0.5, dtype)  # noqa: E731
+    Q, Kb, Vb = bits(ap.q_ld), bits(ap.kv_ld), bits(ap.kv_ld)
+    resident, groups = device.plan_hint(ap)
+    tiles, jobs, n_parts = host.plan_tiles(ps["trees"], groups, 0, None, host.options_mi355x(rows_per_tile, resident))
+    blocks = np.zeros(1, np.int32)
+    pool = torch.zeros(8 * 2 * 16 * ap.kv_ld, dtype=torch.int16, device="cuda")
+    dp = device.DevicePass(ap, ps["trees"], tiles, jobs, n_parts, M, blocks, ps["desc"], ps["pos"], pool_blocks=8)
+    Qd = dev_u16(Q)
+    O = torch.zeros_like(Qd)
+    print(f"noncausal root: H={H} Hkv={Hkv} HD={HD} M={M} rows/tile={rows_per_tile} tiles={len(tiles)}", flush=True)
+    dp.run(Qd, dev_u16(Kb), dev_u16(Vb), pool, O)
+    torch.cuda.synchronize()
+    e.pass_abort()
+    got = f32(to_host_u16(O).reshape(M, -1), dtype).astype(np.float64)
+    want = ob.attn_direct(ap, Q, Kb, Vb, np.zeros(8 * 2 * 16 * ap.kv_ld, np.uint16), blocks, ps["desc"], ps["pos"], ps["trees"], n_threads=4)
+    tol = 2e-3 if dtype == abi.ESP_F16 else 4e-3
+    assert np.abs(got - f32(want, dtype)).max() <= tol
+    q = f32(Q, dtype).astype(np.float64).reshape(M, H, HD)
+    k = f32(Kb, dtype).astype(np.float64).reshape(M, Hkv, HD)
+    v = f32(Vb, dtype).astype(np.float64).reshape(M, Hkv, HD)
+    dense = np.zeros((M, H, HD))
+    for h in range(H):
+        s = q[:, h] @ k[:, h // (H // Hkv)].T * ap.scale
+        w = np.exp(s - s.max(axis=1, keepdims=True))
+        dense[:, h] = (w / w.sum(axis=1, keepdims=True)) @ v[:, h // (H // Hkv)]
+    assert np.abs(got - dense.reshape(M, -1)).max() <= tol
+
+
+def test_checkpoint_file_reloaded_through_slot_adopt_decodes_identically(tmp_path):
+    """save -> load -> decode through the engine (src/model/model.mm:629-752): a slot filled by a prefill pass is
+    exported to a checkpoint file, the file is loaded into a slot the engine adopts (fresh blocks, same length and
+    next position), and a decode step on the adopted slot gives the bits of the same step on the original."""
+    from gpu_utils import dev_u16, to_host_u16
+    sv = Served(8, 2, 128, 16, abi.ESP_F16, 64, 3, seed=17)
+    a, b, c = sv.slots
+    sv.e.slot_free(c)                                              # slot_adopt takes a free slot
+    sv.slots = [a, b]
+    assert sv.run([(-1, a, 77, [], 0)], 128, tag="prefill 77 rows into a")
+    ap, e = sv.ap, sv.e
+    blocks = e.slot_blocks(a)
+    nb, blk = len(blocks), 2 * ap.bt * ap.kv_ld
+    out = torch.zeros(1, nb, blk, dtype=torch.int16, device="cuda")
+    device.kv_export_blocks(ap, sv.pool, device.to_dev(blocks), nb, out[0])
+    torch.cuda.synchronize()
+    path = tmp_path / "a.ckpt"
+    host.slot_file_save(path, e.slot_len(a), e.slot_next_pos(a), 1, to_host_u16(out))
+    got = host.slot_file_load(path, ap.bt)
+    assert got is not None and got["len"] == 77
+    s = e.slot_adopt(got["len"], got["next_pos"], got["n_blocks"])
+    assert s == c and e.slot_len(s) == 77 and e.slot_next_pos(s) == e.slot_next_pos(a)
+    nblocks = e.slot_blocks(s)
+    assert not set(nblocks.tolist()) & set(blocks.tolist())
+    device.kv_import_blocks(ap, dev_u16(got["kv"].view(np.uint16).reshape(nb, blk)), device.to_dev(nblocks), nb, sv.pool)
+    torch.cuda.synchronize()
+    rng = np.random.default_rng(3)
+    bits = lambda w: ob.from_f32(rng.standard_normal((1, w)).astype(np.float32) * 0.5, ap.dtype)  # noqa: E731
+    Q, Kb, Vb = dev_u16(bits(ap.q_ld)), dev_u16(bits(ap.kv_ld)), dev_u16(bits(ap.kv_ld))
+    ap.rows_per_tile = 1
+    resident, groups = device.plan_hint(ap)
+    outs = []
+    for slot in (a, s):
+        ps = e.pass_begin([host.make_spec(parent=slot, save=slot, root_len=1)])
+        tiles, jobs, n_parts = host.plan_tiles(ps["trees"], groups, 0, None, host.options_mi355x(1, resident))
+        dp = device.DevicePass(ap, ps["trees"], tiles, jobs, n_parts, 1, ps["table"], ps["desc"], ps["pos"], pool_blocks=64)
+        O = torch.zeros_like(Q)
+        dp.run(Q, Kb, Vb, sv.pool, O)
+        device.kv_save(ap, Kb, Vb, sv.pool, device.to_dev(ps["saves"]), len(ps["saves"]))
+        torch.cuda.synchronize()
+        e.pass_commit()
+        outs.append(O)
+    assert torch.equal(outs[0], outs[1]) and bool(outs[0].any())
+    assert e.slot_len(a) == e.slot_len(s) == 78

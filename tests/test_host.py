@@ -550,3 +550,60 @@ def test_verify_commit_takes_the_kept_chain_rows_into_the_slot():
     e.chain_commit(a, 0)                                                # declining is always allowed
     assert e.slot_len(a) == 35
     _conservation(e, 16, [a, b, c])
+
+
+def test_slots_of_the_pending_pass_cannot_be_freed_reset_or_forked_over():
+    """Between pass_begin and commit / abort the pass's parent, save and work slots stay as they are: a commit would
+    otherwise write the pass's block lists into a slot the caller has given back."""
+    e = host.Engine(32, 16, 4)
+    a, b, c, d = (e.slot_alloc() for _ in range(4))
+    e.pass_begin([host.make_spec(save=a, root_len=20)])
+    e.pass_commit()
+    e.pass_begin([host.make_spec(parent=a, save=b, work=c, root_len=5)])
+    free = e.free_blocks()
+    for s in (a, b, c):
+        assert e.slot_free(s) != 0 and e.slot_reset(s) != 0, s
+    assert e.slot_fork(d, b) != 0          # b would be overwritten under the pass
+    assert e.slot_fork(a, d) == 0          # reading the parent into a slot outside the pass is fine
+    assert e.slot_reset(d) == 0
+    assert e.free_blocks() == free and e.slot_len(a) == 20
+    e.pass_commit()
+    assert e.slot_len(b) == 25 and e.slot_len(c) == 25
+    assert e.slot_free(b) == 0 and e.slot_free(c) == 0 and e.slot_free(a) == 0
+    assert e.free_blocks() == 32
+
+
+def test_slot_adopt_gives_a_loaded_checkpoint_its_slot_and_blocks():
+    """slot_load's engine side (src/model/model.mm:694-752): counts that do not fit -> -1, no room -> -2, else a slot
+    whose fresh blocks the caller fills; the slot then behaves like any other (decode appends in place)."""
+    e = host.Engine(10, 16, 2, max_ctx=1000)
+    assert e.slot_adopt(33, 33, 2) == -1           # 33 positions need 3 blocks
+    assert e.slot_adopt(2000, 2000, 200) == -1     # beyond max_ctx
+    assert e.slot_adopt(100, 100, 11) == -2        # the pool has 10 blocks
+    s = e.slot_adopt(33, 40, 3)
+    assert s >= 0 and e.slot_len(s) == 33 and e.slot_next_pos(s) == 40 and e.free_blocks() == 7
+    blocks = e.slot_blocks(s)
+    assert len(set(blocks.tolist())) == 3 and all(e.block_ref(int(b)) == 1 for b in blocks)
+    ps = e.pass_begin([host.make_spec(parent=s, save=s, root_len=1)])
+    assert ps["pos"][0, 0] == 40 and len(ps["cow"]) == 0 and ps["saves"][0]["block"] == blocks[2] and ps["saves"][0]["pos"] == 1
+    e.pass_commit()
+    t = e.slot_adopt(16, 16, 1)
+    assert t >= 0 and e.slot_adopt(1, 1, 1) == -2  # no slot left
+    e.slot_free(s)
+    e.slot_free(t)
+    assert e.free_blocks() == 10
+
+
+def test_noncausal_root_rows_are_described_as_seeing_the_whole_root():
+    """A noncausal root (the reference's pplx heads, src/model/impl/forest.h:2402-2403): every root row's descriptor
+    names the whole root as ancestors (anc_len = root_len), so row i also sees rows after it
+    (kernels/40_attention.metal:104-113). Such a tree is a root alone."""
+    e = host.Engine(8, 16, 2)
+    ps = e.pass_begin([host.make_spec(root_len=5, noncausal=1)])
+    assert ps["M"] == 5 and (ps["desc"][:, 2] == 5).all() and (ps["desc"][:, 0] == 0).all()
+    assert ps["pos"][:, 0].tolist() == [0, 1, 2, 3, 4]
+    e.pass_abort()
+    s = e.slot_alloc()
+    for bad in (dict(save=s), dict(parent=s), dict(leaves=[[1]])):
+        with pytest.raises(abi.EspError, match="noncausal"):
+            e.pass_begin([host.make_spec(root_len=5, noncausal=1, **bad)])

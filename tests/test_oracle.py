@@ -332,3 +332,28 @@ def test_kv_copy_blocks_copies_every_layer():
         r = pool[l * region:(l + 1) * region].reshape(4, blk2)
         b = before[l * region:(l + 1) * region].reshape(4, blk2)
         assert (r[3] == b[1]).all() and (r[2] == b[0]).all() and (r[:2] == b[:2]).all()
+
+
+def test_noncausal_root_is_full_bidirectional_attention(oracle):
+    """anc_len = root_len on every row (the reference's noncausal roots, src/model/impl/forest.h:2402-2403, mask rule
+    kernels/40_attention.metal:104-113): row i sees every row of the root, later ones included. Against a dense softmax
+    in float64 that knows no masks at all, and against the truth table of the rule."""
+    from espetero_amd import synth
+    from helpers import max_abs, oracle_direct, small_case
+    M = 7
+    c = small_case(seed=91, H=4, Hkv=2, seqs=((0, M),), rows_per_tile=8, desc_fn=lambda m: np.tile(np.array([0, 0, m, 0], np.int32), (m, 1)))
+    vis = oracle.visible_mask(c.params, c.trees[0], c.desc, c.pos)
+    assert vis.shape == (M, M) and vis.all()
+    p = c.params
+    q = oracle.to_f32(c.Q, p.dtype).astype(np.float64).reshape(M, p.H, p.head_dim)
+    k = oracle.to_f32(c.Kb, p.dtype).astype(np.float64).reshape(M, p.Hkv, p.head_dim)
+    v = oracle.to_f32(c.Vb, p.dtype).astype(np.float64).reshape(M, p.Hkv, p.head_dim)
+    want = np.zeros((M, p.H, p.head_dim))
+    for h in range(p.H):
+        s = q[:, h] @ k[:, h // 2].T * p.scale
+        w = np.exp(s - s.max(axis=1, keepdims=True))
+        want[:, h] = (w / w.sum(axis=1, keepdims=True)) @ v[:, h // 2]
+    assert max_abs(oracle_direct(c), want.reshape(M, -1), p.dtype) <= 2e-3
+    # with a cache in front: the cached keys and the whole root
+    c = small_case(seed=92, H=4, Hkv=2, seqs=((37, M),), rows_per_tile=8, desc_fn=lambda m: np.tile(np.array([0, 0, m, 0], np.int32), (m, 1)))
+    assert oracle.visible_mask(c.params, c.trees[0], c.desc, c.pos).all()
