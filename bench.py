@@ -275,6 +275,77 @@ class LayerMix:
             w.step(6 * i + l, ev[l] if ev else None)
 
 
+class DecodeStep:
+    """The attention part of one decode step of one layer, from the fp32 fused projection to O: esp_attn_prep (with
+    the folded append) followed by esp_attn_forward, or the two as the one call esp_attn_decode_fused."""
+
+    def __init__(self, w, kind, fused, seed=11):
+        import torch
+        from espetero_amd import device, synth
+        self.w, self.fused, self.torch, self.device = w, fused, torch, device
+        self.name = w.name + ("_step_fused" if fused else "_step")
+        n, bt = w.n_rows, w.bt
+        self.pp, a = synth.make_prep(kind, w.H, w.Hkv, w.HD, w.dtype, n, seed=seed, bt=bt)
+        dev = lambda x: None if x is None else torch.from_numpy(np.ascontiguousarray(x)).cuda()  # noqa: E731
+        g = torch.Generator(device="cuda")
+        g.manual_seed(seed)
+        self.X = [torch.randn(n, self.pp.x_ld, generator=g, device="cuda") * 1.5 for _ in range(min(4, w.n_sets))]
+        self.qn_w, self.kn_w = dev(a["qn_w"]), dev(a["kn_w"])
+        self.inv_freq, self.rope_sel, self.pos = dev(a["inv_freq"]), dev(a["rope_sel"]), dev(w.pos)
+        # each row's K / V go to entry P of its own sequence, in the blocks of the rotation set the step reads
+        self.tables = []
+        for blocks in w.tables:
+            t = np.full((n, 4), -1, np.int32)
+            for tr in w.trees:
+                P = int(tr["P"])
+                t[int(tr["base"]), :2] = blocks[int(tr["table"]) + P // bt], P % bt
+            self.tables.append(dev(t))
+        for dp in w.passes:   # the position array serves the prep too: every pass holds it, windowed or not
+            dp.pos = self.pos
+
+    def step(self, i, ev=None):
+        w, d = self.w, self.device
+        k = i % w.n_sets
+        dp, X = w.passes[k], self.X[i % len(self.X)]
+        if self.fused:
+            d.decode_fused(self.pp, w.params, X, self.qn_w, self.kn_w, self.pos, self.inv_freq, self.rope_sel, self.tables[k], w.pool, dp, w.O)
+        else:
+            d.attn_prep(self.pp, X, self.qn_w, self.kn_w, self.pos, self.inv_freq, self.rope_sel, w.Q, w.Kb, w.Vb, self.tables[k], w.pool, w.n_rows)
+            dp.run(w.Q, w.Kb, w.Vb, w.pool, w.O)
+
+
+def decode_step_fusion(args, torch):
+    """Step time of the attention part of a decode layer with and without the prep fused into the attention kernel:
+    eager wall time per step and the time per step of 16 steps replayed from one HIP graph."""
+    out = {"metric": "decode attention step, prep + attention", "unit": "us", "steps": args.steps, "warmup": args.warmup, "configs": {}}
+    for name, kind in (("c1_single_decode", "omni"), ("c2_batched_decode", "omni"), ("c4_decode_sliding", "gemma"), ("c4_decode_global", "gemma")):
+        w = make_workload(name, args.workgroups or None, args.tables == "contiguous", args.page)
+        rec = {}
+        outs = []
+        for fused in (False, True):
+            s = DecodeStep(w, kind, fused)
+            w.O.zero_()
+            s.step(0)
+            torch.cuda.synchronize()
+            outs.append(w.O.clone())
+            for i in range(args.warmup):
+                s.step(i)
+            torch.cuda.synchronize()
+            t0 = time.perf_counter()
+            for i in range(args.steps):
+                s.step(i)
+            torch.cuda.synchronize()
+            tag = "fused" if fused else "two_calls"
+            rec[tag + "_eager_us"] = round((time.perf_counter() - t0) / args.steps * 1e6, 2)
+            rec[tag + "_graph_us"] = graph_replay(s, torch).get("us_per_step")
+        rec["identical_output"] = bool(torch.equal(outs[0].view(torch.int16), outs[1].view(torch.int16)))
+        rec["dispatches"] = {"two_calls": 2 + (1 if w.n_parts else 0), "fused": 1 + (1 if w.n_parts else 0)}
+        out["configs"][name] = rec
+        del w
+        torch.cuda.empty_cache()
+    print(json.dumps(out), flush=True)
+
+
 def make_workload(name, workgroups=None, contiguous=False, page=16):
     from espetero_amd import abi, synth
     from functools import partial
@@ -866,7 +937,7 @@ def main():
     ap.add_argument("--warmup", type=int, default=20)
     ap.add_argument("--workload", default="all",
                     help="all (default): the batched decode as the headline, the chunked prefill, one record per benchmark "
-                         "configuration and the measured ceilings; or one of: hbm_read_ceiling, mfma_issue_ceiling, " + ", ".join(WORKLOADS))
+                         "configuration and the measured ceilings; or one of: hbm_read_ceiling, mfma_issue_ceiling, decode_step_fusion, " + ", ".join(WORKLOADS))
     ap.add_argument("--workgroups", type=int, default=0, help="planner split target (0: ask esp_attn_plan_hint)")
     ap.add_argument("--tables", default="scattered", choices=["scattered", "contiguous"],
                     help="block tables: a seeded permutation of the pool (the benchmark's definition) or address order")
@@ -891,6 +962,8 @@ def main():
         del src, dst
     if args.workload == "all":
         return run_all(args, torch)
+    if args.workload == "decode_step_fusion":
+        return decode_step_fusion(args, torch)
     if args.workload == "hbm_read_ceiling":
         print(json.dumps({"metric": "plain read GB/s", "unit": "GB/s", "peak": HBM_PEAK_GBS, "sizes": Ceilings().hbm_read()}), flush=True)
         return

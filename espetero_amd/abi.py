@@ -96,6 +96,8 @@ ATTN_SYMBOLS = {
     "esp_kv_import_blocks": (C.c_int, (_P, _V, _V, C.c_int32, _V, _V) + _ERR),
     "esp_chain_advance": (C.c_int, (_V, C.c_int32, _V, _V, _V, C.c_int32, C.c_int32, _V) + _ERR),
     "esp_head_gate": (C.c_int, (C.POINTER(GateParams), _V, _V, _V, _V, C.c_int32, _V) + _ERR),
+    "esp_attn_decode_fused": (C.c_int, (C.POINTER(PrepParams), _P, _V, _V, _V, _V, _V, _V, _V, _V, _V, _V, _V, _V, C.c_int32, _V, C.c_int32,
+                                        _V, C.c_int32, C.c_int32, C.c_int32, _V, C.c_size_t, _V) + _ERR),
     "esp_attn_prep": (C.c_int, (C.POINTER(PrepParams), _V, _V, _V, _V, _V, _V, _V, _V, _V, _V, _V, C.c_int32, _V) + _ERR),
 }
 

@@ -9,7 +9,7 @@
 #include "common.hpp"
 
 namespace esp {
-hipError_t launch_stream(int dt, int HD, int NC, const KArgs& a, int n_tiles, hipStream_t st);
+hipError_t launch_stream(int dt, int HD, int NC, const KArgs& a, const PrepArgs* pa, int n_tiles, hipStream_t st);
 hipError_t launch_combine(int dt, int HD, const KArgs& a, const esp_combine* jobs, int n_jobs, hipStream_t st);
 hipError_t launch_tiled(int dt, int HD, const KArgs& a, int n_tiles, hipStream_t st);
 hipError_t launch_kv_save(const esp_attn_params* p, const void* Kb, const void* Vb, void* pool, const esp_kvsave* e, int n,
@@ -218,7 +218,7 @@ static int forward_impl(const esp_attn_params* p, const void* Q, const void* Kb,
                         const int32_t* blocks, const int32_t* desc, const int32_t* pos, void* O, const esp_tile* tiles,
                         int32_t n_tiles, const esp_tree* trees, int32_t n_trees, const esp_combine* jobs, int32_t n_jobs,
                         int32_t n_parts, int32_t n_rows, void* workspace, size_t workspace_bytes, bool own_scratch,
-                        void* stream, char* err, size_t errlen) {
+                        const esp::PrepArgs* prep, void* stream, char* err, size_t errlen) {
   // A pending event pair belongs to this call whatever becomes of it: a call that launches nothing
   // must not leave it armed for some later launch.
   struct DropPair {
@@ -227,7 +227,7 @@ static int forward_impl(const esp_attn_params* p, const void* Q, const void* Kb,
   if (int rc = check_params(p, err, errlen)) return rc;
   if (n_tiles < 0 || n_trees < 0 || n_jobs < 0 || n_parts < 0 || n_rows < 0) return fail(err, errlen, ESP_EINVAL, "negative count");
   if (n_tiles == 0) return ESP_OK;
-  if (!Q || !Kb || !Vb || !O || !tiles || !trees) return fail(err, errlen, ESP_EINVAL, "Q, Kb, Vb, O, tiles, trees must not be NULL");
+  if ((!prep && (!Q || !Kb || !Vb)) || !O || !tiles || !trees) return fail(err, errlen, ESP_EINVAL, "Q, Kb, Vb, O, tiles, trees must not be NULL");
   if (n_trees == 0) return fail(err, errlen, ESP_EINVAL, "%d tiles without trees", n_tiles);
   if (!kv_pool) return fail(err, errlen, ESP_EINVAL, "kv_pool is NULL");
   if (!p->ring && !blocks) return fail(err, errlen, ESP_EINVAL, "blocks is NULL on a layer without rings");
@@ -271,7 +271,7 @@ static int forward_impl(const esp_attn_params* p, const void* Q, const void* Kb,
 
   hipError_t e;
   if (fam > 0) {
-    e = esp::launch_stream(p->dtype, p->head_dim, fam, a, n_tiles, st);
+    e = esp::launch_stream(p->dtype, p->head_dim, fam, a, prep, n_tiles, st);
     if (e != hipSuccess) return hip_fail(err, errlen, "attn_stream launch", e);
   } else {
     if (n_rows > 0) {
@@ -294,7 +294,7 @@ int esp_attn_forward(const esp_attn_params* p, const void* Q, const void* Kb, co
                      int32_t n_parts, int32_t n_rows, void* workspace, size_t workspace_bytes, void* stream, char* err,
                      size_t errlen) {
   return forward_impl(p, Q, Kb, Vb, kv_pool, blocks, desc, pos, O, tiles, n_tiles, trees, n_trees, jobs, n_jobs, n_parts, n_rows,
-                      workspace, workspace_bytes, false, stream, err, errlen);
+                      workspace, workspace_bytes, false, nullptr, stream, err, errlen);
 }
 
 int esp_attn_forward_static(const esp_attn_params* p, const void* Q, const void* Kb, const void* Vb, const void* kv_pool,
@@ -302,7 +302,7 @@ int esp_attn_forward_static(const esp_attn_params* p, const void* Q, const void*
                             int32_t n_tiles, const esp_tree* trees, int32_t n_trees, const esp_combine* jobs, int32_t n_jobs,
                             int32_t n_parts, int32_t n_rows, void* stream, char* err, size_t errlen) {
   return forward_impl(p, Q, Kb, Vb, kv_pool, blocks, desc, pos, O, tiles, n_tiles, trees, n_trees, jobs, n_jobs, n_parts, n_rows,
-                      nullptr, 0, true, stream, err, errlen);
+                      nullptr, 0, true, nullptr, stream, err, errlen);
 }
 
 int esp_attn_validate(const esp_attn_params* p, const esp_tile* tiles, int32_t n_tiles, const esp_tree* trees, int32_t n_trees,
@@ -511,9 +511,8 @@ int esp_head_gate(const esp_gate_params* p, void* O, const void* X, const void* 
   return ESP_OK;
 }
 
-int esp_attn_prep(const esp_prep_params* p, const float* X, const float* qn_w, const float* kn_w, const int32_t* pos,
-                  const float* inv_freq, const int32_t* rope_sel, void* Q, void* Kb, void* Vb, const int32_t* row_table,
-                  void* kv_pool, int32_t n_rows, void* stream, char* err, size_t errlen) {
+// Checks of esp_prep_params shared by esp_attn_prep and esp_attn_decode_fused.
+static int check_prep(const esp_prep_params* p, bool with_table, const void* kv_pool, char* err, size_t errlen) {
   if (!p) return fail(err, errlen, ESP_EINVAL, "params is NULL");
   if (p->H <= 0 || p->Hkv <= 0) return fail(err, errlen, ESP_EINVAL, "H=%d Hkv=%d", p->H, p->Hkv);
   if (p->head_dim != 128 && p->head_dim != 256 && p->head_dim != 512)
@@ -531,21 +530,53 @@ int esp_attn_prep(const esp_prep_params* p, const float* X, const float* qn_w, c
   const int rd = p->rope_dims, rd_min = HD == 512 ? 16 : 8;  // a lane holds 4 consecutive dims (8 at head_dim 512): half of rope_dims is a multiple of that
   if (rd < 0 || rd > HD || (rd != 0 && (rd < rd_min || (rd & (rd - 1)))))
     return fail(err, errlen, ESP_EINVAL, "rope_dims %d: 0 or a power of two in [%d, head_dim]", rd, rd_min);
-  if (n_rows < 0) return fail(err, errlen, ESP_EINVAL, "negative count");
-  if (n_rows == 0) return ESP_OK;
-  if (!X || !qn_w || !kn_w || !Q || !Kb || !Vb) return fail(err, errlen, ESP_EINVAL, "X, qn_w, kn_w, Q, Kb, Vb must not be NULL");
-  if (rd > 0 && (!pos || !inv_freq)) return fail(err, errlen, ESP_EINVAL, "pos and inv_freq must not be NULL when dims rotate");
-  if (row_table) {
+  if (with_table) {
     if (!kv_pool) return fail(err, errlen, ESP_EINVAL, "row_table without kv_pool");
     if (p->bt <= 0 || p->bt % 16) return fail(err, errlen, ESP_EINVAL, "bt %d: tokens per block must be a positive multiple of 16", p->bt);
     if (p->kv_base % 8) return fail(err, errlen, ESP_EINVAL, "kv_base must be a multiple of 8 elements");
   }
+  return ESP_OK;
+}
+
+int esp_attn_prep(const esp_prep_params* p, const float* X, const float* qn_w, const float* kn_w, const int32_t* pos,
+                  const float* inv_freq, const int32_t* rope_sel, void* Q, void* Kb, void* Vb, const int32_t* row_table,
+                  void* kv_pool, int32_t n_rows, void* stream, char* err, size_t errlen) {
+  if (int rc = check_prep(p, row_table != nullptr, kv_pool, err, errlen)) return rc;
+  if (n_rows < 0) return fail(err, errlen, ESP_EINVAL, "negative count");
+  if (n_rows == 0) return ESP_OK;
+  if (!X || !qn_w || !kn_w || !Q || !Kb || !Vb) return fail(err, errlen, ESP_EINVAL, "X, qn_w, kn_w, Q, Kb, Vb must not be NULL");
+  if (p->rope_dims > 0 && (!pos || !inv_freq)) return fail(err, errlen, ESP_EINVAL, "pos and inv_freq must not be NULL when dims rotate");
   esp::PrepArgs a{X, qn_w, kn_w, reinterpret_cast<const int4*>(pos), inv_freq, rope_sel, static_cast<uint16_t*>(Q),
                   static_cast<uint16_t*>(Kb), static_cast<uint16_t*>(Vb), reinterpret_cast<const int4*>(row_table),
                   static_cast<uint16_t*>(kv_pool), *p};
   const hipError_t e = esp::launch_attn_prep(a, n_rows, static_cast<hipStream_t>(stream));
   if (e != hipSuccess) return hip_fail(err, errlen, "attn_prep launch", e);
   return ESP_OK;
+}
+
+int esp_attn_decode_fused(const esp_prep_params* pp, const esp_attn_params* p, const float* X, const float* qn_w, const float* kn_w,
+                          const int32_t* pos, const float* inv_freq, const int32_t* rope_sel, const int32_t* row_table,
+                          void* kv_pool, const int32_t* blocks, const int32_t* desc, void* O, const esp_tile* tiles,
+                          int32_t n_tiles, const esp_tree* trees, int32_t n_trees, const esp_combine* jobs, int32_t n_jobs,
+                          int32_t n_parts, int32_t n_rows, void* workspace, size_t workspace_bytes, void* stream, char* err,
+                          size_t errlen) {
+  if (int rc = check_prep(pp, row_table != nullptr, kv_pool, err, errlen)) return rc;
+  if (int rc = check_params(p, err, errlen)) return rc;
+  if (pp->H != p->H || pp->Hkv != p->Hkv || pp->head_dim != p->head_dim || pp->dtype != p->dtype)
+    return fail(err, errlen, ESP_EINVAL, "the prep and the attention parameters name different heads, head dims or element types");
+  if (row_table && (pp->bt != p->bt || pp->kv_base != p->kv_base))
+    return fail(err, errlen, ESP_EINVAL, "the prep and the attention parameters name different pool regions or block sizes");
+  if (p->head_dim == 512) return fail(err, errlen, ESP_EUNSUPPORTED, "the fused decode serves head dims 128 and 256");
+  if (p->rows_per_tile <= 0 || p->rows_per_tile > 4 || family(p) <= 0)
+    return fail(err, errlen, ESP_EUNSUPPORTED, "rows_per_tile %d: the fused decode takes trees of 1 to 4 rows, one tile each, on the streaming kernel",
+                p->rows_per_tile);
+  if (n_tiles > 0 && (!X || !qn_w || !kn_w)) return fail(err, errlen, ESP_EINVAL, "X, qn_w, kn_w must not be NULL");
+  if (pp->rope_dims > 0 && (!pos || !inv_freq)) return fail(err, errlen, ESP_EINVAL, "pos and inv_freq must not be NULL when dims rotate");
+  if (!pos) return fail(err, errlen, ESP_EINVAL, "pos is NULL");
+  const esp::PrepArgs a{X, qn_w, kn_w, reinterpret_cast<const int4*>(pos), inv_freq, rope_sel, nullptr, nullptr, nullptr,
+                        reinterpret_cast<const int4*>(row_table), static_cast<uint16_t*>(kv_pool), *pp};
+  return forward_impl(p, nullptr, nullptr, nullptr, kv_pool, blocks, desc, pos, O, tiles, n_tiles, trees, n_trees, jobs, n_jobs, n_parts,
+                      n_rows, workspace, workspace_bytes, false, &a, stream, err, errlen);
 }
 
 }  // extern "C"

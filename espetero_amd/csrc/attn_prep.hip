@@ -27,6 +27,7 @@
 #include <type_traits>
 
 #include "common.hpp"
+#include "prep_math.hpp"
 
 namespace esp {
 
@@ -36,8 +37,8 @@ constexpr int kPrepRows = 8;
 template <int DT, int HD>
 __global__ __launch_bounds__(256) void attn_prep_kernel(const PrepArgs a, int n_rows) {
   constexpr int R = kPrepRows;
-  constexpr int EPL = HD > 256 ? 8 : 4;  // consecutive dims per lane: a head never spans more than one wavefront
-  constexpr int LPH = HD / EPL;          // lanes per head
+  constexpr int EPL = prep_epl(HD);  // consecutive dims per lane: a head never spans more than one wavefront
+  constexpr int LPH = HD / EPL;      // lanes per head
   constexpr int HPP = 256 / LPH;         // heads of the workgroup
   __shared__ float2 cs[R][HD / 2];       // (cos, sin) per row and frequency
   __shared__ int run_ok;
@@ -49,12 +50,7 @@ __global__ __launch_bounds__(256) void attn_prep_kernel(const PrepArgs a, int n_
   const int half = p.rope_dims / 2;
   for (int i = tid; i < rows * half; i += 256) {
     const int r = i / half, f = i % half;
-    const int4 pr = a.pos[row0 + r];
-    const int sel = a.rope_sel ? a.rope_sel[f] : 0;
-    const float position = float(sel == 0 ? pr.x : (sel == 1 ? pr.y : pr.z));
-    float sn, c;
-    sincosf(position * a.inv_freq[f], &sn, &c);
-    cs[r][f] = make_float2(c, sn);
+    cs[r][f] = prep_cos_sin(a.pos[row0 + r], a.rope_sel, a.inv_freq, f);
   }
   // Do the 8 rows go to positions ps0 .. ps0 + 7 (ps0 a multiple of 8) of one block, nowhere else?
   int4 ent[R];
@@ -91,33 +87,7 @@ __global__ __launch_bounds__(256) void attn_prep_kernel(const PrepArgs a, int n_
       float x[EPL];
 #pragma unroll
       for (int i = 0; i < EPL; ++i) x[i] = xv[r][i / 4][i % 4];
-      if (kind != 2 || p.v_norm) {
-        float ss = 0.0f;
-#pragma unroll
-        for (int i = 0; i < EPL; ++i) ss += x[i] * x[i];
-#pragma unroll
-        for (int o = LPH / 2; o >= 1; o >>= 1) ss += __shfl_xor(ss, o);
-        const float inv = rsqrtf(ss / float(HD) + p.eps);
-#pragma unroll
-        for (int i = 0; i < EPL; ++i) x[i] = kind == 2 ? x[i] * inv : x[i] * inv * w[i];
-      }
-      if (kind != 2 && half > 0) {
-        // The partner of dim d < half is d + half: half / EPL lanes away. Every lane of the head takes
-        // part in the exchange; only the rotating dims use it.
-        const bool lower = d0 < half;
-#pragma unroll
-        for (int i = 0; i < EPL; ++i) {
-          const float partner = __shfl_xor(x[i], half / EPL);
-          if (d0 < p.rope_dims) {
-            const float2 t = cs[r][(lower ? d0 : d0 - half) + i];
-            x[i] = lower ? x[i] * t.x - partner * t.y : x[i] * t.x + partner * t.y;
-          }
-        }
-      }
-      if (kind == 0) {
-#pragma unroll
-        for (int i = 0; i < EPL; ++i) x[i] *= p.q_scale;
-      }
+      prep_lane<HD>(x, kind, w, cs[r], p, d0);
       using out_t = std::conditional_t<EPL == 8, u32x4, u32x2>;  // EPL storage elements
       out_t out;
 #pragma unroll

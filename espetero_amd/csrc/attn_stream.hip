@@ -33,6 +33,7 @@
 #include <type_traits>
 
 #include "common.hpp"
+#include "prep_math.hpp"
 
 namespace esp {
 
@@ -103,13 +104,19 @@ struct Unit {  // operands of one unit of SBU 16-key sub-blocks
 // SBU: 16-key sub-blocks per unit (2: P.V on 16x16x32 tiles; 1: on 16x16x16 tiles, for
 // head dims whose operands would not fit two register sets otherwise).
 // BT: tokens per block when known at compile time (0: read from the arguments).
-template <int DT, int HD, int NC, int SBU, int BT, int OCC>
-__global__ __launch_bounds__(HD >= 512 ? 128 : 256, OCC) void attn_stream_kernel(const KArgs a) {
+// FUSED: the pass's rows come as the fp32 fused projection and the workgroup applies attn_prep to what it
+// needs of them itself (its tile's query heads; on the `last` tile the rows' key and value head of this KV
+// head, which it also appends to the pool): no prep dispatch in front, no Q / Kb / Vb round trip through
+// memory. For passes whose trees have at most rows_per_tile <= 4 rows (decode, short verify trees).
+template <int DT, int HD, int NC, int SBU, int BT, int OCC, int FUSED>
+__global__ __launch_bounds__(HD >= 512 ? 128 : 256, OCC) void attn_stream_kernel(const KArgs a, const PrepArgs pa) {
   constexpr bool PAIR = HD >= 512;      // two wavefronts per unit, HW dims each
   constexpr int HW = PAIR ? HD / 2 : HD;
   constexpr int NS = PAIR ? 1 : 4;       // unit streams of the workgroup
   constexpr int NW = PAIR ? 2 : 4;       // wavefronts of the workgroup
   static_assert(!PAIR || (NC == 1 && SBU == 1), "paired wavefronts: one column tile, 16-key units");
+  static_assert(!PAIR || !FUSED, "the fused prologue is built for one wavefront per head");
+  constexpr int kFusedRows = 4;  // most rows of a tile on the fused path
   constexpr int KK = HW / 32, MT = HW / 16, LDO = HD + 4, UK = 16 * SBU, USH = SBU == 2 ? 5 : 4;
   extern __shared__ float smem[];  // [NS][NC * 16 cols][LDO] O, then [NS][NC * 16][2] m, l, then (PAIR) [2][NW][64] partial S^T
 
@@ -130,6 +137,68 @@ __global__ __launch_bounds__(HD >= 512 ? 128 : 256, OCC) void attn_stream_kernel
   const int rows_live = min(a.R, end - tile.r0);
   const int rr0 = tile.r0 - tree.base;
 
+  // ---- fused prologue: attn_prep of this workgroup's heads into LDS (the area the final merge uses later),
+  // with the arithmetic and the lane arrangement of the prep kernel (prep_math.hpp), so the bits are its bits.
+  uint16_t* q_lds = reinterpret_cast<uint16_t*>(smem);   // [NC * 16 packed rows][HD]
+  uint16_t* k_lds = q_lds + NC * 16 * HD;                  // [kFusedRows][HD] this KV head's key rows
+  uint16_t* v_lds = k_lds + kFusedRows * HD;               // [kFusedRows][HD] and value rows
+  if constexpr (FUSED) {
+    constexpr int EPL = prep_epl(HD), LPH = HD / EPL, HPP = 256 / LPH;
+    float2* cs = reinterpret_cast<float2*>(v_lds + kFusedRows * HD);  // [kFusedRows][HD / 2]
+    const esp_prep_params& pp = pa.p;
+    const int half = pp.rope_dims / 2;
+    for (int i = threadIdx.x; i < rows_live * half; i += 256) {
+      const int r = i / half, f = i - r * half;
+      cs[r * (HD / 2) + f] = prep_cos_sin(pa.pos[tile.r0 + r], pa.rope_sel, pa.inv_freq, f);
+    }
+    __syncthreads();
+    const int n_q = rows_live * a.G, n_items = n_q + (tile.last ? 2 * rows_live : 0);
+    const int li = threadIdx.x % LPH, d0 = EPL * li;
+    for (int it = threadIdx.x / LPH; it < n_items; it += HPP) {
+      const int kind = it < n_q ? 0 : 1 + (it - n_q) / rows_live;
+      const int m = it < n_q ? it / a.G : (it - n_q) % rows_live;
+      const int h = it < n_q ? kvh * a.G + (it - m * a.G) : kvh;
+      const size_t row = size_t(tile.r0 + m);
+      const size_t col = size_t(kind == 0 ? pp.q_off + h * pp.q_hs : (kind == 1 ? pp.k_off : pp.v_off) + h * HD) + d0;
+      float x[EPL], w[EPL];
+#pragma unroll
+      for (int v = 0; v < EPL / 4; ++v) {
+        const f32x4 xv = *(reinterpret_cast<const f32x4*>(pa.X + row * pp.x_ld + col) + v);
+#pragma unroll
+        for (int i = 0; i < 4; ++i) x[4 * v + i] = xv[i];
+      }
+#pragma unroll
+      for (int i = 0; i < EPL; ++i) w[i] = kind != 2 ? (kind == 0 ? pa.qn_w : pa.kn_w)[d0 + i] : 1.0f;
+      prep_lane<HD>(x, kind, w, cs + m * (HD / 2), pp, d0);
+      using out_t = std::conditional_t<EPL == 8, u32x4, u32x2>;
+      out_t out;
+#pragma unroll
+      for (int i = 0; i < EPL / 2; ++i) out[i] = pack2<DT>(x[2 * i], x[2 * i + 1]);
+      uint16_t* dst = kind == 0 ? q_lds + it * HD : (kind == 1 ? k_lds : v_lds) + m * HD;
+      *reinterpret_cast<out_t*>(dst + d0) = out;
+      if (kind == 0 || !pa.row_table) continue;
+      // the folded append: the row's key and value of this KV head into its pool entries
+      const int4 ent = pa.row_table[row];
+#pragma unroll
+      for (int e = 0; e < 2; ++e) {
+        const int b = e ? ent.z : ent.x, ps = e ? ent.w : ent.y;
+        if (b < 0) continue;
+        uint16_t* hb = pa.pool + pp.kv_base + (size_t(b) * pp.Hkv + h) * size_t(2 * pp.bt * HD);
+        if (kind == 1) {
+          *reinterpret_cast<out_t*>(hb + size_t(ps) * HD + d0) = out;
+        } else {
+          uint16_t* vt = hb + vt_elem(pp.bt, HD, ps, d0);
+#pragma unroll
+          for (int i = 0; i < EPL / 2; ++i) {
+            vt[(2 * i) * kVtDim] = uint16_t(out[i] & 0xffffu);
+            vt[(2 * i + 1) * kVtDim] = uint16_t(out[i] >> 16);
+          }
+        }
+      }
+    }
+    __syncthreads();
+  }
+
   // ---- this lane's packed rows: Q fragments, position, descriptor
   u32x4 qf[NC][KK];
   int rr[NC], qpos[NC];
@@ -144,7 +213,8 @@ __global__ __launch_bounds__(HD >= 512 ? 128 : 256, OCC) void attn_stream_kernel
     const int row = ok[c] ? tile.r0 + m : tile.r0;
     qpos[c] = (a.window > 0) ? a.pos[row].x : 0;
     dsc[c] = a.desc ? a.desc[row] : make_int4(0, 0, 0, 0);
-    const uint16_t* qp = a.Q + size_t(row) * a.q_ld + size_t(kvh * a.G + (ok[c] ? hg : 0)) * HD + dw + 8 * q4;
+    const uint16_t* qp = FUSED ? q_lds + (ok[c] ? col : 0) * HD + dw + 8 * q4
+                               : a.Q + size_t(row) * a.q_ld + size_t(kvh * a.G + (ok[c] ? hg : 0)) * HD + dw + 8 * q4;
 #pragma unroll
     for (int kk = 0; kk < KK; ++kk)
       qf[c][kk] = ok[c] ? *reinterpret_cast<const u32x4*>(qp + 32 * kk) : u32x4{0, 0, 0, 0};
@@ -221,7 +291,9 @@ __global__ __launch_bounds__(HD >= 512 ? 128 : 256, OCC) void attn_stream_kernel
       const int js = j0 + 16 * sb;
       const int jk = js + c16;
       const bool k_ok = jk <= k_last;
-      const uint16_t* kp = a.Kb + size_t(tree.base + (k_ok ? jk : 0)) * a.kv_ld + size_t(kvh) * HD + dw + 8 * q4;
+      // fused: a tree's rows are its one tile's rows, prepared into LDS by the prologue
+      const uint16_t* kp = FUSED ? k_lds + (k_ok ? jk : 0) * HD + dw + 8 * q4
+                                 : a.Kb + size_t(tree.base + (k_ok ? jk : 0)) * a.kv_ld + size_t(kvh) * HD + dw + 8 * q4;
 #pragma unroll
       for (int kk = 0; kk < KK; ++kk)
         U.k[sb][kk] = k_ok ? *reinterpret_cast<const u32x4*>(kp + 32 * kk) : u32x4{0, 0, 0, 0};
@@ -231,7 +303,7 @@ __global__ __launch_bounds__(HD >= 512 ? 128 : 256, OCC) void attn_stream_kernel
 #pragma unroll
       for (int i = 0; i < 4; ++i) {
         if (jv + i > k_last) continue;
-        const uint16_t* vp = a.Vb + size_t(tree.base + jv + i) * a.kv_ld + size_t(kvh) * HD + dw + c16;
+        const uint16_t* vp = FUSED ? v_lds + (jv + i) * HD + dw + c16 : a.Vb + size_t(tree.base + jv + i) * a.kv_ld + size_t(kvh) * HD + dw + c16;
 #pragma unroll
         for (int mt = 0; mt < MT; ++mt) {
           const uint32_t e = uint32_t(vp[16 * mt]) << (16 * (i & 1));
@@ -551,17 +623,17 @@ constexpr int stream_occ(int HD, int NC) { return (HD == 128 && NC == 1) ? 2 : 1
 // Head dim 512: workgroups of two wavefronts, one per SIMD: two fill a compute unit.
 int stream_workgroups_per_cu(int HD, int NC) { return HD >= 512 ? 2 : stream_occ(HD, NC); }
 
-template <int DT, int HD, int NC>
-static hipError_t launch_stream_t(const KArgs& a, int n_tiles, hipStream_t st) {
+template <int DT, int HD, int NC, int FUSED>
+static hipError_t launch_stream_t(const KArgs& a, const PrepArgs& pa, int n_tiles, hipStream_t st) {
   constexpr int SBU = HD == 128 ? 2 : 1;  // 256 and 512 (256 dims per wavefront): 16-key units
   constexpr int OCC = stream_occ(HD, NC);
   const size_t smem = stream_smem_bytes(HD, NC);
-  constexpr auto k16 = attn_stream_kernel<DT, HD, NC, SBU, 16, OCC>;
-  constexpr auto kbt = attn_stream_kernel<DT, HD, NC, SBU, 0, OCC>;
+  constexpr auto k16 = attn_stream_kernel<DT, HD, NC, SBU, 16, OCC, FUSED>;
+  constexpr auto kbt = attn_stream_kernel<DT, HD, NC, SBU, 0, OCC, FUSED>;
   const auto k = a.bt == 16 ? k16 : kbt;
   const hipError_t e = a.bt == 16 ? allow_dynamic_lds<k16>(smem) : allow_dynamic_lds<kbt>(smem);
   if (e != hipSuccess) return e;
-  launch_timed(k, dim3(a.Hkv, n_tiles), dim3(HD >= 512 ? 128 : 256), smem, st, a);
+  launch_timed(k, dim3(a.Hkv, n_tiles), dim3(HD >= 512 ? 128 : 256), smem, st, a, pa);
   return hipGetLastError();
 }
 
@@ -570,8 +642,12 @@ static hipError_t stream_attributes_t() {
   constexpr int SBU = HD == 128 ? 2 : 1;
   constexpr int OCC = stream_occ(HD, NC);
   const size_t smem = stream_smem_bytes(HD, NC);
-  hipError_t e = allow_dynamic_lds<attn_stream_kernel<DT, HD, NC, SBU, 16, OCC>>(smem);
-  if (e == hipSuccess) e = allow_dynamic_lds<attn_stream_kernel<DT, HD, NC, SBU, 0, OCC>>(smem);
+  hipError_t e = allow_dynamic_lds<attn_stream_kernel<DT, HD, NC, SBU, 16, OCC, 0>>(smem);
+  if (e == hipSuccess) e = allow_dynamic_lds<attn_stream_kernel<DT, HD, NC, SBU, 0, OCC, 0>>(smem);
+  if constexpr (HD < 512) {
+    if (e == hipSuccess) e = allow_dynamic_lds<attn_stream_kernel<DT, HD, NC, SBU, 16, OCC, 1>>(smem);
+    if (e == hipSuccess) e = allow_dynamic_lds<attn_stream_kernel<DT, HD, NC, SBU, 0, OCC, 1>>(smem);
+  }
   return e;
 }
 
@@ -589,18 +665,23 @@ hipError_t stream_init_attributes() {
   return e;
 }
 
-// dt, HD, NC are validated by the caller: (HD, NC) in {(128, 1), (128, 2), (256, 1), (512, 1)}.
-hipError_t launch_stream(int dt, int HD, int NC, const KArgs& a, int n_tiles, hipStream_t st) {
-  if (dt == ESP_F16) {
-    if (HD == 128 && NC == 1) return launch_stream_t<ESP_F16, 128, 1>(a, n_tiles, st);
-    if (HD == 128 && NC == 2) return launch_stream_t<ESP_F16, 128, 2>(a, n_tiles, st);
-    if (HD == 256 && NC == 1) return launch_stream_t<ESP_F16, 256, 1>(a, n_tiles, st);
-    if (HD == 512 && NC == 1) return launch_stream_t<ESP_F16, 512, 1>(a, n_tiles, st);
-  } else {
-    if (HD == 128 && NC == 1) return launch_stream_t<ESP_BF16, 128, 1>(a, n_tiles, st);
-    if (HD == 128 && NC == 2) return launch_stream_t<ESP_BF16, 128, 2>(a, n_tiles, st);
-    if (HD == 256 && NC == 1) return launch_stream_t<ESP_BF16, 256, 1>(a, n_tiles, st);
-    if (HD == 512 && NC == 1) return launch_stream_t<ESP_BF16, 512, 1>(a, n_tiles, st);
+// dt, HD, NC are validated by the caller: (HD, NC) in {(128, 1), (128, 2), (256, 1), (512, 1)}; with a prep
+// argument block (the fused prologue) head dim 512 is not served.
+hipError_t launch_stream(int dt, int HD, int NC, const KArgs& a, const PrepArgs* pa, int n_tiles, hipStream_t st) {
+  static const PrepArgs none{};
+#define ESP_STREAM_CASE(D, H_, N_)                                                                   \
+  if (dt == D && HD == H_ && NC == N_)                                                               \
+    return pa ? launch_stream_t<D, H_, N_, 1>(a, *pa, n_tiles, st) : launch_stream_t<D, H_, N_, 0>(a, none, n_tiles, st);
+  ESP_STREAM_CASE(ESP_F16, 128, 1)
+  ESP_STREAM_CASE(ESP_F16, 128, 2)
+  ESP_STREAM_CASE(ESP_F16, 256, 1)
+  ESP_STREAM_CASE(ESP_BF16, 128, 1)
+  ESP_STREAM_CASE(ESP_BF16, 128, 2)
+  ESP_STREAM_CASE(ESP_BF16, 256, 1)
+#undef ESP_STREAM_CASE
+  if (HD == 512 && NC == 1 && !pa) {
+    if (dt == ESP_F16) return launch_stream_t<ESP_F16, 512, 1, 0>(a, none, n_tiles, st);
+    if (dt == ESP_BF16) return launch_stream_t<ESP_BF16, 512, 1, 0>(a, none, n_tiles, st);
   }
   return hipErrorInvalidValue;
 }

@@ -155,9 +155,13 @@ __host__ __device__ __forceinline__ size_t vt_elem(int bt, int HD, int t, int d)
 }
 
 // Block holding cached key j of a tree: its block list, or its slot's ring.
+// The block list is read through the constant address space: no kernel writes it, and a kernel that
+// stores to the pool (the fused prologue's append) would otherwise have to assume its stores reach the
+// list and fetch every entry with a vector load whose wait drains the key and value loads in flight.
 __device__ __forceinline__ int block_of(const KArgs& a, int table, int j) {
+  using const_i32 = const int32_t __attribute__((address_space(4)));
   const int bi = j / a.bt;
-  return a.ring ? table + bi % a.ring : a.blocks[table + bi];
+  return a.ring ? table + bi % a.ring : ((const_i32*)a.blocks)[table + bi];
 }
 
 // Everything the prep kernel reads (esp_attn_prep).

@@ -149,6 +149,16 @@ def attn_prep(params, X, qn_w, kn_w, pos, inv_freq, rope_sel, Q, Kb, Vb, row_tab
                                            _stream(stream), err, _ERRLEN), err)
 
 
+def decode_fused(pp, params, X, qn_w, kn_w, pos, inv_freq, rope_sel, row_table, pool, dp, O, stream=None):
+    """attn_prep fused into the attention of a decode / short verify pass. dp: the DevicePass holding the records."""
+    err = C.create_string_buffer(_ERRLEN)
+    ws = dp.workspace
+    abi.check(abi.attn_lib().esp_attn_decode_fused(
+        C.byref(pp), C.byref(params), _ptr(X), _ptr(qn_w), _ptr(kn_w), _ptr(pos), _ptr(inv_freq), _ptr(rope_sel), _ptr(row_table),
+        _ptr(pool), _ptr(dp.blocks), _ptr(dp.desc), _ptr(O), _ptr(dp.tiles), dp.n_tiles, _ptr(dp.trees), dp.n_trees, _ptr(dp.jobs),
+        dp.n_jobs, dp.n_parts, dp.n_rows, _ptr(ws), ws.numel() * ws.element_size(), _stream(stream), err, _ERRLEN), err)
+
+
 def head_gate(params, O, X, Wg, dots, n_rows, stream=None):
     """Device tensors. O (gated in place) or dots (fp32 [n_rows][H], written) may be None, not both."""
     err = C.create_string_buffer(_ERRLEN)

@@ -285,6 +285,23 @@ int esp_attn_prep(const esp_prep_params* p, const float* X, const float* qn_w, c
                   const float* inv_freq, const int32_t* rope_sel, void* Q, void* Kb, void* Vb, const int32_t* row_table,
                   void* kv_pool, int32_t n_rows, void* stream, char* err, size_t errlen);
 
+/* attn_prep fused into the attention of a decode or short verify pass: replaces the attn_prep dispatch in front
+ * of attn_decode_gqa / g4_attention_dec (the reference encodes the two one after the other, forest.h:4061-4078; its
+ * own fold of kv_save into attn_prep is 40_attention.metal:86-100). Every workgroup of the streaming kernel
+ * prepares what it needs itself from the fp32 projection X - the query heads of its tile, and on a tree's `last`
+ * tile the rows' key and value of its KV head, which it also appends to the pool through row_table - with the
+ * arithmetic of esp_attn_prep, bit for bit; Q, Kb and Vb are never written. Arguments as in esp_attn_prep
+ * (pp, X .. rope_sel, row_table, kv_pool) and esp_attn_forward (the rest); pos serves both. Limits: head dim 128
+ * or 256, rows_per_tile <= 4, packed rows within the streaming kernel's (rows_per_tile * G <= 32, <= 16 at head
+ * dim 256), and every tree of the pass at most rows_per_tile rows, i.e. one tile group per tree. O is what
+ * esp_attn_prep followed by esp_attn_forward gives, and so are the pool entries. */
+int esp_attn_decode_fused(const esp_prep_params* pp, const esp_attn_params* p, const float* X, const float* qn_w, const float* kn_w,
+                          const int32_t* pos, const float* inv_freq, const int32_t* rope_sel, const int32_t* row_table,
+                          void* kv_pool, const int32_t* blocks, const int32_t* desc, void* O, const esp_tile* tiles,
+                          int32_t n_tiles, const esp_tree* trees, int32_t n_trees, const esp_combine* jobs, int32_t n_jobs,
+                          int32_t n_parts, int32_t n_rows, void* workspace, size_t workspace_bytes, void* stream, char* err,
+                          size_t errlen);
+
 /* ---- decode chains ---------------------------------------------------------------
  * The reference runs K greedy decode steps as one GPU chain (run_chain,
  * src/model/model.mm:779-850, docs/design.md:226-243): the host encodes the K

@@ -106,6 +106,32 @@ def test_prep_gate_and_chain_argument_errors():
                                 None, 0, None, err, 256) == 1 and b"gate_headwise" in err.value
 
 
+def test_fused_decode_refuses_what_its_kernel_does_not_serve():
+    """esp_attn_decode_fused: prep and attention parameters must agree, head dim 512 and tiles of more than 4 rows are
+    refused with a message, all before any device call."""
+    from espetero_amd import synth
+    lib = abi.attn_lib()
+    err = C.create_string_buffer(256)
+
+    def call(pp, ap):
+        return lib.esp_attn_decode_fused(C.byref(pp), C.byref(ap), None, None, None, None, None, None, None, None, None, None, None,
+                                         None, 1, None, 1, None, 0, 0, 1, None, 0, None, err, 256)
+
+    pp, _ = synth.make_prep("omni", 8, 2, 128, abi.ESP_F16, 1)
+    ap = synth.make_params(8, 2, 128, abi.ESP_F16, 16, rows_per_tile=8)
+    assert call(pp, ap) == 2 and b"1 to 4 rows" in err.value
+    ap.rows_per_tile = 4
+    assert call(pp, ap) == 1 and b"X, qn_w, kn_w" in err.value
+    ap.Hkv, ap.kv_ld = 4, 512
+    assert call(pp, ap) == 1 and b"different heads" in err.value
+    pp, _ = synth.make_prep("gemma", 8, 1, 512, abi.ESP_F16, 1)
+    ap = synth.make_params(8, 1, 512, abi.ESP_F16, 16, rows_per_tile=1)
+    assert call(pp, ap) == 2 and b"128 and 256" in err.value
+    pp, _ = synth.make_prep("gemma", 32, 2, 256, abi.ESP_F16, 1)
+    ap = synth.make_params(32, 2, 256, abi.ESP_F16, 16, rows_per_tile=4)      # 4 rows x 16 heads per KV head: beyond the packed columns
+    assert call(pp, ap) == 2
+
+
 def _planned_pass():
     """A small decode + verify pass planned on the host: records as numpy arrays."""
     import numpy as np

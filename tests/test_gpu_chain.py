@@ -165,6 +165,19 @@ def test_device_chain_matches_the_checker_step_by_step_and_replays_identically(s
         assert np.array_equal(bits(Kg)[:(p + K) * ap.kv_ld].reshape(p + K, -1), kw)
         assert np.array_equal(bits(Vg)[:(p + K) * ap.kv_ld].reshape(p + K, -1), vw)
 
+    # the chain with attn_prep fused into the attention kernel (no prep dispatch, no Q / Kb / Vb in memory):
+    # the outputs and every pool byte of the three-dispatch chain, bit for bit
+    if ap.head_dim != 512:
+        eager_pool = st["pool"].clone()
+        reset()
+        for s in range(K):
+            device.decode_fused(pp, ap, Xd[s], qn, kn, st["pos"], inv_freq, sel, st["table"], st["pool"], dp, O[s])
+            device.chain_advance(st["trees"], n, st["pos"], st["table"], blocks_d, BT, ap.ring)
+        torch.cuda.synchronize()
+        assert torch.equal(O.view(torch.int16), eager.view(torch.int16)), "fused decode differs from prep + attention"
+        assert torch.equal(st["pool"].view(torch.int16), eager_pool.view(torch.int16)), "fused decode appended other bytes"
+        print("chain fused: identical outputs and pool", flush=True)
+
     # the same chain as one HIP graph, replayed with eager work and synchronisations in between
     reset()
     torch.cuda.synchronize()
@@ -180,3 +193,69 @@ def test_device_chain_matches_the_checker_step_by_step_and_replays_identically(s
         g.replay()
         got = check(f"graph replay {rep}")
         assert torch.equal(got.view(torch.int16), eager.view(torch.int16))
+
+
+@pytest.mark.parametrize("H,Hkv,HD,kind,dtype", [(8, 2, 128, "omni", abi.ESP_F16), (16, 2, 128, "qwen35x", abi.ESP_BF16),
+                                                 (4, 2, 256, "gemma", abi.ESP_F16), (8, 2, 256, "qwen35", abi.ESP_BF16)])
+def test_fused_prep_on_verify_trees_is_prep_then_attention_bit_for_bit(H, Hkv, HD, kind, dtype):
+    """Short verify trees (a root row and a chain of three drafts, 4 rows = one tile) and plain decode rows in one
+    pass: esp_attn_decode_fused against esp_attn_prep followed by esp_attn_forward, with the folded append, split
+    ranges and the merge. Outputs and pool bytes must be identical; the first is also held to the checker."""
+    kind = kind.rstrip("x")
+    device.init(0)
+    rng = np.random.default_rng(23)
+    BT = 16
+    seqs = [(700, 4), (33, 4), (2000, 1), (0, 3)]
+    n_rows = sum(m for _, m in seqs)
+    ap = synth.make_params(H, Hkv, HD, dtype, BT, rows_per_tile=4)
+    pp, a = synth.make_prep(kind, H, Hkv, HD, dtype, n_rows, seed=29, bt=BT)
+    if kind == "qwen35":          # the sigmoid gate beside each query in the projection (40_attention.metal:47, :334-342)
+        pass
+    nb = [(p + m + BT - 1) // BT for p, m in seqs]
+    n_blocks = sum(nb) + 2
+    perm = rng.permutation(n_blocks).astype(np.int32)
+    blocks = perm[:sum(nb)].copy()
+    trees = np.zeros(len(seqs), abi.TREE_DT)
+    desc = np.zeros((n_rows, 4), np.int32)
+    pos = np.zeros((n_rows, 4), np.int32)
+    table = np.full((n_rows, 4), -1, np.int32)
+    base = off = 0
+    for i, (p, m) in enumerate(seqs):
+        trees[i] = (base, p, off, m)
+        if m > 1:
+            desc[base:base + m] = synth.verify_desc(m, 1)
+        pos[base:base + m, :3] = (p + np.arange(m))[:, None]
+        tok = p + np.arange(m)
+        table[base:base + m, 0] = blocks[off + tok // BT]
+        table[base:base + m, 1] = tok % BT
+        base += m
+        off += nb[i]
+    tdt = torch.float16 if dtype == abi.ESP_F16 else torch.bfloat16
+    pool0 = (torch.randn(n_blocks * 2 * BT * ap.kv_ld, device="cuda") * 0.5).to(tdt)
+    resident, groups = device.plan_hint(ap)
+    tiles, jobs, n_parts = host.plan_tiles(trees, groups, 0, None, host.options_mi355x(4, 64))
+    assert n_parts > 0
+    dp = device.DevicePass(ap, trees, tiles, jobs, n_parts, n_rows, blocks, desc, pos, pool_blocks=n_blocks)
+    dev = lambda x: None if x is None else torch.from_numpy(np.ascontiguousarray(x)).cuda()  # noqa: E731
+    Xd, qn, kn, posd = dev(a["X"]), dev(a["qn_w"]), dev(a["kn_w"]), dev(pos)
+    inv_freq, sel, tabd = dev(a["inv_freq"]), dev(a["rope_sel"]), dev(table)
+    print(f"fused verify: H={H} Hkv={Hkv} HD={HD} {kind} tiles={len(tiles)} parts={n_parts}", flush=True)
+    outs, pools = [], []
+    for fused in (False, True):
+        pool = pool0.clone()
+        O = torch.zeros(n_rows, ap.q_ld, dtype=tdt, device="cuda")
+        if fused:
+            device.decode_fused(pp, ap, Xd, qn, kn, posd, inv_freq, sel, tabd, pool, dp, O)
+        else:
+            Q = torch.zeros(n_rows, ap.q_ld, dtype=tdt, device="cuda")
+            Kb = torch.zeros(n_rows, ap.kv_ld, dtype=tdt, device="cuda")
+            Vb = torch.zeros_like(Kb)
+            device.attn_prep(pp, Xd, qn, kn, posd, inv_freq, sel, Q, Kb, Vb, tabd, pool, n_rows)
+            dp.run(Q, Kb, Vb, pool, O)
+        torch.cuda.synchronize()
+        outs.append(O)
+        pools.append(pool)
+    assert bool(outs[0].any())
+    assert torch.equal(outs[0].view(torch.int16), outs[1].view(torch.int16)), "fused output differs"
+    assert torch.equal(pools[0].view(torch.int16), pools[1].view(torch.int16)), "fused append differs"
+    assert not torch.equal(pools[0].view(torch.int16), pool0.view(torch.int16))
