@@ -11,7 +11,7 @@ import pytest
 from espetero_amd import abi, host
 from oracle import binding as ob
 
-from helpers import GOLDEN, golden_names, load_golden_attention, tol_for
+from helpers import GOLDEN, beyond_rounding, golden_names, load_golden_attention, tol_for
 
 
 def test_the_fixture_set_is_complete():
@@ -24,7 +24,7 @@ def test_checker_direct_and_tiled_forms_match_the_fixture(name):
     c, want = load_golden_attention(name)
     p = c.params
     got = ob.to_f32(ob.attn_direct(p, c.Q, c.Kb, c.Vb, c.pool_ref, c.blocks, c.desc, c.pos, c.trees), p.dtype)
-    assert np.abs(got.reshape(want.shape) - want).max() <= tol_for(p.dtype)
+    assert beyond_rounding(got.reshape(want.shape), want, p.dtype, False) <= tol_for(p.dtype, unrounded=True)
     # the same through tiles, partial records and the merge, planned by the reference's rule and by the balanced one
     for o in (host.options_reference(), host.options_mi355x(p.rows_per_tile, 64)):
         rows = p.rows_per_tile
@@ -32,7 +32,7 @@ def test_checker_direct_and_tiled_forms_match_the_fixture(name):
         tiles, jobs, n_parts = host.plan_tiles(c.trees, p.Hkv, p.window, c.pos if p.window else None, o)
         got = ob.to_f32(ob.attn_tiles(p, c.Q, c.Kb, c.Vb, c.pool_ref, c.blocks, c.desc, c.pos, tiles, c.trees, jobs, n_parts), p.dtype)
         p.rows_per_tile = rows
-        assert np.abs(got.reshape(want.shape) - want).max() <= tol_for(p.dtype), (name, o.rows_per_tile)
+        assert beyond_rounding(got.reshape(want.shape), want, p.dtype, False) <= tol_for(p.dtype, unrounded=True), (name, o.rows_per_tile)
 
 
 @pytest.mark.parametrize("kind", golden_names("prep"))

@@ -11,6 +11,8 @@ import torch
 from espetero_amd import abi, device, host, synth
 from oracle import binding as ob
 
+from helpers import TOL, beyond_rounding
+
 pytestmark = pytest.mark.gpu
 
 
@@ -121,7 +123,7 @@ def test_c5_full_size_v_one_linearity_and_row0_equals_decode():
     # linearity in V: O(V) - O(V') depends on V - V' only through the same softmax weights;
     # with V' = 2 V the output doubles
     O2 = _f32(_run(w, Vb=w.Vb * 2, pool=_pool_with_v(w, None, scale=2.0)))
-    assert np.abs(O2 - 2 * O).max() <= 4e-3
+    assert np.abs(O2 - 2 * O).max() <= 2 * TOL   # two results, each within the bar
     # row 0 of every verify tree sees the cache + itself: equal to a decode pass of that row
     trees = w.trees.copy()
     trees["M"] = 1
@@ -186,7 +188,7 @@ def test_c3_chunked_prefill_equals_one_pass_and_brute_force_rows():
         device.kv_save(p, Kb, Vb, pool, device.to_dev(saves), len(saves))
     torch.cuda.synchronize()
     a, b = _f32(whole), _f32(chunked)
-    assert np.abs(a - b).max() <= 4e-3          # bf16 outputs: one rounding step each side
+    assert np.abs(a - b).max() <= 4e-3          # two bf16 computations: probabilities and outputs rounded on each side
     # sampled rows against float64 (K / V of the whole sequence are the batch rows themselves)
     q = _f32(Q).astype(np.float64).reshape(N, H, HD)
     k = _f32(Kb).astype(np.float64).reshape(N, Hkv, HD)
@@ -196,7 +198,7 @@ def test_c3_chunked_prefill_equals_one_pass_and_brute_force_rows():
             s_ = k[:r + 1, h // 5] @ q[r, h] * float(p.scale)
             e = np.exp(s_ - s_.max())
             want = (e / e.sum()) @ v[:r + 1, h // 5]
-            assert np.abs(b[r, h * HD:(h + 1) * HD] - want).max() <= 4e-3, (r, h)
+            assert beyond_rounding(b[r, h * HD:(h + 1) * HD], want, abi.ESP_BF16, False) <= TOL, (r, h)
     # what esp_kv_save wrote is what esp_kv_gather returns: bit exact
     Kg = torch.zeros(N * Hkv * HD, dtype=torch.bfloat16, device="cuda")
     Vg = torch.zeros_like(Kg)
