@@ -61,7 +61,7 @@ struct PlanOptions {
       o.min_chunk = 512;
       o.min_span = 1024;
       o.item_steps = 6;
-      o.part_steps = 16;
+      o.part_steps = 8;
     }
     return o;
   }
@@ -113,25 +113,26 @@ inline void plan_tiles(AttnPlan& A, int groups, int window, const int32_t* pos, 
   auto parts_of = [&](const RowTile& rt, long long chunk) {
     return rt.span >= o.min_span ? std::min<long long>((rt.span + rt.batch + chunk - 1) / chunk, o.max_splits) : 1;
   };
+  std::vector<int> ns_of;  // tiled kernel: parts of every row tile, once chosen
   if (o.balanced && o.item_steps > 0) {
     // Tiled kernel. A pass is tiles x groups workgroups of unequal length (a causal chunk's later tiles
     // see more keys) on groups_target slots; the hardware hands the next workgroup to the first free slot,
     // in the kernel's dispatch order (tile records last to first, the groups of a record together). The
-    // time of the pass is when the last slot finishes, so the chunk is chosen by running that hand-out
+    // time of the pass is when the last slot finishes, so the split is chosen by running that hand-out
     // for every candidate: a few long workgroups leave slots idle at the end, many short ones pay their
     // set-up, partial records and merge more often.
     const int slots = std::max(1, o.groups_target);
     long long max_work = 1;
     for (const RowTile& rt : rts) max_work = std::max<long long>(max_work, rt.span + rt.batch);
     const long long c_lo = std::max(1, o.min_chunk / o.granule), c_hi = (max_work + o.granule - 1) / o.granule;
-    auto finish_time = [&](long long chunk) {  // chunk 0: no tile is split
+    auto finish_time = [&](const std::vector<int>& ns_v) {
       std::priority_queue<long long, std::vector<long long>, std::greater<long long>> free_at;
       for (int i = 0; i < slots; ++i) free_at.push(0);
       long long end = 0;
       for (int i = n_tiles - 1; i >= 0; --i) {
         const RowTile& rt = rts[size_t(i)];
         const long long work = rt.span + rt.batch;
-        const long long ns = chunk > 0 ? parts_of(rt, chunk) : 1;
+        const long long ns = ns_v[size_t(i)];
         const long long per = (work + ns - 1) / ns;
         for (long long p = ns - 1; p >= 0; --p) {  // a record's parts in reverse too
           const long long keys = std::min(per, work - p * per);
@@ -146,15 +147,49 @@ inline void plan_tiles(AttnPlan& A, int groups, int window, const int32_t* pos, 
       }
       return end;
     };
-    // Candidates: the chunks that cut the longest tile into 2 .. 8 parts (fewer parts first: ties keep them).
-    long long best = finish_time(0), best_chunk = 0;
-    for (int parts = 2; parts <= 8; ++parts) {
-      const long long c = std::max(c_lo, (c_hi + parts - 1) / parts);
-      const long long t = finish_time(c * o.granule);
-      if (t < best) best = t, best_chunk = c * o.granule;
+    std::vector<int> cand(size_t(n_tiles), 1);
+    ns_of = cand;
+    long long best = finish_time(cand);
+    const long long items = 1LL * n_tiles * groups, rounds = items / slots;
+    // Fewer workgroups than slots: one chunk for every tile, the chunks that cut the longest tile into 2 .. 8
+    // parts (fewer parts first: ties keep them). With a round or more of whole workgroups such a split was
+    // measured slower than none (two workgroups share a compute unit and the older one is served first, so the
+    // slots are less alike than this hand-out takes them to be).
+    for (int parts = 2; parts <= 8 && rounds == 0; ++parts) {
+      const long long c = std::max(c_lo, (c_hi + parts - 1) / parts) * o.granule;
+      for (int i = 0; i < n_tiles; ++i) cand[size_t(i)] = int(parts_of(rts[size_t(i)], c));
+      const long long t = finish_time(cand);
+      if (t < best) best = t, ns_of = cand;
     }
-    chunk_all = int(best_chunk);
-    budget = best_chunk > 0 ? 2 : 1;
+    // A round or more, and some workgroups over (640 on 512 slots): those would run nearly alone at the end.
+    // Only the tiles with the least work are split, just enough of them that the whole ones fill whole rounds,
+    // and their parts fill the slots beside and behind those; the tile dispatched last gets the most parts, so
+    // that the pass ends on short workgroups. (Measured on 2048-row causal chunks over 2048 .. 6144 cached keys:
+    // 5 to 8 % faster than unsplit; splitting fewer tiles than that, so that some whole ones still spill into
+    // another round, was 3 to 6 % slower.)
+    if (rounds >= 1 && items % slots != 0) {
+      std::vector<int> order(size_t(n_tiles), 0);  // tiles by work, least first (ties: dispatched last first)
+      for (int i = 0; i < n_tiles; ++i) order[size_t(i)] = i;
+      std::stable_sort(order.begin(), order.end(), [&](int x, int y) {
+        return rts[size_t(x)].span + rts[size_t(x)].batch < rts[size_t(y)].span + rts[size_t(y)].batch;
+      });
+      const int n_tail = int((items - rounds * slots + groups - 1) / groups);
+      for (int most = 3; most <= 6; ++most) {  // parts of the tile with the least work; the others one fewer each, down to 2
+        std::fill(cand.begin(), cand.end(), 1);
+        bool any = false;
+        for (int j = 0; j < n_tail; ++j) {
+          const RowTile& rt = rts[size_t(order[size_t(j)])];
+          const long long cap = std::min<long long>((rt.span + rt.batch) / std::max(1, o.min_chunk), o.max_splits);
+          const int want = std::max(2, most - j);
+          const int ns = rt.span >= o.min_span ? int(std::min<long long>(want, cap)) : 1;
+          cand[size_t(order[size_t(j)])] = std::max(1, ns);
+          any = any || ns > 1;
+        }
+        if (!any) break;
+        const long long t = finish_time(cand);
+        if (t < best) best = t, ns_of = cand;
+      }
+    }
   } else if (o.balanced && budget > 1) {
     // The smallest chunk (a granule multiple) whose tile count fits the target: a pass
     // that overshoots the resident workgroup count by a few tiles pays a whole extra round.
@@ -176,7 +211,9 @@ inline void plan_tiles(AttnPlan& A, int groups, int window, const int32_t* pos, 
     const esp_tree& t = A.trees[size_t(rt.tree)];
     const int span = rt.span;
     int ns = 1;
-    if (budget > 1 && span >= o.min_span) {
+    if (!ns_of.empty()) {
+      ns = ns_of[size_t(&rt - rts.data())];
+    } else if (budget > 1 && span >= o.min_span) {
       if (o.balanced) {
         ns = std::min((span + rt.batch + chunk_all - 1) / chunk_all, o.max_splits);
       } else if (o.split > 0) {

@@ -121,6 +121,60 @@ def test_split_algebra_holds_for_both_rules(seed):
         assert seen == parts
 
 
+@pytest.mark.parametrize("seed", range(8))
+def test_tiled_kernel_plans_partition_every_tile(seed):
+    """The balanced rule for 128-row tiles (chosen by simulating the hand-out of workgroups to slots): whatever it
+    picks - no split, one chunk for all tiles, or only the shortest tiles cut - the ranges of a tile partition
+    [0, P), the last part owns the batch keys, parts are numbered in record order and every merge job names them."""
+    rng = np.random.default_rng(900 + seed)
+    n = int(rng.integers(1, 5))
+    trees, base = [], 0
+    for _ in range(n):
+        P, m = int(rng.integers(0, 40) * 256), int(rng.integers(1, 2500))
+        trees.append((base, P, 0, m))
+        base += m
+    groups, slots = int(rng.choice([8, 16, 40])), int(rng.choice([256, 512]))
+    o = host.options_mi355x(128, slots)
+    tiles, jobs, parts = host.plan_tiles(np.array(trees, abi.TREE_DT), groups, 0, None, o)
+    by = {}
+    for x in tiles:
+        by.setdefault((int(x["tree"]), int(x["r0"])), []).append(x)
+    assert set(by) == {(ti, b + r) for ti, (b, P, _, m) in enumerate(trees) for r in range(0, m, 128)}
+    numbered = []
+    for (ti, r0), xs in by.items():
+        P = trees[ti][1]
+        k = 0
+        for i, x in enumerate(xs):
+            assert int(x["k0"]) == k and (int(x["k1"]) > k or P == k)
+            assert int(x["k0"]) % o.granule == 0
+            k = int(x["k1"])
+            assert int(x["last"]) == (1 if i == len(xs) - 1 else 0)
+            assert (int(x["part"]) == -1) == (len(xs) == 1)
+            if len(xs) > 1:
+                numbered.append(int(x["part"]))
+        assert k == P
+    assert numbered == list(range(parts))          # in record order, which is the order the kernel's grid reverses
+    assert sum(int(j["nparts"]) for j in jobs) == parts and all(int(j["nparts"]) >= 2 for j in jobs)
+
+
+def test_a_round_and_a_quarter_of_workgroups_is_cut_at_its_short_end():
+    """A 2048-row causal chunk over 6144 cached keys, 40 workgroups per tile, 512 slots: 640 workgroups. Unsplit,
+    128 of them would run after the first 512, nearly alone. The plan cuts the 4 tiles with the fewest keys (the
+    first rows), the last-dispatched one into the most parts, and leaves 12 x 40 = 480 <= 512 whole workgroups."""
+    trees = np.array([(0, 6144, 0, 2048)], abi.TREE_DT)
+    tiles, jobs, parts = host.plan_tiles(trees, 40, 0, None, host.options_mi355x(128, 512))
+    per_tile = [int((tiles["r0"] == r).sum()) for r in range(0, 2048, 128)]
+    assert per_tile[4:] == [1] * 12 and all(p >= 2 for p in per_tile[:4])
+    assert per_tile[:4] == sorted(per_tile[:4], reverse=True) and per_tile[0] > per_tile[3]
+    assert len(jobs) == 4 and parts == sum(per_tile[:4])
+    # exactly one round of workgroups (16 x 32 = 512): nothing to gain, nothing is cut
+    tiles, jobs, parts = host.plan_tiles(trees, 32, 0, None, host.options_mi355x(128, 512))
+    assert len(tiles) == 16 and parts == 0
+    # a chunk with nothing cached has no range to cut
+    tiles, jobs, parts = host.plan_tiles(np.array([(0, 0, 0, 2048)], abi.TREE_DT), 40, 0, None, host.options_mi355x(128, 512))
+    assert len(tiles) == 16 and parts == 0
+
+
 def test_balanced_rule_equalises_keys_per_workgroup():
     """16 sequences of 512..8192 keys: the reference rule gives every sequence the same
     number of splits; the balanced rule gives every workgroup about the same key count."""
