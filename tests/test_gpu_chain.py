@@ -209,8 +209,6 @@ def test_fused_prep_on_verify_trees_is_prep_then_attention_bit_for_bit(H, Hkv, H
     n_rows = sum(m for _, m in seqs)
     ap = synth.make_params(H, Hkv, HD, dtype, BT, rows_per_tile=4)
     pp, a = synth.make_prep(kind, H, Hkv, HD, dtype, n_rows, seed=29, bt=BT)
-    if kind == "qwen35":          # the sigmoid gate beside each query in the projection (40_attention.metal:47, :334-342)
-        pass
     nb = [(p + m + BT - 1) // BT for p, m in seqs]
     n_blocks = sum(nb) + 2
     perm = rng.permutation(n_blocks).astype(np.int32)
@@ -239,6 +237,9 @@ def test_fused_prep_on_verify_trees_is_prep_then_attention_bit_for_bit(H, Hkv, H
     dev = lambda x: None if x is None else torch.from_numpy(np.ascontiguousarray(x)).cuda()  # noqa: E731
     Xd, qn, kn, posd = dev(a["X"]), dev(a["qn_w"]), dev(a["kn_w"]), dev(pos)
     inv_freq, sel, tabd = dev(a["inv_freq"]), dev(a["rope_sel"]), dev(table)
+    if kind == "qwen35":   # the sigmoid gate beside each query in the projection itself (40_attention.metal:47, :334-342)
+        ap.gate = Xd.data_ptr()
+        ap.gate_ld, ap.gate_hs, ap.gate_off = pp.x_ld, pp.q_hs, HD
     print(f"fused verify: H={H} Hkv={Hkv} HD={HD} {kind} tiles={len(tiles)} parts={n_parts}", flush=True)
     outs, pools = [], []
     for fused in (False, True):
@@ -259,3 +260,4 @@ def test_fused_prep_on_verify_trees_is_prep_then_attention_bit_for_bit(H, Hkv, H
     assert torch.equal(outs[0].view(torch.int16), outs[1].view(torch.int16)), "fused output differs"
     assert torch.equal(pools[0].view(torch.int16), pools[1].view(torch.int16)), "fused append differs"
     assert not torch.equal(pools[0].view(torch.int16), pool0.view(torch.int16))
+    ap.gate = None
