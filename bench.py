@@ -790,6 +790,7 @@ class Ceilings:
         V, I = C.c_void_p, C.c_int32
         self.lib.esp_ceiling_hbm_read.argtypes = [V, V, I, I, I, I, V, V, V, V]
         self.lib.esp_ceiling_mfma_issue.argtypes = [I, I, I, I, I, V, V, V, V]
+        self.lib.esp_ceiling_prefill_step.argtypes = [I, I, I, I, I, V, V, V, V, V, V]
 
     def _events(self, n):
         t = self.torch
@@ -855,6 +856,35 @@ class Ceilings:
             out.append({"valu_per_mfma": nv, "exp_per_mfma": ne, "operands": "random" if rnd else "constant",
                         "TFLOPs": round(flops / float(np.median(ms)) / 1e9, 1),
                         "ns_per_mfma_per_simd": round(float(np.median(ms)) * 1e6 / (iters * 32 * 2), 2)})
+        return out
+
+
+    STAGES = ("matrix instructions, operands in registers", "+ A operands read from LDS", "+ a barrier per step",
+              "+ the softmax's vector work", "+ 32 KB per step staged into LDS")
+
+    def prefill_step(self, cases=((0, 1, 1), (1, 1, 1), (2, 1, 1), (3, 1, 1), (4, 1, 1), (4, 1, 0), (1, 2, 1), (3, 2, 1), (4, 2, 1)), iters=3000):
+        """TFLOP/s of the prefill kernel's step as a bare instruction stream, one ingredient more per stage, at 32
+        rows per wavefront and two workgroups per compute unit (the kernels as built) or 64 rows and one, on random
+        or constant operands; with the clock each launch ran at, read inside the kernel."""
+        t = self.torch
+        src = t.full(((4 << 20) + 65536,), 0x5b, dtype=t.uint8, device="cuda")
+        st = self.C.c_void_p(t.cuda.current_stream().cuda_stream)
+        out = []
+        for stage, rows, rnd in cases:
+            wgs = 2 * N_CU if rows == 1 else N_CU
+            outbuf = t.zeros(wgs * 256, dtype=t.float32, device="cuda")
+            clk = t.zeros(2 * wgs, dtype=t.int64, device="cuda")
+            evs = self._events(4)
+            for a, b in evs:
+                rc = self.lib.esp_ceiling_prefill_step(stage, rows, rnd, wgs, iters, self.C.c_void_p(outbuf.data_ptr()), self.C.c_void_p(src.data_ptr()),
+                                                       self.C.c_void_p(clk.data_ptr()), st, self.C.c_void_p(a.cuda_event), self.C.c_void_p(b.cuda_event))
+                assert rc == 0, rc
+            t.cuda.synchronize()
+            ms = float(np.median([a.elapsed_time(b) for a, b in evs][1:]))
+            ck = clk.cpu().numpy().reshape(wgs, 2).astype(np.float64)
+            out.append({"stage": stage, "what": self.STAGES[stage], "rows_per_wavefront": 32 * rows, "operands": "random" if rnd else "constant",
+                        "TFLOPs": round(wgs * 4 * iters * 32 * rows * 32768 / ms / 1e9, 1),
+                        "clock_GHz": round(float((ck[:, 0] / (ck[:, 1] / 100e6)).mean()) / 1e9, 3)})
         return out
 
 
@@ -937,7 +967,7 @@ def main():
     ap.add_argument("--warmup", type=int, default=20)
     ap.add_argument("--workload", default="all",
                     help="all (default): the batched decode as the headline, the chunked prefill, one record per benchmark "
-                         "configuration and the measured ceilings; or one of: hbm_read_ceiling, mfma_issue_ceiling, decode_step_fusion, " + ", ".join(WORKLOADS))
+                         "configuration and the measured ceilings; or one of: hbm_read_ceiling, mfma_issue_ceiling, prefill_step_ceiling, decode_step_fusion, " + ", ".join(WORKLOADS))
     ap.add_argument("--workgroups", type=int, default=0, help="planner split target (0: ask esp_attn_plan_hint)")
     ap.add_argument("--tables", default="scattered", choices=["scattered", "contiguous"],
                     help="block tables: a seeded permutation of the pool (the benchmark's definition) or address order")
@@ -970,6 +1000,10 @@ def main():
     if args.workload == "mfma_issue_ceiling":
         print(json.dumps({"metric": "matrix cores under vector issue, TFLOP/s", "unit": "TFLOP/s", "peak": MFMA_PEAK_TFLOPS,
                           "mixes": Ceilings().mfma_issue()}), flush=True)
+        return
+    if args.workload == "prefill_step_ceiling":
+        print(json.dumps({"metric": "the prefill kernels' step as a bare instruction stream, TFLOP/s", "unit": "TFLOP/s",
+                          "peak": MFMA_PEAK_TFLOPS, "stages": Ceilings().prefill_step()}), flush=True)
         return
     w = make_workload(args.workload, args.workgroups or None, args.tables == "contiguous", args.page)
     K, W = args.steps, args.warmup

@@ -2,7 +2,8 @@
 // of their own (include/espetero_ceilings.h): what a plain streaming read reaches at a given size and
 // page scatter, and what the matrix cores reach when the wavefront that feeds them also issues a given
 // amount of vector arithmetic. The reference states its kernels against measured machine limits the
-// same way (docs/kernel-guidelines.md:19-27: a measured stream peak and a measured MMA rate).
+// same way (docs/kernel-guidelines.md:19-27: a measured stream peak and a measured MMA rate). A third kernel
+// is the prefill kernel's step as a bare instruction stream, ingredient by ingredient.
 // Measurement only: nothing in the attention path calls these.
 #include <hip/hip_runtime.h>
 #include <hip/hip_ext.h>
@@ -100,6 +101,128 @@ __global__ __launch_bounds__(256, 2) void issue_kernel(float* out, int iters, ui
   out[blockIdx.x * 256 + threadIdx.x] = r;
 }
 
+// The prefill kernel's step as an instruction stream, built up one ingredient at a time (STAGE):
+//   0  32 matrix instructions per step in chains of 8 on alternating accumulators, operands in registers
+//   1  + the A operand of every matrix instruction read from LDS, 8 reads a group ahead of their use
+//   2  + one workgroup barrier per step
+//   3  + the softmax's share of vector work on the two middle groups (two v_exp_f32, two subtracts, two adds
+//        per matrix instruction), laid by hand behind each matrix instruction
+//   4  + each wavefront staging 8 KB per step from global memory straight into LDS (global_load_lds_dwordx4),
+//        from a 4 MB window of `src` that stays in the caches
+// ROWS: 1 = 32 query rows per wavefront (the kernels as built), 2 = 64 rows: every operand read feeds two
+// matrix instructions, at one wavefront per SIMD. clk[2 w], clk[2 w + 1]: cycles and 100 MHz ticks workgroup w
+// was alive, which give the clock the part ran at under this load.
+__device__ __forceinline__ void stage_to_lds(const char* base, uint32_t lane_off, uint32_t lds_addr) {
+  lds_addr = uint32_t(__builtin_amdgcn_readfirstlane(int(lds_addr)));
+  const uint64_t b64 = reinterpret_cast<uint64_t>(base);
+  const uint32_t b_lo = uint32_t(__builtin_amdgcn_readfirstlane(int(uint32_t(b64))));
+  const uint32_t b_hi = uint32_t(__builtin_amdgcn_readfirstlane(int(uint32_t(b64 >> 32))));
+  base = reinterpret_cast<const char*>(uint64_t(b_lo) | (uint64_t(b_hi) << 32));
+  asm volatile(
+      "s_mov_b32 m0, %0\n\ts_nop 0\n\t"
+      "global_load_lds_dwordx4 %1, %2\n\t"
+      "global_load_lds_dwordx4 %1, %2 offset:1024\n\t"
+      "global_load_lds_dwordx4 %1, %2 offset:2048\n\t"
+      "global_load_lds_dwordx4 %1, %2 offset:3072"
+      :
+      : "s"(lds_addr), "v"(lane_off), "s"(base)
+      : "memory");
+}
+
+template <int STAGE, int ROWS>
+__global__ __launch_bounds__(256, ROWS == 2 ? 1 : 2) void step_kernel(float* out, int iters, uint32_t seed, int random_data, const char* src,
+                                                                       unsigned long long* clk) {
+  const unsigned long long c0 = __builtin_readcyclecounter(), r0 = __builtin_amdgcn_s_memrealtime();
+  extern __shared__ __attribute__((aligned(16))) char lds[];  // 32 KB of operands, 32 KB of staging space
+  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+  auto rnd = [&](uint32_t x) {
+    x = x * 2654435761u + seed;
+    x ^= x >> 15;
+    x *= 2246822519u;
+    x ^= x >> 13;
+    return random_data ? (x & 0x807f807fu) | 0x3e803e80u | ((x >> 3) & 0x01000100u) : 0x3f803f80u;
+  };
+  const u32x4 a = {rnd(threadIdx.x), rnd(threadIdx.x + 999), rnd(threadIdx.x + 77), rnd(threadIdx.x + 5)};
+  const u32x4 b = {rnd(threadIdx.x + 11), rnd(threadIdx.x + 13), rnd(threadIdx.x + 17), rnd(threadIdx.x + 19)};
+  const u32x4 b2 = {rnd(threadIdx.x + 21), rnd(threadIdx.x + 23), rnd(threadIdx.x + 27), rnd(threadIdx.x + 29)};
+  f32x16 c[4] = {}, c2[4] = {};
+  float v[16], w[16];
+#pragma unroll
+  for (int i = 0; i < 16; ++i) {
+    v[i] = -float(threadIdx.x + i) * 1e-3f;
+    w[i] = v[i] * 0.5f;
+  }
+  for (int i = threadIdx.x; i < 16384; i += 256) reinterpret_cast<uint32_t*>(lds)[i] = rnd(i * 7 + blockIdx.x);
+  __syncthreads();
+  using lds_ptr = const __attribute__((address_space(3))) u32x4*;
+  const uint32_t lds0 = uint32_t(uintptr_t(lds)), base = lds0 + lane * 16;
+  auto mm = [](u32x4 x, u32x4 y, f32x16 z) { return __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(bf16x8, x), __builtin_bit_cast(bf16x8, y), z, 0, 0, 0); };
+  u32x4 ring[2][8];
+  if constexpr (STAGE >= 1) {
+#pragma unroll
+    for (int j = 0; j < 8; ++j) ring[0][j] = *reinterpret_cast<lds_ptr>(base + j * 1024);
+  }
+  for (int it = 0; it < iters; ++it) {
+#pragma unroll
+    for (int g = 0; g < 4; ++g) {
+      if constexpr (STAGE >= 1) {
+#pragma unroll
+        for (int j = 0; j < 8; ++j) ring[(g + 1) & 1][j] = *reinterpret_cast<lds_ptr>(base + ((g + 1) & 3) * 8192 + j * 1024);
+        __builtin_amdgcn_s_waitcnt(0xC07F | (8 << 8));  // the 8 reads of a group ago have landed
+      }
+#pragma unroll
+      for (int j = 0; j < 8; ++j) {
+        const int ci = (g & 1) + 2 * (g >> 1);
+        const u32x4 x = STAGE >= 1 ? ring[g & 1][j] : a;
+        c[ci] = mm(x, b, c[ci]);
+        if constexpr (ROWS == 2) c2[ci] = mm(x, b2, c2[ci]);
+        if constexpr (STAGE >= 3) {
+          if (g == 1 || g == 2) {
+            v[2 * j] = __builtin_amdgcn_exp2f(v[2 * j] - c[3][0]);
+            v[2 * j + 1] = __builtin_amdgcn_exp2f(v[2 * j + 1] - c[3][0]);
+            v[(2 * j + 5) & 15] += v[(2 * j + 7) & 15];
+            v[(2 * j + 9) & 15] += v[(2 * j + 11) & 15];
+            asm volatile("" : "+v"(v[2 * j]), "+v"(v[2 * j + 1]));
+            if constexpr (ROWS == 2) {
+              w[2 * j] = __builtin_amdgcn_exp2f(w[2 * j] - c2[3][0]);
+              w[2 * j + 1] = __builtin_amdgcn_exp2f(w[2 * j + 1] - c2[3][0]);
+              w[(2 * j + 5) & 15] += w[(2 * j + 7) & 15];
+              w[(2 * j + 9) & 15] += w[(2 * j + 11) & 15];
+              asm volatile("" : "+v"(w[2 * j]), "+v"(w[2 * j + 1]));
+            }
+          }
+        }
+        __builtin_amdgcn_sched_barrier(0);
+      }
+    }
+    if constexpr (STAGE >= 4) asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+    if constexpr (STAGE >= 2) __syncthreads();
+    if constexpr (STAGE >= 4) {
+      const size_t off = (size_t(blockIdx.x) * 977 * 16 + size_t(it) * 32768 + wave * 8192) & ((size_t(4) << 20) - 1 - 65535);
+      stage_to_lds(src + off, lane * 16, lds0 + 32768 + wave * 8192);
+      stage_to_lds(src + off + 4096, lane * 16, lds0 + 32768 + wave * 8192 + 4096);
+    }
+  }
+  if constexpr (STAGE >= 4) asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+  if (threadIdx.x == 0 && clk) {
+    clk[2 * blockIdx.x] = __builtin_readcyclecounter() - c0;
+    clk[2 * blockIdx.x + 1] = __builtin_amdgcn_s_memrealtime() - r0;
+  }
+  float r = 0;
+#pragma unroll
+  for (int i = 0; i < 16; ++i) r += c[0][i] + c[1][i] + c[2][i] + c[3][i] + v[i] + c2[0][i] + c2[1][i] + c2[2][i] + c2[3][i] + w[i];
+  out[blockIdx.x * 256 + threadIdx.x] = r;
+}
+
+template <typename K, typename... Args>
+hipError_t launch_lds(K k, size_t lds_bytes, dim3 grid, dim3 block, hipStream_t st, hipEvent_t e0, hipEvent_t e1, Args... args) {
+  hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(k), hipFuncAttributeMaxDynamicSharedMemorySize, int(lds_bytes));
+  if (e != hipSuccess) return e;
+  if (e0 && e1) hipExtLaunchKernelGGL(k, grid, block, lds_bytes, st, e0, e1, 0, args...);
+  else hipLaunchKernelGGL(k, grid, block, lds_bytes, st, args...);
+  return hipGetLastError();
+}
+
 template <typename K, typename... Args>
 hipError_t launch(K k, dim3 grid, dim3 block, hipStream_t st, hipEvent_t e0, hipEvent_t e1, Args... args) {
   if (e0 && e1) hipExtLaunchKernelGGL(k, grid, block, 0, st, e0, e1, 0, args...);
@@ -143,6 +266,28 @@ int esp_ceiling_mfma_issue(int32_t valu_per_mfma, int32_t exp_per_mfma, int32_t 
     case 31: e = launch(issue_kernel<3, 1>, g, b, st, e0, e1, out, iters, 1u, random_data); break;
     case 41: e = launch(issue_kernel<4, 1>, g, b, st, e0, e1, out, iters, 1u, random_data); break;
     case 51: e = launch(issue_kernel<5, 1>, g, b, st, e0, e1, out, iters, 1u, random_data); break;
+    default: return 2;
+  }
+  return e == hipSuccess ? 0 : 3;
+}
+
+int esp_ceiling_prefill_step(int32_t stage, int32_t rows, int32_t random_data, int32_t workgroups, int32_t iters, float* out, const void* src,
+                             unsigned long long* clk, void* stream, void* start_event, void* stop_event) {
+  if (!out || workgroups <= 0 || iters <= 0 || (stage >= 4 && !src)) return 1;
+  const auto st = static_cast<hipStream_t>(stream);
+  const auto e0 = static_cast<hipEvent_t>(start_event), e1 = static_cast<hipEvent_t>(stop_event);
+  const dim3 g(workgroups), b(256);
+  const char* s = static_cast<const char*>(src);
+  hipError_t e;
+  switch (stage * 10 + rows) {
+    case 1: e = launch_lds(step_kernel<0, 1>, 65536, g, b, st, e0, e1, out, iters, 1u, random_data, s, clk); break;
+    case 11: e = launch_lds(step_kernel<1, 1>, 65536, g, b, st, e0, e1, out, iters, 1u, random_data, s, clk); break;
+    case 21: e = launch_lds(step_kernel<2, 1>, 65536, g, b, st, e0, e1, out, iters, 1u, random_data, s, clk); break;
+    case 31: e = launch_lds(step_kernel<3, 1>, 65536, g, b, st, e0, e1, out, iters, 1u, random_data, s, clk); break;
+    case 41: e = launch_lds(step_kernel<4, 1>, 65536, g, b, st, e0, e1, out, iters, 1u, random_data, s, clk); break;
+    case 12: e = launch_lds(step_kernel<1, 2>, 65536, g, b, st, e0, e1, out, iters, 1u, random_data, s, clk); break;
+    case 32: e = launch_lds(step_kernel<3, 2>, 65536, g, b, st, e0, e1, out, iters, 1u, random_data, s, clk); break;
+    case 42: e = launch_lds(step_kernel<4, 2>, 65536, g, b, st, e0, e1, out, iters, 1u, random_data, s, clk); break;
     default: return 2;
   }
   return e == hipSuccess ? 0 : 3;

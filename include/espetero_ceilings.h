@@ -3,8 +3,8 @@
  *
  * No counterpart among the reference's kernels; its documentation holds its kernels against
  * measured limits of the machine rather than data-sheet figures (docs/kernel-guidelines.md:19-27:
- * a measured stream bandwidth and a measured MMA rate). These two calls produce the same two
- * figures on an MI355X; bench.py reports them (--workload hbm_read_ceiling, mfma_issue_ceiling)
+ * a measured stream bandwidth and a measured MMA rate). The first two calls produce the same two
+ * figures on an MI355X, the third the ceiling of the prefill kernels' own step; bench.py reports them (--workload hbm_read_ceiling, mfma_issue_ceiling, prefill_step_ceiling)
  * and states every roofline fraction against the data-sheet peak and against them.
  * Conventions as in espetero_attn.h: device pointers, work enqueued on `stream`, 0 or an error
  * code (1 bad argument, 2 unsupported, 3 launch failure). start_event / stop_event: two
@@ -37,6 +37,19 @@ int esp_ceiling_hbm_read(const void* base, const int32_t* pages, int32_t n_pages
  * Flops of a launch: workgroups * 4 * iters * 32 * 32768. */
 int esp_ceiling_mfma_issue(int32_t valu_per_mfma, int32_t exp_per_mfma, int32_t random_data, int32_t workgroups, int32_t iters, float* out, void* stream,
                            void* start_event, void* stop_event);
+
+/* The prefill kernels' key step as a bare instruction stream, one ingredient more per stage: 0 = 32
+ * v_mfma_f32_32x32x16_bf16 per step in chains of 8 with operands in registers; 1 = + every A operand read from
+ * LDS a group ahead; 2 = + a workgroup barrier per step; 3 = + the softmax's share of vector work behind the
+ * matrix instructions of two of the four groups; 4 = + every wavefront staging 8 KB per step from `src` (a
+ * device buffer of at least 4 MB + 64 KB, cache resident) straight into LDS. rows: 1 = 32 query rows per wavefront,
+ * two workgroups per compute unit (the kernels as built); 2 = 64 rows, every operand read feeding two matrix
+ * instructions, one workgroup per compute unit (stages 1, 3, 4 only). What stage 4 reaches is the ceiling of
+ * that kernel design; the difference between stages is what each ingredient costs. clk (NULL or 2 * workgroups
+ * 64-bit words): cycles and 100 MHz ticks each workgroup was alive; cycles / ticks * 100 MHz is the clock the
+ * part ran at. out: workgroups * 256 floats. Flops of a launch: workgroups * 4 * iters * 32 * rows * 32768. */
+int esp_ceiling_prefill_step(int32_t stage, int32_t rows, int32_t random_data, int32_t workgroups, int32_t iters, float* out, const void* src,
+                             unsigned long long* clk, void* stream, void* start_event, void* stop_event);
 
 #ifdef __cplusplus
 }

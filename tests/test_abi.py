@@ -33,6 +33,21 @@ def test_engine_library_exports_every_declared_symbol():
         assert hasattr(lib, n), n
 
 
+def test_ceilings_library_exports_every_declared_symbol_and_refuses_bad_arguments():
+    names = _declared("espetero_ceilings.h")
+    assert names == ["esp_ceiling_hbm_read", "esp_ceiling_mfma_issue", "esp_ceiling_prefill_step"]
+    lib = C.CDLL(os.path.join(ROOT, "espetero_amd", "csrc", "libespetero_ceilings.so"))
+    for n in names:
+        assert hasattr(lib, n), n
+    V, I = C.c_void_p, C.c_int32
+    lib.esp_ceiling_hbm_read.argtypes = [V, V, I, I, I, I, V, V, V, V]
+    lib.esp_ceiling_mfma_issue.argtypes = [I, I, I, I, I, V, V, V, V]
+    lib.esp_ceiling_prefill_step.argtypes = [I, I, I, I, I, V, V, V, V, V, V]
+    assert lib.esp_ceiling_hbm_read(None, None, 4, 8192, 1, 8, None, None, None, None) == 1        # no buffer: refused on the host
+    assert lib.esp_ceiling_mfma_issue(0, 0, 1, 8, 10, None, None, None, None) == 1
+    assert lib.esp_ceiling_prefill_step(4, 1, 1, 8, 10, None, None, None, None, None, None) == 1
+
+
 def test_record_layouts_match_the_reference_structs():
     """AttnTree 16 B, tile 32 B, combine 16 B, KVSave 16 B (kernels/40_attention.metal:134-150,
     804-809, 868-873): field order is part of the contract."""
