@@ -160,7 +160,9 @@ int device_state(DeviceState** out, char* err, size_t errlen) {
 }  // namespace
 
 namespace esp {
-static TimeNext g_time_next;
+// One pending pair per calling thread: the thread that armed it is the one whose next launch takes it, so a
+// second thread driving other streams neither sees nor consumes it.
+static thread_local TimeNext g_time_next;
 TimeNext take_time_next() {
   const TimeNext t = g_time_next;
   g_time_next = TimeNext{};

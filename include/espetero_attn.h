@@ -199,8 +199,8 @@ int esp_attn_validate(const esp_attn_params* p, const esp_tile* tiles, int32_t n
  * into them: hipEventElapsedTime(start, stop) is then that kernel's duration,
  * without marker packets between the kernels of the stream. The pair is used
  * once, by the next such call, whether or not that call launches anything (a call
- * that returns early drops it). One pending pair per process: a single caller
- * thread arms it and makes the call. Both NULL clears a pending pair. */
+ * that returns early drops it). One pending pair per calling thread: the
+ * thread that arms it makes the call that takes it; other threads' calls neither see nor consume it. Both NULL clears a pending pair. */
 int esp_attn_time_next(void* start_event, void* stop_event);
 
 /* The split-K merge alone: attention_combine (40_:811-864, 80_:568-597) as its
