@@ -314,11 +314,12 @@ class DecodeStep:
             dp.run(w.Q, w.Kb, w.Vb, w.pool, w.O)
 
 
-def decode_step_fusion(args, torch):
+def decode_step_fusion(args, torch, names=("c1_single_decode", "c2_batched_decode", "c4_decode_sliding", "c4_decode_global"), emit=True):
     """Step time of the attention part of a decode layer with and without the prep fused into the attention kernel:
     eager wall time per step and the time per step of 16 steps replayed from one HIP graph."""
     out = {"metric": "decode attention step, prep + attention", "unit": "us", "steps": args.steps, "warmup": args.warmup, "configs": {}}
-    for name, kind in (("c1_single_decode", "omni"), ("c2_batched_decode", "omni"), ("c4_decode_sliding", "gemma"), ("c4_decode_global", "gemma")):
+    for name in names:
+        kind = "omni" if name.startswith(("c1", "c2")) else "gemma"
         w = make_workload(name, args.workgroups or None, args.tables == "contiguous", args.page)
         rec = {}
         outs = []
@@ -343,7 +344,9 @@ def decode_step_fusion(args, torch):
         out["configs"][name] = rec
         del w
         torch.cuda.empty_cache()
-    print(json.dumps(out), flush=True)
+    if emit:
+        print(json.dumps(out), flush=True)
+    return out
 
 
 def make_workload(name, workgroups=None, contiguous=False, page=16):
@@ -956,6 +959,9 @@ def run_all(args, torch):
                        "kernel_us_median": pre["roofline"]["kernel_us_median"], "kernel_us_min": pre["roofline"]["kernel_us_min"],
                        "max_abs_err_vs_cpu": pre.get("max_abs_err_vs_cpu"), "tolerance": pre["tolerance"], "see": "prefill"})
     out["configs"] = configs
+    # the decode step from the fp32 projection to O: esp_attn_prep + esp_attn_forward against esp_attn_decode_fused
+    fa = argparse.Namespace(**{**vars(args), "steps": 100, "warmup": 10})
+    out["decode_step"] = decode_step_fusion(fa, torch, ("c1_single_decode", "c2_batched_decode", "c4_decode_sliding"), emit=False)["configs"]
     out["ceilings"] = {"hbm_read": reads, "mfma_issue": issue}
     print(json.dumps(out), flush=True)
 
