@@ -19,12 +19,15 @@ constexpr int prep_epl(int HD) { return HD > 256 ? 8 : 4; }
 template <int HD>
 __device__ __forceinline__ void prep_lane(float (&x)[prep_epl(HD)], int kind, const float (&w)[prep_epl(HD)], const float2* cs,
                                           const esp_prep_params& p, int d0) {
+  // Two kernels inline this function and must agree to the bit, so nothing here is left to the compiler's
+  // choice of which multiply to fuse with which add: the fused operations are spelled out, the rest stays apart.
+#pragma clang fp contract(off)
   constexpr int EPL = prep_epl(HD), LPH = HD / EPL;
   const int half = p.rope_dims / 2;
   if (kind != 2 || p.v_norm) {
     float ss = 0.0f;
 #pragma unroll
-    for (int i = 0; i < EPL; ++i) ss += x[i] * x[i];
+    for (int i = 0; i < EPL; ++i) ss = __builtin_fmaf(x[i], x[i], ss);
 #pragma unroll
     for (int o = LPH / 2; o >= 1; o >>= 1) ss += __shfl_xor(ss, o);
     const float inv = rsqrtf(ss / float(HD) + p.eps);
@@ -40,7 +43,8 @@ __device__ __forceinline__ void prep_lane(float (&x)[prep_epl(HD)], int kind, co
       const float partner = __shfl_xor(x[i], half / EPL);
       if (d0 < p.rope_dims) {
         const float2 t = cs[(lower ? d0 : d0 - half) + i];
-        x[i] = lower ? x[i] * t.x - partner * t.y : x[i] * t.x + partner * t.y;
+        const float turned = partner * t.y;
+        x[i] = __builtin_fmaf(x[i], t.x, lower ? -turned : turned);
       }
     }
   }
