@@ -400,10 +400,15 @@ def make_workload(name, workgroups=None, contiguous=False, page=16):
 def measured_traffic(workload):
     """HBM bytes one launch of the dominant kernel moves, as measured with the rocprofv3 FETCH_SIZE and
     WRITE_SIZE counters (each scaled by what the same counter reads for a plain 256 MiB copy); the
-    summaries under profiles/ show the runs. None for a workload that has not been measured."""
+    summaries under profiles/ show the runs. A step of several launches (the chunked prefill, the layer mixes) is
+    the sum over its launches. None for a workload that has not been measured."""
+    parts = {"c3_chunked_prefill": ["c3_prefill_p0", "c3_prefill_p2048", "c3_prefill_p4096", "c3_prefill_p6144"],   # one launch per chunk
+             "c4_decode_mix": ["c4_decode_sliding"] * 5 + ["c4_decode_global"],
+             "c4_prefill_mix": ["c4_prefill_sliding"] * 5 + ["c4_prefill_global"]}.get(workload, [workload])
     try:
         with open(os.path.join(ROOT, "profiles", "traffic.json")) as f:
-            return int(json.load(f)[workload]["hbm_bytes_per_launch"])
+            t = json.load(f)
+        return sum(int(t[x]["hbm_bytes_per_launch"]) for x in parts)
     except (OSError, KeyError, ValueError):
         return None
 
