@@ -212,6 +212,22 @@ def test_validate_accepts_a_planned_pass_and_names_the_first_bad_record():
         device.validate(p, tl, tr, jb, npart, 1, None, 11)
 
 
+def test_validate_accepts_the_tiled_planner_s_partly_split_chunk():
+    """A prefill chunk planned for the tiled kernel (128-row tiles, only the shortest tiles cut into parts of unequal
+    count) passes the validator; dropping one of a tile's parts does not."""
+    import numpy as np
+    import pytest
+    from espetero_amd import device, synth
+    p = synth.make_params(40, 8, 128, abi.ESP_BF16, 16, rows_per_tile=128)
+    trees = np.array([(0, 6144, 0, 2048)], abi.TREE_DT)
+    tiles, jobs, n_parts = host.plan_tiles(trees, 40, 0, None, host.options_mi355x(128, 512))
+    assert n_parts > 4 and len(jobs) == 4
+    blocks = np.arange((6144 + 2048) // 16, dtype=np.int32)
+    device.validate(p, tiles, trees, jobs, n_parts, 2048, blocks, len(blocks))
+    with pytest.raises(abi.EspError, match="which no tile writes"):
+        device.validate(p, np.delete(tiles, 1), trees, jobs, n_parts, 2048, blocks, len(blocks))
+
+
 def test_forward_static_refuses_what_does_not_fit_its_scratch_array():
     """The entry point without a workspace names its limit; checked on the host before any launch or device call."""
     from espetero_amd import synth
