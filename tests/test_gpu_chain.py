@@ -261,3 +261,69 @@ def test_fused_prep_on_verify_trees_is_prep_then_attention_bit_for_bit(H, Hkv, H
     assert torch.equal(pools[0].view(torch.int16), pools[1].view(torch.int16)), "fused append differs"
     assert not torch.equal(pools[0].view(torch.int16), pool0.view(torch.int16))
     ap.gate = None
+
+
+def test_fused_decode_on_seeded_random_shapes_is_prep_then_attention_bit_for_bit():
+    """40 seeded random decode / short-verify passes (head dim, grouping, element type, block size, prep arrangement,
+    rows per tile, ragged cached lengths incl. empty ones, window over block lists, split target): the fused call and
+    the two calls must leave identical outputs and identical pools."""
+    device.init(0)
+    rng = np.random.default_rng(77)
+    dev = lambda x: None if x is None else torch.from_numpy(np.ascontiguousarray(x)).cuda()  # noqa: E731
+    for it in range(40):
+        HD = int(rng.choice([128, 256]))
+        G = int(rng.choice([1, 2, 4, 5, 8]))
+        Hkv = int(rng.choice([1, 2, 4]))
+        H = G * Hkv
+        max_cols = 32 if HD == 128 else 16
+        R = int(rng.integers(1, min(4, max_cols // G) + 1))
+        BT = int(rng.choice([16, 32, 64]))
+        dtype = int(rng.choice([abi.ESP_F16, abi.ESP_BF16]))
+        kind = str(rng.choice(["omni", "gemma", "qwen35"]))
+        window = int(rng.choice([0, 0, 200]))
+        seqs = [(int(rng.choice([0, 1, 15, 16, 17, 300, 1500, 4000])), int(rng.integers(1, R + 1))) for _ in range(int(rng.integers(1, 7)))]
+        n_rows = sum(m for _, m in seqs)
+        ap = synth.make_params(H, Hkv, HD, dtype, BT, window=window, rows_per_tile=R)
+        pp, a = synth.make_prep(kind, H, Hkv, HD, dtype, n_rows, seed=1000 + it, bt=BT)
+        nb = [(p + m + BT - 1) // BT for p, m in seqs]
+        n_blocks = sum(nb) + 2
+        blocks = rng.permutation(n_blocks).astype(np.int32)[:sum(nb)].copy()
+        trees = np.zeros(len(seqs), abi.TREE_DT)
+        desc = np.zeros((n_rows, 4), np.int32)
+        pos = np.zeros((n_rows, 4), np.int32)
+        table = np.full((n_rows, 4), -1, np.int32)
+        base = off = 0
+        for i, (p, m) in enumerate(seqs):
+            trees[i] = (base, p, off, m)
+            if m > 1:
+                desc[base:base + m] = synth.verify_desc(m, 1)
+            tok = p + np.arange(m)
+            pos[base:base + m, :3] = tok[:, None]
+            table[base:base + m, 0] = blocks[off + tok // BT]
+            table[base:base + m, 1] = tok % BT
+            base += m
+            off += nb[i]
+        tdt = torch.float16 if dtype == abi.ESP_F16 else torch.bfloat16
+        pool0 = (torch.randn(n_blocks * 2 * BT * ap.kv_ld, device="cuda") * 0.5).to(tdt)
+        resident, groups = device.plan_hint(ap)
+        tiles, jobs, n_parts = host.plan_tiles(trees, groups, window, pos if window else None, host.options_mi355x(R, int(rng.choice([8, 64, resident]))))
+        print(f"fused random {it}: H={H} Hkv={Hkv} HD={HD} R={R} bt={BT} dtype={dtype} {kind} window={window} seqs={seqs} tiles={len(tiles)} parts={n_parts}", flush=True)
+        dp = device.DevicePass(ap, trees, tiles, jobs, n_parts, n_rows, blocks, desc, pos, pool_blocks=n_blocks)
+        Xd, qn, kn, posd = dev(a["X"]), dev(a["qn_w"]), dev(a["kn_w"]), dev(pos)
+        inv_freq, sel, tabd = dev(a["inv_freq"]), dev(a["rope_sel"]), dev(table)
+        res = []
+        for fused in (False, True):
+            pool = pool0.clone()
+            O = torch.zeros(n_rows, ap.q_ld, dtype=tdt, device="cuda")
+            if fused:
+                device.decode_fused(pp, ap, Xd, qn, kn, posd, inv_freq, sel, tabd, pool, dp, O)
+            else:
+                Q = torch.zeros(n_rows, ap.q_ld, dtype=tdt, device="cuda")
+                Kb = torch.zeros(n_rows, ap.kv_ld, dtype=tdt, device="cuda")
+                Vb = torch.zeros_like(Kb)
+                device.attn_prep(pp, Xd, qn, kn, posd, inv_freq, sel, Q, Kb, Vb, tabd, pool, n_rows)
+                dp.run(Q, Kb, Vb, pool, O)
+            torch.cuda.synchronize()
+            res.append((O, pool))
+        assert torch.equal(res[0][0].view(torch.int16), res[1][0].view(torch.int16)), (it, "output")
+        assert torch.equal(res[0][1].view(torch.int16), res[1][1].view(torch.int16)), (it, "pool")
