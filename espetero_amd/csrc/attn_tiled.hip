@@ -195,7 +195,7 @@ __global__ __launch_bounds__(256, OCC) void attn_tiled_kernel(const KArgs a, int
   // (32 V^T rows of 16 tokens are 1024 bytes, in the pool's sub-blocks and in the staged batch rows alike)
   const uint32_t voff = uint32_t(l32 * 32 + hb * 16);
 
-  // interior: the caller knows that all four sub-blocks of the step are cached keys.
+  // interior: the caller knows that all four sub-blocks of the step are cached keys, or batch rows that exist.
   auto fill = [&](int step, int stage, auto interior) __attribute__((always_inline)) {
     const int s = 4 * step + wave;
     const uint32_t kdst = lds_base + stage * KBUF + wave * (16 * ROWB);
@@ -206,7 +206,7 @@ __global__ __launch_bounds__(256, OCC) void attn_tiled_kernel(const KArgs a, int
     // memory, whose reloads wait on the same counter as the staging loads and serialise them.
     uint32_t kc = kcol0, kr = uint32_t(r0);
     asm volatile("" : "+v"(kc), "+v"(kr));
-    if (decltype(interior)::value || s < n_c) {
+    if (s < n_c) {
       const int js = (c0 + s) << 4;
       const int b = block_id(step);
       const int t0 = a.bt == 16 ? 0 : js % a.bt;
@@ -220,9 +220,9 @@ __global__ __launch_bounds__(256, OCC) void attn_tiled_kernel(const KArgs a, int
                          kro + (kc ^ kswz(q + 3)), kdst + q * 1024);
 #pragma unroll
       for (int q = 0; q < VP; q += 4) load_to_lds16_x4(vb + q * 1024, voff, voff, voff, voff, vdst + q * 1024);
-    } else if (s < n_sb) {
+    } else if (decltype(interior)::value || s < n_sb) {
       const int g = a0 + (s - n_c);
-      const int lim = a.n_rows - 1 - 16 * g;  // batch rows past the pass's last row do not exist
+      const int lim = decltype(interior)::value ? 15 : a.n_rows - 1 - 16 * g;  // batch rows past the pass's last row do not exist
       const char* kb = reinterpret_cast<const char*>(a.Kb + size_t(16 * g) * a.kv_ld + size_t(kvh) * HD);
       const char* vb = reinterpret_cast<const char*>(a.vt_stage + (size_t(kvh) * n_groups + g) * size_t(HD) * 16);
       const uint32_t kld = uint32_t(a.kv_ld) * 2;
@@ -619,15 +619,30 @@ __global__ __launch_bounds__(256, OCC) void attn_tiled_kernel(const KArgs a, int
     mma_group.template operator()<NG - 1, 0, GP>(ring[(NG - 1) & 1]);
     __builtin_amdgcn_sched_barrier(0);
   };
-  // Steps [int_lo, int_hi) are interior.
-  int int_lo, int_hi;
+  // Mask-free steps: every key is one that every row of the tile sees and nothing needs fixing up. Two runs
+  // of them: cached steps [int_lo, c_hi) - inside [k0, k1) and inside every row's window - and batch steps
+  // [b_lo, b_hi), whose rows all lie below the tile's first row (and at or above b0, inside every segment,
+  // with no ancestors and no per-key window test pending). Where the cached range ends on a step boundary
+  // the two runs are one. An interior iteration i needs steps i .. i + 2 in one run.
+  int int_lo, c_hi, b_lo = 0, b_hi = 0;
   {
     const int first = c0 << 4;  // key of sub-block 0
     int lo_key = tile.k0;
     if (a.window > 0) lo_key = max(lo_key, qpos_max - a.window + 1);
     int_lo = lo_key <= first ? 0 : (lo_key - first + 63) >> 6;
-    const int full_steps = ((tile.k1 >> 4) - c0) >> 2;  // steps wholly inside the cached range
-    int_hi = min(full_steps - 2, my_steps);
+    c_hi = ((tile.k1 >> 4) - c0) >> 2;  // steps wholly inside the cached range
+    if (n_b > 0 && !batch_window && !anc_any && seg_max != INT32_MAX) {
+      const int lo_b = max(max(tile.b0, seg_max), 0);
+      const int g_lo = (tree.base + lo_b + 15) >> 4;           // first group of 16 rows wholly at or above lo_b
+      const int g_hi = ((tree.base + rr0) >> 4) - 1;           // last group wholly below the tile's first row
+      const int s_lo = n_c + g_lo - a0, s_hi = n_c + g_hi - a0;  // as sub-blocks of the range
+      b_lo = (s_lo + 3) >> 2;
+      b_hi = max(b_lo, (s_hi + 1) >> 2);
+      if (b_lo == c_hi && (n_c & 3) == 0 && (tile.k1 & 15) == 0 && c_hi > int_lo) {  // one run
+        c_hi = b_hi;
+        b_lo = b_hi = 0;
+      }
+    }
   }
   constexpr std::false_type general{};
   constexpr std::true_type inner{};
@@ -641,22 +656,27 @@ __global__ __launch_bounds__(256, OCC) void attn_tiled_kernel(const KArgs a, int
   if (n_steps > 1) fill(1, 1, general);
   read_group.template operator()<0, 0>(ring[0]);
   __builtin_amdgcn_sched_barrier(0);
-  // Pairs of steps (one per stage): general ones up to the interior range, the interior
-  // range, general ones again. The two general stretches share one loop's code.
-  const int in0 = min((int_lo + 1) & ~1, my_steps & ~1);
-  const int in1 = int_hi > in0 ? in0 + ((int_hi - in0) & ~1) : in0;
+  // Pairs of steps (one per stage): general ones up to the first mask-free run, that run, general ones,
+  // the second run, general ones again. The general stretches share one loop's code, and so do the runs.
+  const int even_steps = my_steps & ~1;
+  const int a_hi = min(c_hi - 2, my_steps), bb_hi = min(b_hi - 2, my_steps);  // interior iterations end two steps short of a run
+  const int in0 = min((int_lo + 1) & ~1, even_steps);
+  const int in1 = a_hi > in0 ? in0 + ((a_hi - in0) & ~1) : in0;
+  const int in2 = max(in1, min((b_lo + 1) & ~1, even_steps));
+  const int in3 = bb_hi > in2 ? in2 + ((bb_hi - in2) & ~1) : in2;
   int i = 0;
 #pragma nounroll
-  for (int seg = 0; seg < 2; ++seg) {
-    const int bound = seg == 0 ? in0 : my_steps;
+  for (int seg = 0; seg < 3; ++seg) {
+    const int bound = seg == 0 ? in0 : (seg == 1 ? in2 : my_steps);
 #pragma nounroll
     for (; i + 2 <= bound; i += 2) {
       iter.template operator()<0>(i, general);
       iter.template operator()<1>(i + 1, general);
     }
-    if (seg == 0) {
+    if (seg < 2) {
+      const int end = seg == 0 ? in1 : in3;
 #pragma nounroll
-      for (; i + 2 <= in1; i += 2) {
+      for (; i + 2 <= end; i += 2) {
         iter.template operator()<0>(i, inner);
         iter.template operator()<1>(i + 1, inner);
       }
