@@ -448,12 +448,14 @@ __global__ __launch_bounds__(256, OCC) void attn_tiled_kernel(const KArgs a, int
     }
   };
   // Head dim 256: the straight-line part with the scale and the reference in one fused multiply-add per score.
-  auto softmax_exp_fma = [&](auto kt_c) __attribute__((always_inline)) {
+  // T0 .. T1: which of the half step's two sub-blocks of 16 keys (8 scores of this lane each) to do now: with
+  // two groups of matrix instructions per half step the second sub-block waits for the second group.
+  auto softmax_exp_fma = [&]<int T0, int T1>(auto kt_c) __attribute__((always_inline)) {
     constexpr int kt = decltype(kt_c)::value;
     const float m_safe = (m_run == -INFINITY) ? 0.0f : m_run;
     float ps = 0.0f;
 #pragma unroll
-    for (int t = 0; t < 2; ++t) {
+    for (int t = T0; t < T1; ++t) {
       float p[8];
 #pragma unroll
       for (int e = 0; e < 8; ++e) {
@@ -461,11 +463,12 @@ __global__ __launch_bounds__(256, OCC) void attn_tiled_kernel(const KArgs a, int
         ps += p[e];
       }
       pb[kt][t] = u32x4{pack2<DT>(p[0], p[1]), pack2<DT>(p[2], p[3]), pack2<DT>(p[4], p[5]), pack2<DT>(p[6], p[7])};
+      // Pin the results here: without a use in this block the arithmetic above is sunk to the
+      // block of its first real use, away from the matrix instructions it should overlap with.
+      asm volatile("" : "+v"(pb[kt][t]));
     }
     l_run += ps;
-    // Pin the results here: without a use in this block the arithmetic above is sunk to the
-    // block of its first real use, away from the matrix instructions it should overlap with.
-    asm volatile("" : "+v"(pb[kt][0]), "+v"(pb[kt][1]), "+v"(l_run));
+    asm volatile("" : "+v"(l_run));
   };
   // The straight-line part in eight slices, one pair of scores each: slice q subtracts the reference and
   // takes the exponentials of pair q, and packs and sums pair q - 1, whose exponentials have had a slice's
@@ -568,12 +571,23 @@ __global__ __launch_bounds__(256, OCC) void attn_tiled_kernel(const KArgs a, int
         softmax_pre(step, std::integral_constant<int, G == GK ? 0 : 1>{}, interior);
         __builtin_amdgcn_sched_barrier(0);
         mma_group.template operator()<G, HEAD, GP>(ring[G & 1]);
-        softmax_exp_fma(std::integral_constant<int, G == GK ? 0 : 1>{});
+        constexpr bool TWO = GK >= 2;  // the half step's Q K^T (or P V) is two groups: the second carries the other half
+        softmax_exp_fma.template operator()<0, TWO ? 1 : 2>(std::integral_constant<int, G == GK ? 0 : 1>{});
 #pragma unroll
         for (int j = HEAD; j < GP; ++j) {
           __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
-          __builtin_amdgcn_sched_group_barrier(0x002, 13, 0);
+          __builtin_amdgcn_sched_group_barrier(0x002, TWO ? 7 : 13, 0);
         }
+      }
+    } else if constexpr (!LEAN && GK >= 2 && (G == GK + 1 || G == 2 * GK + 1)) {
+      // the second sub-block's share of the softmax beside the half step's second group of matrix instructions
+      __builtin_amdgcn_sched_barrier(0);
+      mma_group.template operator()<G, 0, GP>(ring[G & 1]);
+      softmax_exp_fma.template operator()<1, 2>(std::integral_constant<int, G == GK + 1 ? 0 : 1>{});
+#pragma unroll
+      for (int j = 0; j < GP; ++j) {
+        __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
+        __builtin_amdgcn_sched_group_barrier(0x002, 4, 0);
       }
     } else {
       __builtin_amdgcn_sched_barrier(0);
