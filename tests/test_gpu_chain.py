@@ -327,3 +327,44 @@ def test_fused_decode_on_seeded_random_shapes_is_prep_then_attention_bit_for_bit
             res.append((O, pool))
         assert torch.equal(res[0][0].view(torch.int16), res[1][0].view(torch.int16)), (it, "output")
         assert torch.equal(res[0][1].view(torch.int16), res[1][1].view(torch.int16)), (it, "pool")
+
+
+def test_fused_decode_without_an_append_and_without_descriptors_leaves_the_pool_alone():
+    """row_table NULL: the rows' K / V take part in the attention but are not written anywhere; desc NULL: plain decode
+    rows. Outputs equal those of esp_attn_prep (no table) + esp_attn_forward, and the pool is untouched."""
+    device.init(0)
+    rng = np.random.default_rng(5)
+    H, Hkv, HD, BT, dtype = 8, 2, 128, 16, abi.ESP_BF16
+    seqs = [(900, 1), (31, 1), (0, 1)]
+    n_rows = len(seqs)
+    ap = synth.make_params(H, Hkv, HD, dtype, BT, rows_per_tile=1)
+    pp, a = synth.make_prep("gemma", H, Hkv, HD, dtype, n_rows, seed=3, bt=BT)
+    nb = [(p + BT - 1) // BT for p, _ in seqs]
+    n_blocks = sum(nb) + 1
+    blocks = rng.permutation(n_blocks).astype(np.int32)[:max(sum(nb), 1)].copy()
+    trees = np.zeros(n_rows, abi.TREE_DT)
+    pos = np.zeros((n_rows, 4), np.int32)
+    off = 0
+    for i, (p, m) in enumerate(seqs):
+        trees[i] = (i, p, off, 1)
+        pos[i, :3] = p
+        off += nb[i]
+    pool0 = (torch.randn(n_blocks * 2 * BT * ap.kv_ld, device="cuda") * 0.5).to(torch.bfloat16)
+    resident, groups = device.plan_hint(ap)
+    tiles, jobs, n_parts = host.plan_tiles(trees, groups, 0, None, host.options_mi355x(1, 32))
+    dp = device.DevicePass(ap, trees, tiles, jobs, n_parts, n_rows, blocks, None, None, pool_blocks=n_blocks)
+    dev = lambda x: None if x is None else torch.from_numpy(np.ascontiguousarray(x)).cuda()  # noqa: E731
+    Xd, qn, kn, posd, inv_freq = dev(a["X"]), dev(a["qn_w"]), dev(a["kn_w"]), dev(pos), dev(a["inv_freq"])
+    pool = pool0.clone()
+    O1 = torch.zeros(n_rows, ap.q_ld, dtype=torch.bfloat16, device="cuda")
+    device.decode_fused(pp, ap, Xd, qn, kn, posd, inv_freq, None, None, pool, dp, O1)
+    torch.cuda.synchronize()
+    assert torch.equal(pool.view(torch.int16), pool0.view(torch.int16))
+    Q = torch.zeros(n_rows, ap.q_ld, dtype=torch.bfloat16, device="cuda")
+    Kb = torch.zeros(n_rows, ap.kv_ld, dtype=torch.bfloat16, device="cuda")
+    Vb = torch.zeros_like(Kb)
+    O2 = torch.zeros_like(O1)
+    device.attn_prep(pp, Xd, qn, kn, posd, inv_freq, None, Q, Kb, Vb, None, None, n_rows)
+    dp.run(Q, Kb, Vb, pool, O2)
+    torch.cuda.synchronize()
+    assert bool(O1.any()) and torch.equal(O1.view(torch.int16), O2.view(torch.int16))
