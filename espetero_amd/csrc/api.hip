@@ -10,7 +10,7 @@
 
 namespace esp {
 hipError_t launch_stream(int dt, int HD, int NC, const KArgs& a, const PrepArgs* pa, int n_tiles, hipStream_t st);
-hipError_t launch_combine(int dt, int HD, const KArgs& a, const esp_combine* jobs, int n_jobs, hipStream_t st);
+hipError_t launch_combine(int dt, int HD, const KArgs& a, const esp_combine* jobs, int n_jobs, int n_parts, hipStream_t st);
 hipError_t launch_tiled(int dt, int HD, const KArgs& a, int n_tiles, hipStream_t st);
 hipError_t launch_kv_save(const esp_attn_params* p, const void* Kb, const void* Vb, void* pool, const esp_kvsave* e, int n,
                           hipStream_t st);
@@ -284,7 +284,7 @@ static int forward_impl(const esp_attn_params* p, const void* Q, const void* Kb,
     if (e != hipSuccess) return hip_fail(err, errlen, "attn_tiled launch", e);
   }
   if (n_jobs > 0) {
-    e = esp::launch_combine(p->dtype, p->head_dim, a, jobs, n_jobs, st);
+    e = esp::launch_combine(p->dtype, p->head_dim, a, jobs, n_jobs, n_parts, st);
     if (e != hipSuccess) return hip_fail(err, errlen, "attn_combine launch", e);
   }
   return ESP_OK;
@@ -405,7 +405,7 @@ int esp_attn_combine(const esp_attn_params* p, void* O, const esp_combine* jobs,
   if (reinterpret_cast<uintptr_t>(workspace) % 16) return fail(err, errlen, ESP_EINVAL, "workspace must be 16-byte aligned");
   esp::KArgs a = make_args(p, c, workspace, n_rows);
   a.O = static_cast<uint16_t*>(O);
-  hipError_t e = esp::launch_combine(p->dtype, p->head_dim, a, jobs, n_jobs, static_cast<hipStream_t>(stream));
+  hipError_t e = esp::launch_combine(p->dtype, p->head_dim, a, jobs, n_jobs, n_parts, static_cast<hipStream_t>(stream));
   return e == hipSuccess ? ESP_OK : hip_fail(err, errlen, "attn_combine launch", e);
 }
 

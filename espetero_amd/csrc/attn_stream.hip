@@ -40,13 +40,16 @@ namespace esp {
 // Merge of the partial records of one split tile group for 4 dims of one (row, query head), in part
 // order (attention_combine, kernels/40_attention.metal:811-864; kernels/80_gemma.metal:568-597), then
 // the normalised (optionally gated) output.
-template <int DT, int HD>
-__device__ __forceinline__ void merge_records(const KArgs& a, const esp_combine& job, int r, int h, int d) {
+// LP lanes share one output (consecutive lanes of a wavefront, `lp` = this lane's place among them): lane lp
+// merges records lp, lp + LP, .. in that order, and the LP running triples (max, sum, O) are then merged pairwise
+// across the lanes. One lane (LP = 1) is the plain merge in part order.
+template <int DT, int HD, int LP = 1>
+__device__ __forceinline__ void merge_records(const KArgs& a, const esp_combine& job, int r, int h, int d, int lp = 0) {
   const int kvh = h / a.G, hg = h - kvh * a.G;
   const int col = r * a.G + hg;
   const size_t stride = size_t(a.Hkv) * a.cols;  // records from one part to the next
   const size_t rec0 = (size_t(job.part0) * a.Hkv + kvh) * a.cols + col;
-  // One pass, 8 records in flight at a time, merged in part order with a running maximum
+  // One pass, up to 32 records in flight at a time, merged in part order with a running maximum
   // (a loop that waits for each record's loads in turn is latency bound: the reference
   // measured 39 us against 11 us for the same change, 40_attention.metal:801-803).
   float M = -INFINITY, L = 0.0f;
@@ -58,8 +61,8 @@ __device__ __forceinline__ void merge_records(const KArgs& a, const esp_combine&
     f32x4 oN[N];
 #pragma unroll
     for (int i = 0; i < N; ++i) {
-      const bool in = s + i < job.nparts;
-      const size_t rec = rec0 + size_t(in ? s + i : s) * stride;
+      const bool in = s + i * LP < job.nparts;
+      const size_t rec = rec0 + size_t(in ? s + i * LP : min(s, job.nparts - 1)) * stride;
       mN[i] = in ? a.parts_ml[rec * 2] : -INFINITY;
       lN[i] = a.parts_ml[rec * 2 + 1];
       oN[i] = *reinterpret_cast<const f32x4*>(a.parts_o + rec * HD + d);
@@ -78,10 +81,32 @@ __device__ __forceinline__ void merge_records(const KArgs& a, const esp_combine&
       o += oN[i] * w;
     }
   };
-  if (job.nparts <= 2) {  // the split of a prefill tile: two records, nothing to repeat
+  // As many records in flight as the group has, in four sizes: every round of loads is a memory latency, and a
+  // finely split sequence (a single long one has dozens of parts) would otherwise pay one per 8 records.
+  if constexpr (LP > 1) {
+    for (int s = lp; s < job.nparts; s += 4 * LP) merge(s, std::integral_constant<int, 4>{});
+    // pairwise across the LP lanes; a + b == b + a, so both lanes of a pair go on with the same triple
+#pragma unroll
+    for (int off = 1; off < LP; off <<= 1) {
+      const float M2 = __shfl_xor(M, off), L2 = __shfl_xor(L, off);
+      f32x4 o2;
+#pragma unroll
+      for (int e = 0; e < 4; ++e) o2[e] = __shfl_xor(o[e], off);
+      const float Mn = fmaxf(M, M2);
+      const float c1 = (M == -INFINITY) ? 0.0f : fast_exp2(M - Mn), c2 = (M2 == -INFINITY) ? 0.0f : fast_exp2(M2 - Mn);
+      L = L * c1 + L2 * c2;
+      o = o * c1 + o2 * c2;
+      M = Mn;
+    }
+    if (lp != 0) return;
+  } else if (job.nparts <= 2) {  // the split of a prefill tile: two records, nothing to repeat
     merge(0, std::integral_constant<int, 2>{});
+  } else if (job.nparts <= 8) {
+    merge(0, std::integral_constant<int, 8>{});
+  } else if (job.nparts <= 16) {
+    merge(0, std::integral_constant<int, 16>{});
   } else {
-    for (int s = 0; s < job.nparts; s += 8) merge(s, std::integral_constant<int, 8>{});
+    for (int s = 0; s < job.nparts; s += 32) merge(s, std::integral_constant<int, 32>{});
   }
   const int row = job.r0 + r;
   const float inv = L > 0.0f ? 1.0f / L : 0.0f;
@@ -596,11 +621,15 @@ __global__ __launch_bounds__(HD >= 512 ? 128 : 256, OCC) void attn_stream_kernel
   }
 }
 
-// The merge as its own dispatch: one thread per (job, row, head, 4 dims).
-template <int DT, int HD>
+// The merge as its own dispatch: LP threads per (job, row, head, 4 dims). One thread each is what a pass of many
+// tile groups wants; a pass of few groups with many parts each (one long sequence decoded alone: 1024 outputs of 65
+// records) would leave all but a handful of compute units idle, so there 8 lanes share an output.
+template <int DT, int HD, int LP>
 __global__ __launch_bounds__(256) void attn_combine_kernel(const KArgs a, const esp_combine* jobs, int n_jobs) {
   const int per_job = a.R * a.H * (HD / 4);
-  const long gid = long(blockIdx.x) * 256 + threadIdx.x;
+  const long tid_g = long(blockIdx.x) * 256 + threadIdx.x;
+  const long gid = tid_g / LP;
+  const int lp = int(tid_g % LP);
   if (gid >= long(n_jobs) * per_job) return;
   const int ji = int(gid / per_job);
   int rem = int(gid % per_job);
@@ -609,7 +638,7 @@ __global__ __launch_bounds__(256) void attn_combine_kernel(const KArgs a, const 
   const int h = rem / (HD / 4), d = (rem % (HD / 4)) * 4;
   const esp_combine job = jobs[ji];
   if (r >= job.rows) return;
-  merge_records<DT, HD>(a, job, r, h, d);
+  merge_records<DT, HD, LP>(a, job, r, h, d, lp);
 }
 
 size_t stream_smem_bytes(int HD, int NC) {
@@ -686,15 +715,24 @@ hipError_t launch_stream(int dt, int HD, int NC, const KArgs& a, const PrepArgs*
   return hipErrorInvalidValue;
 }
 
-hipError_t launch_combine(int dt, int HD, const KArgs& a, const esp_combine* jobs, int n_jobs, hipStream_t st) {
+template <int DT, int HD>
+static void launch_combine_t(const KArgs& a, const esp_combine* jobs, int n_jobs, int n_parts, hipStream_t st) {
   const long n = long(n_jobs) * a.R * a.H * (HD / 4);
-  const dim3 grid((unsigned)((n + 255) / 256));
-  if (dt == ESP_F16 && HD == 128) hipLaunchKernelGGL((attn_combine_kernel<ESP_F16, 128>), grid, dim3(256), 0, st, a, jobs, n_jobs);
-  else if (dt == ESP_F16 && HD == 256) hipLaunchKernelGGL((attn_combine_kernel<ESP_F16, 256>), grid, dim3(256), 0, st, a, jobs, n_jobs);
-  else if (dt == ESP_BF16 && HD == 128) hipLaunchKernelGGL((attn_combine_kernel<ESP_BF16, 128>), grid, dim3(256), 0, st, a, jobs, n_jobs);
-  else if (dt == ESP_BF16 && HD == 256) hipLaunchKernelGGL((attn_combine_kernel<ESP_BF16, 256>), grid, dim3(256), 0, st, a, jobs, n_jobs);
-  else if (dt == ESP_F16 && HD == 512) hipLaunchKernelGGL((attn_combine_kernel<ESP_F16, 512>), grid, dim3(256), 0, st, a, jobs, n_jobs);
-  else if (dt == ESP_BF16 && HD == 512) hipLaunchKernelGGL((attn_combine_kernel<ESP_BF16, 512>), grid, dim3(256), 0, st, a, jobs, n_jobs);
+  // more than 8 records per group on average and few outputs: share each output among 8 lanes
+  if (n_parts > 8 * n_jobs && n * 8 <= (1L << 22)) {
+    hipLaunchKernelGGL((attn_combine_kernel<DT, HD, 8>), dim3((unsigned)((n * 8 + 255) / 256)), dim3(256), 0, st, a, jobs, n_jobs);
+  } else {
+    hipLaunchKernelGGL((attn_combine_kernel<DT, HD, 1>), dim3((unsigned)((n + 255) / 256)), dim3(256), 0, st, a, jobs, n_jobs);
+  }
+}
+
+hipError_t launch_combine(int dt, int HD, const KArgs& a, const esp_combine* jobs, int n_jobs, int n_parts, hipStream_t st) {
+  if (dt == ESP_F16 && HD == 128) launch_combine_t<ESP_F16, 128>(a, jobs, n_jobs, n_parts, st);
+  else if (dt == ESP_F16 && HD == 256) launch_combine_t<ESP_F16, 256>(a, jobs, n_jobs, n_parts, st);
+  else if (dt == ESP_BF16 && HD == 128) launch_combine_t<ESP_BF16, 128>(a, jobs, n_jobs, n_parts, st);
+  else if (dt == ESP_BF16 && HD == 256) launch_combine_t<ESP_BF16, 256>(a, jobs, n_jobs, n_parts, st);
+  else if (dt == ESP_F16 && HD == 512) launch_combine_t<ESP_F16, 512>(a, jobs, n_jobs, n_parts, st);
+  else if (dt == ESP_BF16 && HD == 512) launch_combine_t<ESP_BF16, 512>(a, jobs, n_jobs, n_parts, st);
   else return hipErrorInvalidValue;
   return hipGetLastError();
 }
