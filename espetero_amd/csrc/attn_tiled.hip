@@ -88,19 +88,16 @@ __global__ __launch_bounds__(256, OCC) void attn_tiled_kernel(const KArgs a, int
   const int rr = rr0 + m_row;
   const int4 d = a.desc ? a.desc[row] : make_int4(0, 0, 0, 0);
   const int qpos = a.window > 0 ? a.pos[row].x : 0;
-  // Q fragments; on the lean path multiplied once by scale * log2(e) and rounded back to the storage type:
-  // the matrix instructions then deliver scores in the log2 units the softmax works in, and no vector
-  // instruction per score is spent on the scale.
+  // Q fragments as stored. The scale (times log2 e) is applied to the fp32 score in the same fused
+  // multiply-add that subtracts the row's reference: multiplying Q itself and rounding it back to the
+  // storage type would cost every score a relative 2^-9 (bf16) before the exponential, which at logits
+  // of a few units is more than the 2e-3 the path promises (the reference pre-scales Q only by an
+  // exact power of two, kernels/40_attention.metal:195-200).
   u32x4 qf[KS];
   {
     const uint16_t* qp = a.Q + size_t(row) * a.q_ld + size_t(h) * HD + 8 * hb;
 #pragma unroll
-    for (int ks = 0; ks < KS; ++ks) {
-      const u32x4 q = row_ok ? *reinterpret_cast<const u32x4*>(qp + 16 * ks) : u32x4{0, 0, 0, 0};
-#pragma unroll
-      for (int e = 0; e < 4; ++e)
-        qf[ks][e] = LEAN ? pack2<DT>(unpack_lo<DT>(q[e]) * a.scale_log2, unpack_hi<DT>(q[e]) * a.scale_log2) : q[e];
-    }
+    for (int ks = 0; ks < KS; ++ks) qf[ks] = row_ok ? *reinterpret_cast<const u32x4*>(qp + 16 * ks) : u32x4{0, 0, 0, 0};
   }
 
   // ---- tile-wide facts about the rows (for the batch range and the no-mask fast path)
@@ -280,12 +277,9 @@ __global__ __launch_bounds__(256, OCC) void attn_tiled_kernel(const KArgs a, int
   auto lds_ptr = [](uint32_t addr) __attribute__((always_inline)) { return reinterpret_cast<lds_u32x4*>(addr); };
 
   f32x16 acc[NT];
-  // The row's running reference m_run (log2 units; -inf: no key seen yet), kept a second time as 16
-  // registers of -m_run (0 while there is none): the block a score tile's first matrix instruction takes
-  // as its addend, so that the scores arrive already relative to the reference.
+  // The row's running reference m_run (log2 units of the scaled score; -inf: no key seen yet).
   // l_run: this lane's share (16 of every 32 keys) of the row's sum. p_limit: what a half step's share
   // of the sum may reach before the reference has to move (-1: it has to be set first).
-  // owed: what the reference moved by after the second half step's score tile had been started.
   float m_run = -INFINITY, l_run = 0.0f, p_limit = -1.0f;
 #pragma unroll
   for (int nt = 0; nt < NT; ++nt)
@@ -346,9 +340,15 @@ __global__ __launch_bounds__(256, OCC) void attn_tiled_kernel(const KArgs a, int
 
   // Online softmax of half step (step, kt) in three parts.
   //   softmax_pre     the masks (nothing on the mask-free path); branchy.
-  //   softmax_exp     straight-line: P = exp2(S) - the scores are already relative to the reference - packed
-  //                   to the storage type, and the lane's share of the row sum, taken from the packed P two
-  //                   at a time (v_dot2: the sum is that of the rounded P the products use). No maximum is
+  //   softmax_exp     straight-line: P = exp2(S * scale - m_run), one fused multiply-add and one exponential
+  //                   per score, packed to the storage type, and the lane's share of the row sum, taken from
+  //                   the packed P two at a time (v_dot2 against (1, 1), fp32 accumulation): the sum is that
+  //                   of the rounded P the products use, so O = sum(P~ v) / sum(P~) and a row that one key
+  //                   dominates returns that key's V whatever P~ was rounded to. The reference sums the
+  //                   unrounded P (kernels/40_attention.metal:292-297) against an exact running maximum,
+  //                   where the dominant P is exactly 1 and carries no rounding; under a reference that
+  //                   moves lazily the dominant P is any number up to 2^8, and summing the unrounded P would
+  //                   leave its rounding (2^-9 relative on bf16) in the output. No maximum is
   //                   taken: all P >= 0, so a share <= 2^8 bounds every one of them, P fits its 16 bits and
   //                   the accumulators need no rescaling. This is the code the scheduler lays between the
   //                   matrix instructions of the next group: one v_exp and one and a half other vector
@@ -458,11 +458,10 @@ __global__ __launch_bounds__(256, OCC) void attn_tiled_kernel(const KArgs a, int
     for (int t = T0; t < T1; ++t) {
       float p[8];
 #pragma unroll
-      for (int e = 0; e < 8; ++e) {
-        p[e] = fast_exp2(__builtin_fmaf(s[kt][8 * t + e], a.scale_log2, -m_safe));
-        ps += p[e];
-      }
+      for (int e = 0; e < 8; ++e) p[e] = fast_exp2(__builtin_fmaf(s[kt][8 * t + e], a.scale_log2, -m_safe));
       pb[kt][t] = u32x4{pack2<DT>(p[0], p[1]), pack2<DT>(p[2], p[3]), pack2<DT>(p[4], p[5]), pack2<DT>(p[6], p[7])};
+#pragma unroll
+      for (int e = 0; e < 4; ++e) ps = sum2<DT>(pb[kt][t][e], ps);  // the sum of the P the products use (see slice_pack)
       // Pin the results here: without a use in this block the arithmetic above is sunk to the
       // block of its first real use, away from the matrix instructions it should overlap with.
       asm volatile("" : "+v"(pb[kt][t]));
@@ -479,16 +478,16 @@ __global__ __launch_bounds__(256, OCC) void attn_tiled_kernel(const KArgs a, int
     uint32_t w = pack2<DT>(pv[2 * Q], pv[2 * Q + 1]);
     asm volatile("" : "+v"(w));  // packed here, not sunk to the block of its first use
     pb[KT][Q / 4][Q % 4] = w;
-    if constexpr (Q & 1) ps1 += pv[2 * Q] + pv[2 * Q + 1];
-    else ps0 += pv[2 * Q] + pv[2 * Q + 1];
+    if constexpr (Q & 1) ps1 = sum2<DT>(w, ps1);
+    else ps0 = sum2<DT>(w, ps0);
   };
   auto slice = [&]<int KT, int Q>() __attribute__((always_inline)) {
     if constexpr (Q == 0) {
       ps0 = ps1 = 0.0f;
       m_sub = (m_run == -INFINITY) ? 0.0f : m_run;
     }
-    pv[2 * Q] = fast_exp2(s[KT][2 * Q] - m_sub);
-    pv[2 * Q + 1] = fast_exp2(s[KT][2 * Q + 1] - m_sub);
+    pv[2 * Q] = fast_exp2(__builtin_fmaf(s[KT][2 * Q], a.scale_log2, -m_sub));
+    pv[2 * Q + 1] = fast_exp2(__builtin_fmaf(s[KT][2 * Q + 1], a.scale_log2, -m_sub));
     if constexpr (Q > 0) slice_pack.template operator()<KT, Q - 1>();
   };
   auto softmax_finish = [&]<int KT>() __attribute__((always_inline)) -> float {
@@ -512,6 +511,7 @@ __global__ __launch_bounds__(256, OCC) void attn_tiled_kernel(const KArgs a, int
       float x = -INFINITY;
 #pragma unroll
       for (int i = 0; i < 16; ++i) x = fmaxf(x, sv[i]);
+      x *= a.scale_log2;  // scale > 0: the max commutes with it
       const float m_new = fmaxf(m_run, fmaxf(x, __shfl_xor(x, 32)));
       const float corr = (m_run == -INFINITY) ? 1.0f : fast_exp2(m_run - m_new);
       m_run = m_new;

@@ -290,11 +290,12 @@ __global__ __launch_bounds__(256, 1) void attn_tiled512_kernel(const KArgs a, in
     for (int t = 0; t < 2; ++t) {
       float p[8];
 #pragma unroll
-      for (int e = 0; e < 8; ++e) {
-        p[e] = fast_exp2(__builtin_fmaf(s[8 * t + e], a.scale_log2, -m_safe));
-        ps += p[e];
-      }
+      for (int e = 0; e < 8; ++e) p[e] = fast_exp2(__builtin_fmaf(s[8 * t + e], a.scale_log2, -m_safe));
       pb[t] = u32x4{pack2<DT>(p[0], p[1]), pack2<DT>(p[2], p[3]), pack2<DT>(p[4], p[5]), pack2<DT>(p[6], p[7])};
+      // The row sum is that of the rounded P the products use: under a lazily moved reference the dominant P is
+      // not exactly 1, and O = sum(P~ v) / sum(P~) keeps its rounding out of a row that one key dominates.
+#pragma unroll
+      for (int e = 0; e < 4; ++e) ps = sum2<DT>(pb[t][e], ps);
     }
     l_run += ps;
     __builtin_amdgcn_sched_barrier(0);

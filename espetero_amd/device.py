@@ -195,16 +195,28 @@ class DevicePass:
         self.pos = to_dev(np.ascontiguousarray(pos, dtype=np.int32), device) if pos is not None else None
         nbytes = workspace_bytes(params, n_rows, n_parts)
         self.workspace = None if static else torch.empty(nbytes, dtype=torch.uint8, device=device)
+        self._key, self._fn, self._args, self._err = None, None, None, C.create_string_buffer(_ERRLEN)
 
     def run(self, Q, Kb, Vb, pool, O, stream=None, merge=True):
-        if self.static:
-            forward_static(self.params, Q, Kb, Vb, pool, self.blocks, self.desc, self.pos, O, self.tiles, self.n_tiles,
-                           self.trees, self.n_trees, self.jobs if merge else None, self.n_jobs if merge else 0, self.n_parts,
-                           self.n_rows, stream)
-            return
-        forward(self.params, Q, Kb, Vb, pool, self.blocks, self.desc, self.pos, O, self.tiles, self.n_tiles, self.trees,
-                self.n_trees, self.jobs if merge else None, self.n_jobs if merge else 0, self.n_parts, self.n_rows,
-                self.workspace, stream)
+        """Enqueues the pass. The ctypes argument list is built once per set of buffers and reused: a decode step is
+        tens of microseconds on the GPU, and rebuilding twenty pointer objects per call costs the host as much."""
+        st = torch.cuda.current_stream().cuda_stream if stream is None else stream.cuda_stream
+        key = (Q.data_ptr(), Kb.data_ptr(), Vb.data_ptr(), pool.data_ptr(), O.data_ptr(), st, merge,
+               None if self.pos is None else self.pos.data_ptr())
+        if self._key != key:
+            jobs, n_jobs = (self.jobs, self.n_jobs) if merge else (None, 0)
+            head = [C.byref(self.params), _ptr(Q), _ptr(Kb), _ptr(Vb), _ptr(pool), _ptr(self.blocks), _ptr(self.desc), _ptr(self.pos),
+                    _ptr(O), _ptr(self.tiles), self.n_tiles, _ptr(self.trees), self.n_trees, _ptr(jobs), n_jobs, self.n_parts, self.n_rows]
+            if self.static:
+                self._fn, self._args = abi.attn_lib().esp_attn_forward_static, head + [C.c_void_p(st), self._err, _ERRLEN]
+            else:
+                ws = self.workspace
+                self._fn = abi.attn_lib().esp_attn_forward
+                self._args = head + [_ptr(ws), ws.numel() * ws.element_size(), C.c_void_p(st), self._err, _ERRLEN]
+            self._key = key
+        rc = self._fn(*self._args)
+        if rc:
+            abi.check(rc, self._err)
 
     def merge(self, O, stream=None):
         if self.n_jobs:

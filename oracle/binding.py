@@ -41,6 +41,25 @@ def _p(a):
     return None if a is None else a.ctypes.data_as(C.c_void_p)
 
 
+TOL = 2e-3  # max-abs contract of the path (fp32 accumulation, fp16 / bf16 storage)
+
+
+def bf16_ulp(x):
+    """One unit in the last place of a bf16 number of x's magnitude: 8 significant bits, 2^(floor(log2 |x|) - 7)."""
+    ax = np.maximum(np.abs(np.asarray(x, np.float64)), 2.0 ** -126)
+    return 2.0 ** (np.floor(np.log2(ax)) - 7)
+
+
+def beyond_rounding(got, want, dtype, want_rounded):
+    """Largest |got - want| once the rounding of the stored output itself is taken off: nothing for fp16 (half a unit
+    in the last place of an output below 1 is 2.4e-4, inside the bar), and for bf16 half a unit in the last place
+    against an unrounded expectation, a whole unit against one that was itself rounded to bf16 (two results a hair
+    apart may round to neighbouring bf16 numbers). The one bar every comparison of this path uses is TOL on this."""
+    got, want = np.asarray(got, np.float64), np.asarray(want, np.float64).reshape(np.shape(got))
+    allow = 0.0 if dtype == abi.ESP_F16 else bf16_ulp(np.maximum(np.abs(got), np.abs(want))) * (1.0 if want_rounded else 0.5)
+    return float(np.maximum(np.abs(got - want) - allow, 0.0).max())
+
+
 def _u16(a):
     a = np.ascontiguousarray(a)
     assert a.dtype == np.uint16

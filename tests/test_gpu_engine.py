@@ -100,7 +100,7 @@ class Served:
         dp.run(Qd, Kd, Vd, self.pool, O)
         torch.cuda.synchronize()
         want = ob.attn_direct(ap, Q, Kb, Vb, self.pool_ref, blocks, ps["desc"], ps["pos"], ps["trees"], n_threads=8)
-        err = float(np.abs(f32(to_host_u16(O).reshape(M, -1), dtype) - f32(want, dtype)).max())
+        err = beyond_rounding(f32(to_host_u16(O).reshape(M, -1), dtype), f32(want, dtype), dtype, True)
         assert err <= self.tol, (tag, err)
         if self.W:                                                 # the same rows through the sliding layer
             rg = e.pass_rings(self.W, self.rb)
@@ -116,7 +116,7 @@ class Served:
             dps.run(Qsd, Ksd, Vsd, self.ring, Os)
             torch.cuda.synchronize()
             want = ob.attn_direct(aps, Qs, Kbs, Vbs, self.ring_ref, np.zeros(1, np.int32), ps["desc"], ps["pos"], rg["trees"], n_threads=8)
-            err = float(np.abs(f32(to_host_u16(Os).reshape(M, -1), dtype) - f32(want, dtype)).max())
+            err = beyond_rounding(f32(to_host_u16(Os).reshape(M, -1), dtype), f32(want, dtype), dtype, True)
             assert err <= self.tol, (tag, "sliding", err)
             if commit and len(rg["saves"]):
                 device.kv_save(aps, Ksd, Vsd, self.ring, device.to_dev(rg["saves"]), len(rg["saves"]))
@@ -322,7 +322,7 @@ def test_noncausal_root_through_the_engine(H, Hkv, HD, M, rows_per_tile, dtype):
     e.pass_abort()
     got = f32(to_host_u16(O).reshape(M, -1), dtype).astype(np.float64)
     want = ob.attn_direct(ap, Q, Kb, Vb, np.zeros(8 * 2 * 16 * ap.kv_ld, np.uint16), blocks, ps["desc"], ps["pos"], ps["trees"], n_threads=4)
-    assert np.abs(got - f32(want, dtype)).max() <= tol_for(dtype)
+    assert beyond_rounding(got, f32(want, dtype), dtype, True) <= tol_for(dtype)
     q = f32(Q, dtype).astype(np.float64).reshape(M, H, HD)
     k = f32(Kb, dtype).astype(np.float64).reshape(M, Hkv, HD)
     v = f32(Vb, dtype).astype(np.float64).reshape(M, Hkv, HD)

@@ -188,7 +188,7 @@ def test_c3_chunked_prefill_equals_one_pass_and_brute_force_rows():
         device.kv_save(p, Kb, Vb, pool, device.to_dev(saves), len(saves))
     torch.cuda.synchronize()
     a, b = _f32(whole), _f32(chunked)
-    assert np.abs(a - b).max() <= 4e-3          # two bf16 computations: probabilities and outputs rounded on each side
+    assert beyond_rounding(a, b, abi.ESP_BF16, True) <= 2e-3   # two bf16 results: one unit in the last place of the stored output is taken off first
     # sampled rows against float64 (K / V of the whole sequence are the batch rows themselves)
     q = _f32(Q).astype(np.float64).reshape(N, H, HD)
     k = _f32(Kb).astype(np.float64).reshape(N, Hkv, HD)

@@ -2,7 +2,7 @@
 type, page size, decode / verify / chunk / prefill / image passes, windows over lists and rings, split
 targets, head-wise gates. Each case is small enough for the checker; together they reach corners the
 hand-written cases do not (two defects were found this way: a partial 16-key unit at head dim 256, a
-one-row remainder tile on a sliding layer). Bar: helpers.tol_for (2e-3; 4e-3 between two bf16 computations)."""
+one-row remainder tile on a sliding layer). Bar: 2e-3 beyond the stored output's own rounding (helpers.max_abs)."""
 import numpy as np
 import pytest
 import torch
