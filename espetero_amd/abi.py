@@ -11,7 +11,8 @@ import numpy as np
 
 ESP_F16, ESP_BF16 = 0, 1
 ESP_LAYOUT_REFERENCE, ESP_LAYOUT_NATIVE = 0, 1
-ESP_ABI_VERSION = 2
+ESP_ABI_VERSION = 3
+ESP_PASS_FUSED, ESP_PASS_ROWS_IN_POOL = 1, 2
 ESP_STATIC_SCRATCH_BYTES = 32 << 20
 
 _PKG_DIR = os.path.dirname(os.path.abspath(__file__))
@@ -86,6 +87,8 @@ ATTN_SYMBOLS = {
                                           C.c_int32, C.c_int32, _V) + _ERR),
     "esp_attn_validate": (C.c_int, (_P, _V, C.c_int32, _V, C.c_int32, _V, C.c_int32, C.c_int32, C.c_int32, _V, C.c_int32,
                                     C.c_int32) + _ERR),
+    "esp_attn_validate_for": (C.c_int, (_P, C.c_int32, _V, C.c_int32, _V, C.c_int32, _V, C.c_int32, C.c_int32, C.c_int32, _V, C.c_int32,
+                                        C.c_int32) + _ERR),
     "esp_attn_time_next": (C.c_int, (_V, _V)),
     "esp_attn_combine": (C.c_int, (_P, _V, _V, C.c_int32, C.c_int32, C.c_int32, _V, C.c_size_t, _V) + _ERR),
     "esp_kv_save": (C.c_int, (_P, _V, _V, _V, _V, C.c_int32, _V) + _ERR),

@@ -127,6 +127,12 @@ esp::KArgs make_args(const esp_attn_params* p, const Carve& c, void* workspace, 
   return a;
 }
 
+// A pending event pair (esp_attn_time_next) belongs to the next call that could have used it, whatever becomes of
+// that call: one that launches nothing or fails its checks must not leave it armed for some later launch.
+struct DropPair {
+  ~DropPair() { (void)esp::take_time_next(); }
+};
+
 constexpr int kMaxDevices = 64;
 struct DeviceState {
   unsigned char* scratch = nullptr;  // this device's copy of `scratch`
@@ -221,15 +227,13 @@ static int forward_impl(const esp_attn_params* p, const void* Q, const void* Kb,
                         int32_t n_tiles, const esp_tree* trees, int32_t n_trees, const esp_combine* jobs, int32_t n_jobs,
                         int32_t n_parts, int32_t n_rows, void* workspace, size_t workspace_bytes, bool own_scratch,
                         const esp::PrepArgs* prep, void* stream, char* err, size_t errlen) {
-  // A pending event pair belongs to this call whatever becomes of it: a call that launches nothing
-  // must not leave it armed for some later launch.
-  struct DropPair {
-    ~DropPair() { (void)esp::take_time_next(); }
-  } drop_pair;
+  DropPair drop_pair;
   if (int rc = check_params(p, err, errlen)) return rc;
   if (n_tiles < 0 || n_trees < 0 || n_jobs < 0 || n_parts < 0 || n_rows < 0) return fail(err, errlen, ESP_EINVAL, "negative count");
   if (n_tiles == 0) return ESP_OK;
-  if ((!prep && (!Q || !Kb || !Vb)) || !O || !tiles || !trees) return fail(err, errlen, ESP_EINVAL, "Q, Kb, Vb, O, tiles, trees must not be NULL");
+  if ((!prep && !Q) || !O || !tiles || !trees) return fail(err, errlen, ESP_EINVAL, "Q, O, tiles, trees must not be NULL");
+  if (!prep && ((Kb == nullptr) != (Vb == nullptr))) return fail(err, errlen, ESP_EINVAL, "Kb and Vb: both, or neither (the pass's rows are read from the pool)");
+  const bool rows_in_pool = !prep && !Kb;
   if (n_trees == 0) return fail(err, errlen, ESP_EINVAL, "%d tiles without trees", n_tiles);
   if (!kv_pool) return fail(err, errlen, ESP_EINVAL, "kv_pool is NULL");
   if (!p->ring && !blocks) return fail(err, errlen, ESP_EINVAL, "blocks is NULL on a layer without rings");
@@ -276,7 +280,7 @@ static int forward_impl(const esp_attn_params* p, const void* Q, const void* Kb,
     e = esp::launch_stream(p->dtype, p->head_dim, fam, a, prep, n_tiles, st);
     if (e != hipSuccess) return hip_fail(err, errlen, "attn_stream launch", e);
   } else {
-    if (n_rows > 0) {
+    if (n_rows > 0 && !rows_in_pool) {
       e = esp::launch_vt_stage(p, Vb, a.vt_stage, n_rows, st);
       if (e != hipSuccess) return hip_fail(err, errlen, "vt_stage launch", e);
     }
@@ -381,6 +385,58 @@ int esp_attn_validate(const esp_attn_params* p, const esp_tile* tiles, int32_t n
     for (int q = 0; q < n_parts; ++q)
       if (part_job[size_t(q)] >= 0 && !part_written[size_t(q)])
         return fail(err, errlen, ESP_EINVAL, "job %d merges partial record %d, which no tile writes", part_job[size_t(q)], q);
+  return ESP_OK;
+}
+
+int esp_attn_validate_for(const esp_attn_params* p, int32_t mode, const esp_tile* tiles, int32_t n_tiles, const esp_tree* trees,
+                          int32_t n_trees, const esp_combine* jobs, int32_t n_jobs, int32_t n_parts, int32_t n_rows, const int32_t* blocks,
+                          int32_t n_block_entries, int32_t pool_blocks, char* err, size_t errlen) {
+  if (int rc = esp_attn_validate(p, tiles, n_tiles, trees, n_trees, jobs, n_jobs, n_parts, n_rows, blocks, n_block_entries, pool_blocks,
+                                 err, errlen))
+    return rc;
+  if (mode & ~(ESP_PASS_FUSED | ESP_PASS_ROWS_IN_POOL)) return fail(err, errlen, ESP_EINVAL, "mode %d", mode);
+  if (mode & ESP_PASS_FUSED) {
+    if (p->head_dim == 512 || p->rows_per_tile > 4 || family(p) <= 0)
+      return fail(err, errlen, ESP_EUNSUPPORTED, "rows_per_tile %d at head_dim %d: the fused decode takes trees of 1 to 4 rows on the streaming kernel, head dim 128 or 256",
+                  p->rows_per_tile, p->head_dim);
+    // The fused kernel prepares the rows of its own tile only and reads a tree's batch keys from that tile's LDS
+    // area: a tree is one tile group, whose first row is the tree's first row.
+    for (int i = 0; i < n_trees; ++i)
+      if (trees[i].M > p->rows_per_tile)
+        return fail(err, errlen, ESP_EINVAL, "tree %d: %d rows; a fused pass takes trees of at most rows_per_tile = %d rows", i, trees[i].M,
+                    p->rows_per_tile);
+    for (int i = 0; i < n_tiles; ++i)
+      if (tiles[i].r0 != trees[tiles[i].tree].base)
+        return fail(err, errlen, ESP_EINVAL, "tile %d: first row %d is not its tree's first row %d (a fused pass has one tile group per tree)", i,
+                    tiles[i].r0, trees[tiles[i].tree].base);
+  }
+  if (mode & ESP_PASS_ROWS_IN_POOL) {
+    // Row j of a tree is read at position P + j of the tree's own block list (or ring).
+    const int64_t bt = p->bt;
+    for (int i = 0; i < n_trees; ++i) {
+      const esp_tree& t = trees[i];
+      if (t.M == 0) continue;
+      if (family(p) < 0 && (t.P - t.base) % 16)
+        return fail(err, errlen, ESP_EINVAL, "tree %d: P %d - base %d is no multiple of 16: the tiled kernel reads a pass's rows from the pool in "
+                    "16-token sub-blocks (pass Kb / Vb for this pass)", i, t.P, t.base);
+      if (p->ring) {
+        if (int64_t(t.table) + p->ring > pool_blocks)
+          return fail(err, errlen, ESP_EINVAL, "tree %d: ring blocks [%d, %d + %d) outside the pool's %d blocks", i, t.table, t.table, p->ring, pool_blocks);
+        if (t.M > int64_t(p->ring) * bt - p->window + 1)
+          return fail(err, errlen, ESP_EINVAL, "tree %d: %d rows appended to a ring of %d x %lld tokens overwrite keys that its first rows still see "
+                      "(window %d): pass Kb / Vb for this pass", i, t.M, p->ring, (long long)bt, p->window);
+      } else {
+        const int64_t nb = (int64_t(t.P) + t.M + bt - 1) / bt;
+        if (t.table + nb > n_block_entries)
+          return fail(err, errlen, ESP_EINVAL, "tree %d: block list [%d, %d + %lld) with its own rows appended lies outside the %d entries of blocks", i,
+                      t.table, t.table, (long long)nb, n_block_entries);
+        for (int64_t b = (int64_t(t.P) + bt - 1) / bt; b < nb; ++b)
+          if (blocks[t.table + b] < 0 || blocks[t.table + b] >= pool_blocks)
+            return fail(err, errlen, ESP_EINVAL, "tree %d: block %d (entry %lld of its list) outside the pool's %d blocks", i, blocks[t.table + b],
+                        (long long)b, pool_blocks);
+      }
+    }
+  }
   return ESP_OK;
 }
 
@@ -543,10 +599,13 @@ static int check_prep(const esp_prep_params* p, bool with_table, const void* kv_
 int esp_attn_prep(const esp_prep_params* p, const float* X, const float* qn_w, const float* kn_w, const int32_t* pos,
                   const float* inv_freq, const int32_t* rope_sel, void* Q, void* Kb, void* Vb, const int32_t* row_table,
                   void* kv_pool, int32_t n_rows, void* stream, char* err, size_t errlen) {
+  DropPair drop_pair;
   if (int rc = check_prep(p, row_table != nullptr, kv_pool, err, errlen)) return rc;
   if (n_rows < 0) return fail(err, errlen, ESP_EINVAL, "negative count");
   if (n_rows == 0) return ESP_OK;
-  if (!X || !qn_w || !kn_w || !Q || !Kb || !Vb) return fail(err, errlen, ESP_EINVAL, "X, qn_w, kn_w, Q, Kb, Vb must not be NULL");
+  if (!X || !qn_w || !kn_w || !Q) return fail(err, errlen, ESP_EINVAL, "X, qn_w, kn_w, Q must not be NULL");
+  if ((!Kb || !Vb) && (Kb || Vb || !row_table))
+    return fail(err, errlen, ESP_EINVAL, "Kb and Vb may be left out together, and only with a row_table (the rows then live in the pool alone)");
   if (p->rope_dims > 0 && (!pos || !inv_freq)) return fail(err, errlen, ESP_EINVAL, "pos and inv_freq must not be NULL when dims rotate");
   esp::PrepArgs a{X, qn_w, kn_w, reinterpret_cast<const int4*>(pos), inv_freq, rope_sel, static_cast<uint16_t*>(Q),
                   static_cast<uint16_t*>(Kb), static_cast<uint16_t*>(Vb), reinterpret_cast<const int4*>(row_table),

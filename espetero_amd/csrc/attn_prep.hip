@@ -96,7 +96,8 @@ __global__ __launch_bounds__(256) void attn_prep_kernel(const PrepArgs a, int n_
         *reinterpret_cast<out_t*>(a.Q + row * size_t(p.q_ld) + size_t(h) * HD + d0) = out;
         continue;
       }
-      *reinterpret_cast<out_t*>((kind == 1 ? a.Kb : a.Vb) + row * size_t(p.kv_ld) + size_t(h) * HD + d0) = out;
+      // Kb / Vb may be left out when the rows go to the pool anyway (a pass whose attention reads them from there)
+      if (uint16_t* kv = kind == 1 ? a.Kb : a.Vb) *reinterpret_cast<out_t*>(kv + row * size_t(p.kv_ld) + size_t(h) * HD + d0) = out;
       // The folded append: the same bits into the row's pool entries (a row saved into two slots has two).
       if (kind == 2 && run) {
         *reinterpret_cast<out_t*>(&vstage[r][(slot - slot0) * HD + d0]) = out;

@@ -308,7 +308,10 @@ __global__ __launch_bounds__(HD >= 512 ? 128 : 256, OCC) void attn_stream_kernel
     }
   };
 
-  // Batch units: rows of the pass (row major Kb / Vb); V gathered element by element.
+  // Batch units: rows of the pass (row major Kb / Vb); V gathered element by element. Without Kb / Vb the rows
+  // are read from the pool: they were appended before the attention (esp_attn_prep with a row table, or
+  // esp_kv_save), row j of a tree at position P + j of the tree's own block list.
+  const bool in_pool = !FUSED && a.Kb == nullptr;
   auto load_batch = [&](int u, Unit<HW, SBU>& U) {
     const int j0 = u << USH;
 #pragma unroll
@@ -317,8 +320,15 @@ __global__ __launch_bounds__(HD >= 512 ? 128 : 256, OCC) void attn_stream_kernel
       const int jk = js + c16;
       const bool k_ok = jk <= k_last;
       // fused: a tree's rows are its one tile's rows, prepared into LDS by the prologue
-      const uint16_t* kp = FUSED ? k_lds + (k_ok ? jk : 0) * HD + dw + 8 * q4
-                                 : a.Kb + size_t(tree.base + (k_ok ? jk : 0)) * a.kv_ld + size_t(kvh) * HD + dw + 8 * q4;
+      const uint16_t* kp;
+      if (FUSED) {
+        kp = k_lds + (k_ok ? jk : 0) * HD + dw + 8 * q4;
+      } else if (in_pool) {
+        const int q = tree.P + (k_ok ? jk : 0);
+        kp = a.pool + head_base(a, HD, block_of(a, table, q), kvh) + (q % bt) * HD + dw + 8 * q4;
+      } else {
+        kp = a.Kb + size_t(tree.base + (k_ok ? jk : 0)) * a.kv_ld + size_t(kvh) * HD + dw + 8 * q4;
+      }
 #pragma unroll
       for (int kk = 0; kk < KK; ++kk)
         U.k[sb][kk] = k_ok ? *reinterpret_cast<const u32x4*>(kp + 32 * kk) : u32x4{0, 0, 0, 0};
@@ -328,10 +338,20 @@ __global__ __launch_bounds__(HD >= 512 ? 128 : 256, OCC) void attn_stream_kernel
 #pragma unroll
       for (int i = 0; i < 4; ++i) {
         if (jv + i > k_last) continue;
-        const uint16_t* vp = FUSED ? v_lds + (jv + i) * HD + dw + c16 : a.Vb + size_t(tree.base + jv + i) * a.kv_ld + size_t(kvh) * HD + dw + c16;
+        const uint16_t* vp;
+        int vs = 16;  // elements from dim d to dim d + 16
+        if (FUSED) {
+          vp = v_lds + (jv + i) * HD + dw + c16;
+        } else if (in_pool) {
+          const int q = tree.P + jv + i;
+          vp = a.pool + head_base(a, HD, block_of(a, table, q), kvh) + vt_elem(bt, HD, q % bt, dw + c16);
+          vs = 16 * kVtDim;
+        } else {
+          vp = a.Vb + size_t(tree.base + jv + i) * a.kv_ld + size_t(kvh) * HD + dw + c16;
+        }
 #pragma unroll
         for (int mt = 0; mt < MT; ++mt) {
-          const uint32_t e = uint32_t(vp[16 * mt]) << (16 * (i & 1));
+          const uint32_t e = uint32_t(vp[vs * mt]) << (16 * (i & 1));
           if (i < 2) U.v[sb][mt].x |= e;
           else U.v[sb][mt].y |= e;
         }
@@ -533,7 +553,8 @@ __global__ __launch_bounds__(HD >= 512 ? 128 : 256, OCC) void attn_stream_kernel
         if (ok[c]) kl = max(kl, max(rr[c], max(dsc[c].z - 1, a.bidi ? dsc[c].w - 1 : -1)));
 #pragma unroll
       for (int o = 32; o >= 1; o >>= 1) kl = max(kl, __shfl_xor(kl, o));
-      k_last = __builtin_amdgcn_readfirstlane(min(kl, tree.M - 1));
+      // fused: the batch keys are the tile's own rows in LDS, never more than the tile holds
+      k_last = __builtin_amdgcn_readfirstlane(min(kl, (FUSED ? min(tree.M, rows_live) : tree.M) - 1));
       bp0 = tile.b0 >> USH;
       n_batch = max(0, ((k_last + UK) >> USH) - bp0);
     }

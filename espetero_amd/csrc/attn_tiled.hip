@@ -150,6 +150,12 @@ __global__ __launch_bounds__(256, OCC) void attn_tiled_kernel(const KArgs a, int
   const int n_sb = n_c + n_b;
   const int n_steps = (n_sb + 3) >> 2;
   const int n_groups = (a.n_rows + 15) >> 4;
+  // Batch rows in the pool (no Kb / Vb): the pass's rows were appended before the attention (esp_attn_prep with a
+  // row table, or esp_kv_save), row j of a tree at position P + j of the tree's own block list, and P - base is a
+  // multiple of 16 (the caller's promise; esp_attn_validate checks it). A batch sub-block - 16 absolute rows - is
+  // then one 16-token sub-block of the pool and is staged like a cached one; the masks stay in row numbers.
+  const bool in_pool = a.Kb == nullptr;
+  const int pool_shift = tree.P - tree.base;  // pool position of absolute row r: r + pool_shift
 
   // Windowed layers: do this tile's batch keys need the per-key position test at all? Not when
   // the oldest position among them is inside the window of the row with the largest position.
@@ -174,7 +180,8 @@ __global__ __launch_bounds__(256, OCC) void attn_tiled_kernel(const KArgs a, int
     if (step < ids_step0 || step >= ids_step0 + 64) {
       ids_step0 = step;
       const int sl = 4 * (step + lane) + wave;
-      ids = sl < n_c ? block_of(a, table, (c0 + sl) << 4) : 0;
+      const int js = sl < n_c ? (c0 + sl) << 4 : (in_pool && sl < n_sb) ? ((a0 + sl - n_c) << 4) + pool_shift : -1;
+      ids = js >= 0 ? block_of(a, table, js) : 0;
     }
     return __builtin_amdgcn_readlane(ids, step - ids_step0);
   };
@@ -203,8 +210,9 @@ __global__ __launch_bounds__(256, OCC) void attn_tiled_kernel(const KArgs a, int
     // memory, whose reloads wait on the same counter as the staging loads and serialise them.
     uint32_t kc = kcol0, kr = uint32_t(r0);
     asm volatile("" : "+v"(kc), "+v"(kr));
-    if (s < n_c) {
-      const int js = (c0 + s) << 4;
+    const bool batch_sb = s >= n_c && (decltype(interior)::value || s < n_sb);
+    if (s < n_c || (in_pool && batch_sb)) {
+      const int js = s < n_c ? (c0 + s) << 4 : ((a0 + s - n_c) << 4) + pool_shift;
       const int b = block_id(step);
       const int t0 = a.bt == 16 ? 0 : js % a.bt;
       const char* hbp = reinterpret_cast<const char*>(a.pool + head_base(a, HD, b, kvh));
@@ -217,7 +225,7 @@ __global__ __launch_bounds__(256, OCC) void attn_tiled_kernel(const KArgs a, int
                          kro + (kc ^ kswz(q + 3)), kdst + q * 1024);
 #pragma unroll
       for (int q = 0; q < VP; q += 4) load_to_lds16_x4(vb + q * 1024, voff, voff, voff, voff, vdst + q * 1024);
-    } else if (decltype(interior)::value || s < n_sb) {
+    } else if (batch_sb) {
       const int g = a0 + (s - n_c);
       const int lim = decltype(interior)::value ? 15 : a.n_rows - 1 - 16 * g;  // batch rows past the pass's last row do not exist
       const char* kb = reinterpret_cast<const char*>(a.Kb + size_t(16 * g) * a.kv_ld + size_t(kvh) * HD);
@@ -244,15 +252,28 @@ __global__ __launch_bounds__(256, OCC) void attn_tiled_kernel(const KArgs a, int
   // memory never written; their V must not reach the products.
   auto fix = [&](int step, int stage) __attribute__((always_inline)) {
     const int s = 4 * step + wave;
-    if (s >= n_c) return;
-    const int j0 = (c0 + s) << 4;
-    if (j0 >= tile.k0 && j0 + 16 <= tile.k1) return;
+    // keys [v0, v1) of the sub-block's own numbering are memory that has been written: the tile's cached range, or,
+    // for batch rows read from the pool, everything up to the tree's last row (what lies below its first row is the
+    // end of its cached keys)
+    int j0, v0, v1;
+    if (s < n_c) {
+      j0 = (c0 + s) << 4;
+      v0 = tile.k0;
+      v1 = tile.k1;
+    } else if (in_pool && s < n_sb) {
+      j0 = ((a0 + s - n_c) << 4) - tree.base;
+      v0 = INT32_MIN;
+      v1 = tree.M;
+    } else {
+      return;
+    }
+    if (j0 >= v0 && j0 + 16 <= v1) return;
     const int jv = j0 + 8 * hb;
     u32x4 msk;
 #pragma unroll
     for (int e = 0; e < 4; ++e) {
-      const bool lo = jv + 2 * e >= tile.k0 && jv + 2 * e < tile.k1;
-      const bool hi = jv + 2 * e + 1 >= tile.k0 && jv + 2 * e + 1 < tile.k1;
+      const bool lo = jv + 2 * e >= v0 && jv + 2 * e < v1;
+      const bool hi = jv + 2 * e + 1 >= v0 && jv + 2 * e + 1 < v1;
       msk[e] = (lo ? 0xffffu : 0u) | (hi ? 0xffff0000u : 0u);
     }
 #pragma unroll

@@ -105,6 +105,10 @@ __global__ __launch_bounds__(256, 1) void attn_tiled512_kernel(const KArgs a, in
   const int n_sb = n_c + n_b;
   const int n_steps = (n_sb + 1) >> 1;
   const int n_groups = (a.n_rows + 15) >> 4;
+  // Batch rows in the pool (no Kb / Vb): row j of a tree lies at position P + j of the tree's block list, P - base a
+  // multiple of 16: a batch sub-block of 16 absolute rows is one 16-token sub-block of the pool, staged like a cached one.
+  const bool in_pool = a.Kb == nullptr;
+  const int pool_shift = tree.P - tree.base;
 
   // ---- staging, 16 bytes per lane straight into LDS. K: this wavefront brings rows 4 wave .. + 3 of each
   // sub-block; the lane that fills chunk position `lane` of row r brings chunk lane ^ (pi(r) & 15), and
@@ -118,7 +122,8 @@ __global__ __launch_bounds__(256, 1) void attn_tiled512_kernel(const KArgs a, in
     if (sidx < ids0 || sidx >= ids0 + 64) {
       ids0 = sidx;
       const int sl = sidx + lane;
-      ids = sl < n_c ? block_of(a, table, (c0 + sl) << 4) : 0;
+      const int js = sl < n_c ? (c0 + sl) << 4 : (in_pool && sl < n_sb) ? ((a0 + sl - n_c) << 4) + pool_shift : -1;
+      ids = js >= 0 ? block_of(a, table, js) : 0;
     }
     return __builtin_amdgcn_readlane(ids, sidx - ids0);
   };
@@ -131,8 +136,8 @@ __global__ __launch_bounds__(256, 1) void attn_tiled512_kernel(const KArgs a, in
       const uint32_t kdst = lds_base + stage * kStage + (16 * t + 4 * wave) * 1024;
       const uint32_t vdst = lds_base + stage * kStage + kKStage + t * kVSub + wave * 4096;
       const uint32_t kl = uint32_t(lane);
-      if (sidx < n_c) {
-        const int js = (c0 + sidx) << 4;
+      if (sidx < n_c || (in_pool && sidx < n_sb)) {
+        const int js = sidx < n_c ? (c0 + sidx) << 4 : ((a0 + sidx - n_c) << 4) + pool_shift;
         const int b = block_id(sidx);
         const int t0 = js % a.bt;
         const char* hbp = reinterpret_cast<const char*>(a.pool + head_base(a, kHD, b, kvh));
@@ -162,15 +167,27 @@ __global__ __launch_bounds__(256, 1) void attn_tiled512_kernel(const KArgs a, in
 #pragma unroll
     for (int t = 0; t < 2; ++t) {
       const int sidx = 2 * step + t;
-      if (sidx >= n_c) continue;
-      const int j0 = (c0 + sidx) << 4;
-      if (j0 >= tile.k0 && j0 + 16 <= tile.k1) continue;
+      // keys [v0, v1) of the sub-block's own numbering are memory that has been written: the tile's cached range,
+      // or, for batch rows read from the pool, everything up to the tree's last row
+      int j0, v0, v1;
+      if (sidx < n_c) {
+        j0 = (c0 + sidx) << 4;
+        v0 = tile.k0;
+        v1 = tile.k1;
+      } else if (in_pool && sidx < n_sb) {
+        j0 = ((a0 + sidx - n_c) << 4) - tree.base;
+        v0 = INT32_MIN;
+        v1 = tree.M;
+      } else {
+        continue;
+      }
+      if (j0 >= v0 && j0 + 16 <= v1) continue;
       const int jv = j0 + 8 * ((lane & 1) ^ ((lane >> 4) & 1));  // the half of the piece at this lane's position
       u32x4 msk;
 #pragma unroll
       for (int e = 0; e < 4; ++e) {
-        const bool lo = jv + 2 * e >= tile.k0 && jv + 2 * e < tile.k1;
-        const bool hi = jv + 2 * e + 1 >= tile.k0 && jv + 2 * e + 1 < tile.k1;
+        const bool lo = jv + 2 * e >= v0 && jv + 2 * e < v1;
+        const bool hi = jv + 2 * e + 1 >= v0 && jv + 2 * e + 1 < v1;
         msk[e] = (lo ? 0xffffu : 0u) | (hi ? 0xffff0000u : 0u);
       }
 #pragma unroll

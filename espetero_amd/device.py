@@ -77,17 +77,19 @@ def forward_static(params, Q, Kb, Vb, pool, blocks, desc, pos, O, tiles, n_tiles
     abi.check(rc, err)
 
 
-def validate(params, tiles, trees, jobs, n_parts, n_rows, blocks, pool_blocks):
-    """Host-side bounds check of a pass's records (numpy arrays) before they are uploaded. Raises EspError."""
+def validate(params, tiles, trees, jobs, n_parts, n_rows, blocks, pool_blocks, fused=False, rows_in_pool=False):
+    """Host-side bounds check of a pass's records (numpy arrays) before they are uploaded. Raises EspError.
+    fused: the pass goes to esp_attn_decode_fused (also: one tile group per tree, trees of at most rows_per_tile rows).
+    rows_in_pool: the pass runs without Kb / Vb (also: block lists that reach P + M, P - base a multiple of 16 on the tiled kernel)."""
     tiles = np.ascontiguousarray(tiles, dtype=abi.TILE_DT)
     trees = np.ascontiguousarray(trees, dtype=abi.TREE_DT)
     jobs = np.ascontiguousarray(jobs, dtype=abi.COMBINE_DT)
     blocks = None if blocks is None else np.ascontiguousarray(blocks, dtype=np.int32)
     hp = lambda a: None if a is None or a.size == 0 else a.ctypes.data  # noqa: E731
     err = C.create_string_buffer(_ERRLEN)
-    rc = abi.attn_lib().esp_attn_validate(C.byref(params), hp(tiles), len(tiles), hp(trees), len(trees), hp(jobs), len(jobs),
-                                          n_parts, n_rows, hp(blocks), 0 if blocks is None else len(blocks), pool_blocks,
-                                          err, _ERRLEN)
+    mode = (abi.ESP_PASS_FUSED if fused else 0) | (abi.ESP_PASS_ROWS_IN_POOL if rows_in_pool else 0)
+    rc = abi.attn_lib().esp_attn_validate_for(C.byref(params), mode, hp(tiles), len(tiles), hp(trees), len(trees), hp(jobs), len(jobs),
+                                              n_parts, n_rows, hp(blocks), 0 if blocks is None else len(blocks), pool_blocks, err, _ERRLEN)
     abi.check(rc, err)
 
 
@@ -178,11 +180,12 @@ class DevicePass:
     replays esp_attn_forward (what a decode chain does between host syncs)."""
 
     def __init__(self, params, trees, tiles, jobs, n_parts, n_rows, blocks, desc=None, pos=None, device="cuda",
-                 pool_blocks=None, static=False):
-        """pool_blocks: blocks in the pool; when given, the records are checked on the host before the upload.
+                 pool_blocks=None, static=False, fused=False, rows_in_pool=False):
+        """pool_blocks: blocks in the pool; when given, the records are checked on the host before the upload
+        (fused: with the checks of a pass meant for decode_fused).
         static: run over the library's own scratch array (esp_attn_forward_static) instead of a workspace."""
         if pool_blocks is not None:
-            validate(params, tiles, trees, jobs, n_parts, n_rows, blocks, pool_blocks)
+            validate(params, tiles, trees, jobs, n_parts, n_rows, blocks, pool_blocks, fused=fused, rows_in_pool=rows_in_pool)
         self.params = params
         self.static = static
         self.n_trees, self.n_tiles, self.n_jobs = len(trees), len(tiles), len(jobs)
@@ -201,7 +204,7 @@ class DevicePass:
         """Enqueues the pass. The ctypes argument list is built once per set of buffers and reused: a decode step is
         tens of microseconds on the GPU, and rebuilding twenty pointer objects per call costs the host as much."""
         st = torch.cuda.current_stream().cuda_stream if stream is None else stream.cuda_stream
-        key = (Q.data_ptr(), Kb.data_ptr(), Vb.data_ptr(), pool.data_ptr(), O.data_ptr(), st, merge,
+        key = (Q.data_ptr(), None if Kb is None else Kb.data_ptr(), None if Vb is None else Vb.data_ptr(), pool.data_ptr(), O.data_ptr(), st, merge,
                None if self.pos is None else self.pos.data_ptr())
         if self._key != key:
             jobs, n_jobs = (self.jobs, self.n_jobs) if merge else (None, 0)

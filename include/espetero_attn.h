@@ -45,7 +45,7 @@
 extern "C" {
 #endif
 
-#define ESP_ABI_VERSION 2
+#define ESP_ABI_VERSION 3
 
 enum { ESP_OK = 0, ESP_EINVAL = 1, ESP_EUNSUPPORTED = 2, ESP_ELAUNCH = 3, ESP_EWORKSPACE = 4 };
 enum { ESP_F16 = 0, ESP_BF16 = 1 };
@@ -157,7 +157,13 @@ size_t esp_attn_workspace_bytes(const esp_attn_params* p, int32_t n_rows, int32_
  * window == 0. O [n_rows][q_ld]. The kernel family is chosen from
  * rows_per_tile * G (streaming split-K kernel up to 32 packed rows, tiled
  * MFMA kernel above), as the reference chooses from its plan (forest.h:2863-2868).
- * n_jobs = 0 with n_parts > 0 skips the merge (see esp_attn_combine). */
+ * n_jobs = 0 with n_parts > 0 skips the merge (see esp_attn_combine).
+ * Kb and Vb both NULL: the pass's rows are already in the pool - appended before this call by esp_attn_prep with a
+ * row_table (the reference's fold of kv_save into attn_prep, 40_:86-100) or by esp_kv_save - row j of a tree at
+ * position P + j of the tree's own block list, and the kernels read them from there: no Kb / Vb round trip through
+ * memory and no staging copy in front of the tiled kernel. What the caller promises with it is what
+ * esp_attn_validate_for(ESP_PASS_ROWS_IN_POOL) checks; a pass that cannot promise it (verify trees whose rows are
+ * not stored behind their parent's keys, P - base not a multiple of 16 on the tiled kernel) passes Kb / Vb. */
 int esp_attn_forward(const esp_attn_params* p, const void* Q, const void* Kb, const void* Vb, const void* kv_pool,
                      const int32_t* blocks, const int32_t* desc, const int32_t* pos, void* O, const esp_tile* tiles,
                      int32_t n_tiles, const esp_tree* trees, int32_t n_trees, const esp_combine* jobs, int32_t n_jobs,
@@ -189,6 +195,19 @@ int esp_attn_forward_static(const esp_attn_params* p, const void* Q, const void*
 int esp_attn_validate(const esp_attn_params* p, const esp_tile* tiles, int32_t n_tiles, const esp_tree* trees, int32_t n_trees,
                       const esp_combine* jobs, int32_t n_jobs, int32_t n_parts, int32_t n_rows, const int32_t* blocks,
                       int32_t n_block_entries, int32_t pool_blocks, char* err, size_t errlen);
+
+/* esp_attn_validate for a pass that will run in one of the forms whose promises only the records can answer (they
+ * live in device memory when the pass runs). mode, a sum of
+ *   ESP_PASS_FUSED         the pass goes to esp_attn_decode_fused: every tree at most rows_per_tile rows and every tile
+ *                          starting at its tree's first row, i.e. one tile group per tree;
+ *   ESP_PASS_ROWS_IN_POOL  the pass goes to esp_attn_forward without Kb / Vb: row j of every tree is read at position
+ *                          P + j of the tree's own block list, which must reach that far; on the tiled kernel P - base
+ *                          is a multiple of 16; on ring layers a tree's rows must not overwrite keys its first rows see.
+ * Same arguments as esp_attn_validate otherwise. Host pointers; touches no device. */
+enum { ESP_PASS_FUSED = 1, ESP_PASS_ROWS_IN_POOL = 2 };
+int esp_attn_validate_for(const esp_attn_params* p, int32_t mode, const esp_tile* tiles, int32_t n_tiles, const esp_tree* trees,
+                          int32_t n_trees, const esp_combine* jobs, int32_t n_jobs, int32_t n_parts, int32_t n_rows, const int32_t* blocks,
+                          int32_t n_block_entries, int32_t pool_blocks, char* err, size_t errlen);
 
 /* Measurement hook; no counterpart in the reference (its bench times command
  * buffers, src/model/impl/bench.h:697-722). The next esp_attn_forward (or
@@ -275,7 +294,8 @@ typedef struct esp_prep_params {
 /* X [n_rows][x_ld] fp32; qn_w / kn_w [head_dim] fp32; pos int32[4] per row (x, y, z
  * position components); inv_freq [rope_dims / 2]; rope_sel [rope_dims / 2]: which position
  * component each frequency rotates by (40_:62-63, 82_:77-79), NULL: all by pos.x (80_:99).
- * Q [n_rows][q_ld], Kb / Vb [n_rows][kv_ld]: storage type.
+ * Q [n_rows][q_ld], Kb / Vb [n_rows][kv_ld]: storage type; with a row_table Kb and Vb may both be NULL (the rows
+ * then live in the pool alone, for an attention call that reads them there).
  * row_table NULL, or int32[4] per row = (block, position, block2, position2), -1 none
  * (kv_row_table, forest.h:1737-1749): the row's K and V also go to those entries of
  * kv_pool in the native layout, which replaces the kv_save dispatch after the attention

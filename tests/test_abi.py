@@ -212,6 +212,59 @@ def test_validate_accepts_a_planned_pass_and_names_the_first_bad_record():
         device.validate(p, tl, tr, jb, npart, 1, None, 11)
 
 
+def test_validate_fused_wants_one_tile_group_per_tree():
+    """esp_attn_validate_fused: esp_attn_validate plus what esp_attn_decode_fused relies on and cannot see on the device:
+    trees of at most rows_per_tile rows, each tile starting at its tree's first row."""
+    import numpy as np
+    import pytest
+    from espetero_amd import device
+    p, trees, tiles, jobs, n_parts, n_rows, blocks, pool_blocks = _planned_pass()
+    device.validate(p, tiles, trees, jobs, n_parts, n_rows, blocks, pool_blocks, fused=True)   # trees of 4, 1 and 2 rows at 4 rows per tile
+    p.rows_per_tile = 2                         # the first tree now needs two tile groups
+    tl, jb, npart = host.plan_tiles(trees, 4, 0, None, host.options_mi355x(2, 64))
+    device.validate(p, tl, trees, jb, npart, n_rows, blocks, pool_blocks)
+    with pytest.raises(abi.EspError, match="tree 0: 4 rows"):
+        device.validate(p, tl, trees, jb, npart, n_rows, blocks, pool_blocks, fused=True)
+    p.rows_per_tile = 8
+    tl, jb, npart = host.plan_tiles(trees, 4, 0, None, host.options_mi355x(8, 64))
+    with pytest.raises(abi.EspError, match="fused decode takes trees of 1 to 4 rows"):
+        device.validate(p, tl, trees, jb, npart, n_rows, blocks, pool_blocks, fused=True)
+
+
+def test_validate_names_what_a_pass_without_kb_vb_has_to_promise():
+    """ESP_PASS_ROWS_IN_POOL: block lists that reach P + M, P - base a multiple of 16 on the tiled kernel, no ring overrun."""
+    import numpy as np
+    import pytest
+    from espetero_amd import device, synth
+    opts = host.options_mi355x(128, 512)
+
+    def case(seqs, **kw):   # block lists sized for P + M keys, of which P are cached
+        c = synth.make_case("rows_in_pool", 64, 4, 2, 128, abi.ESP_F16, 16, [(P + M, M) for P, M in seqs], **kw)
+        for t, (P, M) in zip(c.trees, seqs):
+            t["P"] = P
+        return c
+    c = case([(48, 128), (208, 8)], rows_per_tile=128)   # P - base = 48 and 208 - 128 = 80; the second tree's rows open a block of their own
+    tiles, jobs, n_parts = host.plan_tiles(c.trees, 4, 0, None, opts)
+    device.validate(c.params, tiles, c.trees, jobs, n_parts, c.n_rows, c.blocks, c.n_blocks, rows_in_pool=True)
+    with pytest.raises(abi.EspError, match="with its own rows appended"):
+        device.validate(c.params, tiles, c.trees, jobs, n_parts, c.n_rows, c.blocks[:-1], c.n_blocks, rows_in_pool=True)
+    c = case([(40, 130)], rows_per_tile=128)            # P - base = 40
+    tiles, jobs, n_parts = host.plan_tiles(c.trees, 4, 0, None, opts)
+    device.validate(c.params, tiles, c.trees, jobs, n_parts, c.n_rows, c.blocks, c.n_blocks)
+    with pytest.raises(abi.EspError, match="no multiple of 16"):
+        device.validate(c.params, tiles, c.trees, jobs, n_parts, c.n_rows, c.blocks, c.n_blocks, rows_in_pool=True)
+    c.params.rows_per_tile = 4                          # the streaming kernel reads row by row: any P
+    tiles, jobs, n_parts = host.plan_tiles(c.trees, 2, 0, None, host.options_mi355x(4, 512))
+    device.validate(c.params, tiles, c.trees, jobs, n_parts, c.n_rows, c.blocks, c.n_blocks, rows_in_pool=True)
+    c = synth.make_case("ring", 66, 4, 2, 128, abi.ESP_F16, 16, [(900, 40)], window=256, ring_layer=True, rows_per_tile=8)
+    tiles, jobs, n_parts = host.plan_tiles(c.trees, 2, 256, c.pos, host.options_mi355x(8, 512))
+    with pytest.raises(abi.EspError, match="overwrite keys"):
+        device.validate(c.params, tiles, c.trees, jobs, n_parts, c.n_rows, None, c.n_blocks, rows_in_pool=True)
+    c.trees[0]["M"] = 1
+    tiles, jobs, n_parts = host.plan_tiles(c.trees, 2, 256, c.pos, host.options_mi355x(8, 512))
+    device.validate(c.params, tiles, c.trees, jobs, n_parts, c.n_rows, None, c.n_blocks, rows_in_pool=True)
+
+
 def test_validate_accepts_the_tiled_planner_s_partly_split_chunk():
     """A prefill chunk planned for the tiled kernel (128-row tiles, only the shortest tiles cut into parts of unequal
     count) passes the validator; dropping one of a tile's parts does not."""

@@ -233,7 +233,7 @@ def test_fused_prep_on_verify_trees_is_prep_then_attention_bit_for_bit(H, Hkv, H
     resident, groups = device.plan_hint(ap)
     tiles, jobs, n_parts = host.plan_tiles(trees, groups, 0, None, host.options_mi355x(4, 64))
     assert n_parts > 0
-    dp = device.DevicePass(ap, trees, tiles, jobs, n_parts, n_rows, blocks, desc, pos, pool_blocks=n_blocks)
+    dp = device.DevicePass(ap, trees, tiles, jobs, n_parts, n_rows, blocks, desc, pos, pool_blocks=n_blocks, fused=True)
     dev = lambda x: None if x is None else torch.from_numpy(np.ascontiguousarray(x)).cuda()  # noqa: E731
     Xd, qn, kn, posd = dev(a["X"]), dev(a["qn_w"]), dev(a["kn_w"]), dev(pos)
     inv_freq, sel, tabd = dev(a["inv_freq"]), dev(a["rope_sel"]), dev(table)
@@ -308,7 +308,7 @@ def test_fused_decode_on_seeded_random_shapes_is_prep_then_attention_bit_for_bit
         resident, groups = device.plan_hint(ap)
         tiles, jobs, n_parts = host.plan_tiles(trees, groups, window, pos if window else None, host.options_mi355x(R, int(rng.choice([8, 64, resident]))))
         print(f"fused random {it}: H={H} Hkv={Hkv} HD={HD} R={R} bt={BT} dtype={dtype} {kind} window={window} seqs={seqs} tiles={len(tiles)} parts={n_parts}", flush=True)
-        dp = device.DevicePass(ap, trees, tiles, jobs, n_parts, n_rows, blocks, desc, pos, pool_blocks=n_blocks)
+        dp = device.DevicePass(ap, trees, tiles, jobs, n_parts, n_rows, blocks, desc, pos, pool_blocks=n_blocks, fused=True)
         Xd, qn, kn, posd = dev(a["X"]), dev(a["qn_w"]), dev(a["kn_w"]), dev(pos)
         inv_freq, sel, tabd = dev(a["inv_freq"]), dev(a["rope_sel"]), dev(table)
         res = []
@@ -352,7 +352,7 @@ def test_fused_decode_without_an_append_and_without_descriptors_leaves_the_pool_
     pool0 = (torch.randn(n_blocks * 2 * BT * ap.kv_ld, device="cuda") * 0.5).to(torch.bfloat16)
     resident, groups = device.plan_hint(ap)
     tiles, jobs, n_parts = host.plan_tiles(trees, groups, 0, None, host.options_mi355x(1, 32))
-    dp = device.DevicePass(ap, trees, tiles, jobs, n_parts, n_rows, blocks, None, None, pool_blocks=n_blocks)
+    dp = device.DevicePass(ap, trees, tiles, jobs, n_parts, n_rows, blocks, None, None, pool_blocks=n_blocks, fused=True)
     dev = lambda x: None if x is None else torch.from_numpy(np.ascontiguousarray(x)).cuda()  # noqa: E731
     Xd, qn, kn, posd, inv_freq = dev(a["X"]), dev(a["qn_w"]), dev(a["kn_w"]), dev(pos), dev(a["inv_freq"])
     pool = pool0.clone()

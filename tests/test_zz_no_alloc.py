@@ -36,6 +36,33 @@ def test_static_entry_point_matches_the_workspace_one_on_two_calls_in_a_row():
     _both(small, host.options_mi355x(128, 64))
 
 
+def test_static_entry_point_leaves_device_memory_as_it_found_it():
+    """Free device memory as the driver reports it is the same before and after a run of static calls (every buffer
+    of the passes themselves is allocated before the first reading)."""
+    import torch
+    from gpu_utils import dev_u16, native_pool, plan
+    device.init(0)
+    runs = []
+    for case, wg in ((small_case(seed=76, seqs=((5000, 1), (300, 1)), H=32, Hkv=4, rows_per_tile=1), 256),
+                     (small_case(seed=77, seqs=((1500, 200),), H=10, Hkv=2, dtype=abi.ESP_BF16, rows_per_tile=128), 64)):
+        tiles, jobs, n_parts = plan(case, host.options_mi355x(case.params.rows_per_tile, wg))
+        assert n_parts > 0
+        dp = device.DevicePass(case.params, case.trees, tiles, jobs, n_parts, case.n_rows, case.blocks, case.desc, case.pos,
+                               pool_blocks=case.n_blocks, static=True)
+        Q = dev_u16(case.Q)
+        runs.append((dp, Q, dev_u16(case.Kb), dev_u16(case.Vb), native_pool(case), torch.zeros_like(Q)))
+    for dp, Q, Kb, Vb, pool, O in runs:   # first calls: whatever one-time set-up there is has happened
+        dp.run(Q, Kb, Vb, pool, O)
+    torch.cuda.synchronize()
+    free0, _ = torch.cuda.mem_get_info()
+    for _ in range(5):
+        for dp, Q, Kb, Vb, pool, O in runs:
+            dp.run(Q, Kb, Vb, pool, O)
+    torch.cuda.synchronize()
+    free1, _ = torch.cuda.mem_get_info()
+    assert free1 == free0, f"free device memory went from {free0} to {free1} over ten static calls"
+
+
 def test_static_entry_point_names_its_limit():
     """A pass whose records do not fit the array is refused before anything is launched."""
     import torch
