@@ -32,7 +32,7 @@ class Workload:
     """Device-resident inputs of one benchmark shape plus the planned passes."""
 
     def __init__(self, name, H, Hkv, HD, dtype, bt, seqs, window=0, rows_per_tile=1, desc_fn=None, pool_pages=65536,
-                 seed=0, workgroups=None, bound="hbm", contiguous=False):
+                 seed=0, workgroups=None, bound="hbm", contiguous=False, rows_in_pool=None):
         import torch
         from espetero_amd import abi, device, host, synth
         self.torch, self.abi, self.device, self.host = torch, abi, device, host
@@ -85,9 +85,24 @@ class Workload:
         if contiguous:  # experiment: pages in address order
             perm = np.arange(self.pool_pages, dtype=np.int32)
         self.tables = [perm[s * pages_per_set:(s + 1) * pages_per_set].copy() for s in range(self.n_sets)]
+        # Prefill passes read their own rows from the pool (esp_attn_forward without Kb / Vb): the rows are appended
+        # once, here, to positions P + j of every rotation set's block lists, as esp_attn_prep with a row table leaves
+        # them in front of the attention of a layer. Decode and verify passes hand their rows over as Kb / Vb.
+        self.rows_in_pool = (rows_per_tile > 32) if rows_in_pool is None else rows_in_pool
         self.passes = [device.DevicePass(p, trees, self.tiles, self.jobs, self.n_parts, n_rows, t,
-                                         desc if desc_fn is not None else None, pos if window > 0 else None)
+                                         desc if desc_fn is not None else None, pos if window > 0 else None,
+                                         pool_blocks=self.pool_pages, rows_in_pool=self.rows_in_pool)
                        for t in self.tables]
+        if self.rows_in_pool:
+            e = np.zeros(n_rows, abi.KVSAVE_DT)
+            e["src_row"] = np.arange(n_rows)
+            for t in self.tables:
+                for tr in trees:
+                    b0, P, tab, M = int(tr["base"]), int(tr["P"]), int(tr["table"]), int(tr["M"])
+                    q = P + np.arange(M)
+                    e["block"][b0:b0 + M], e["pos"][b0:b0 + M] = t[tab + q // bt], q % bt
+                device.kv_save(p, self.Kb, self.Vb, self.pool, device.to_dev(e), n_rows)
+            torch.cuda.synchronize()
         # algorithmic work: every visible K and V element once + Q + O + block-table entries; visible (q, k) pairs
         es = 2
         vis_keys, pairs = 0, 0
@@ -105,7 +120,10 @@ class Workload:
         dp = self.passes[i % self.n_sets]
         if ev:
             self.device.time_next(ev[0], ev[1])  # the launch of the attention kernel records into them
-        dp.run(self.Q, self.Kb, self.Vb, self.pool, self.O)  # attention + split-K merge, one call
+        if self.rows_in_pool:
+            dp.run(self.Q, None, None, self.pool, self.O)
+        else:
+            dp.run(self.Q, self.Kb, self.Vb, self.pool, self.O)  # attention + split-K merge, one call
 
 
 class PrepWorkload:
@@ -194,13 +212,16 @@ class GateWorkload:
 
 
 class ChunkedPrefill:
-    """One sequence of 8192 tokens in four 2048-token chunks against the paged cache: chunk c attends to
-    the 2048 c cached tokens and causally to itself, then its K / V rows are appended (esp_kv_save).
-    A step is the whole sequence: 4 x (attention + split-K merge + append)."""
+    """One sequence of 8192 tokens in four 2048-token chunks against the paged cache: chunk c's K / V rows are
+    appended (esp_kv_save), then it attends to the 2048 c cached tokens and causally to itself, its own rows read
+    from the pool (esp_attn_forward without Kb / Vb). A step is the whole sequence: 4 x (append + attention +
+    split-K merge). rows_in_pool=False: the attention takes the rows as Kb / Vb (a staging copy of V in front of the
+    kernel) and the append follows it."""
 
     launches_per_step = 4
 
-    def __init__(self, name, H=40, Hkv=8, HD=128, chunk=2048, n_chunks=4, bt=16, seed=3, workgroups=None):
+    def __init__(self, name, H=40, Hkv=8, HD=128, chunk=2048, n_chunks=4, bt=16, seed=3, workgroups=None, rows_in_pool=True):
+        self.rows_in_pool = rows_in_pool
         import torch
         from espetero_amd import abi, device, host, synth
         self.torch, self.device = torch, device
@@ -229,7 +250,8 @@ class ChunkedPrefill:
             for c in range(n_chunks):
                 trees = np.array([(0, c * chunk, 0, chunk)], abi.TREE_DT)
                 tiles, jobs, n_parts = host.plan_tiles(trees, groups, 0, None, opts)
-                dp = device.DevicePass(p, trees, tiles, jobs, n_parts, chunk, table, None, None)
+                dp = device.DevicePass(p, trees, tiles, jobs, n_parts, chunk, table, None, None, pool_blocks=self.pool_pages,
+                                       rows_in_pool=rows_in_pool)
                 tok = c * chunk + np.arange(chunk)
                 e = np.zeros(chunk, abi.KVSAVE_DT)
                 e["src_row"], e["block"], e["pos"] = np.arange(chunk), table[tok // bt], tok % bt
@@ -247,8 +269,12 @@ class ChunkedPrefill:
         for c, (dp, saves, rows) in enumerate(self.sets[i % self.n_sets]):
             if ev:
                 d.time_next(ev[c][0], ev[c][1])
-            dp.run(self.Q[rows], self.Kb[rows], self.Vb[rows], self.pool, self.O[rows])
-            d.kv_save(self.params, self.Kb[rows], self.Vb[rows], self.pool, saves, rows.stop - rows.start)
+            if self.rows_in_pool:
+                d.kv_save(self.params, self.Kb[rows], self.Vb[rows], self.pool, saves, rows.stop - rows.start)
+                dp.run(self.Q[rows], None, None, self.pool, self.O[rows])
+            else:
+                dp.run(self.Q[rows], self.Kb[rows], self.Vb[rows], self.pool, self.O[rows])
+                d.kv_save(self.params, self.Kb[rows], self.Vb[rows], self.pool, saves, rows.stop - rows.start)
 
 
 class LayerMix:
@@ -314,6 +340,88 @@ class DecodeStep:
             dp.run(w.Q, w.Kb, w.Vb, w.pool, w.O)
 
 
+class PrefillStep:
+    """The attention part of the chunked prefill of one layer from the fp32 fused projection to O, chunk by chunk:
+    esp_attn_prep, esp_attn_forward with the rows as Kb / Vb (a staging copy of V in front of the kernel), esp_kv_save;
+    or, folded: esp_attn_prep with the row table and no Kb / Vb of its own, esp_attn_forward reading the rows from the pool."""
+
+    def __init__(self, w, folded, seed=13):
+        import torch
+        from espetero_amd import device, synth
+        self.w, self.folded, self.torch, self.device = w, folded, torch, device
+        self.name = w.name + ("_step_folded" if folded else "_step")
+        N, bt = w.n_rows, w.bt
+        self.pp, a = synth.make_prep("omni", w.H, w.Hkv, w.HD, w.dtype, N, seed=seed, bt=bt, max_pos=1)
+        a["pos"][:, :3] = np.arange(N)[:, None]
+        dev = lambda x: None if x is None else torch.from_numpy(np.ascontiguousarray(x)).cuda()  # noqa: E731
+        g = torch.Generator(device="cuda")
+        g.manual_seed(seed)
+        self.X = torch.randn(N, self.pp.x_ld, generator=g, device="cuda") * 1.5
+        self.qn_w, self.kn_w, self.pos = dev(a["qn_w"]), dev(a["kn_w"]), dev(a["pos"])
+        self.inv_freq, self.rope_sel = dev(a["inv_freq"]), dev(a["rope_sel"])
+        self.tables = []
+        for chunks in w.sets:
+            table = chunks[0][0].blocks.cpu().numpy()
+            t = np.full((N, 4), -1, np.int32)
+            t[:, 0], t[:, 1] = table[np.arange(N) // bt], np.arange(N) % bt
+            self.tables.append(dev(t))
+        # the same planned passes in both forms: the records do not depend on where the rows are read
+        self.passes = [[device.DevicePass(w.params, dp.trees_host, dp.tiles_host, dp.jobs_host, dp.n_parts, dp.n_rows, table_of(chunks), None, None,
+                                          rows_in_pool=folded) for dp, _, _ in chunks] for chunks in w.sets]
+
+    def step(self, i, ev=None):
+        w, d = self.w, self.device
+        k = i % w.n_sets
+        for c, (dp0, saves, rows) in enumerate(w.sets[k]):
+            dp = self.passes[k][c]
+            n = rows.stop - rows.start
+            args = (self.pp, self.X[rows], self.qn_w, self.kn_w, self.pos[rows], self.inv_freq, self.rope_sel, w.Q[rows])
+            if self.folded:
+                d.attn_prep(*args, None, None, self.tables[k][rows], w.pool, n)
+                dp.run(w.Q[rows], None, None, w.pool, w.O[rows])
+            else:
+                d.attn_prep(*args, w.Kb[rows], w.Vb[rows], None, None, n)
+                dp.run(w.Q[rows], w.Kb[rows], w.Vb[rows], w.pool, w.O[rows])
+                d.kv_save(w.params, w.Kb[rows], w.Vb[rows], w.pool, saves, n)
+
+
+def table_of(chunks):
+    return chunks[0][0].blocks.cpu().numpy()
+
+
+def prefill_step_fusion(args, torch, emit=True, steps=10, warmup=2):
+    """Step time of the attention part of the chunked prefill (config 3: four chunks) from the fp32 projection to O,
+    with the rows handed from the prep to the attention through Kb / Vb and appended afterwards, against the folded form."""
+    w = make_workload("c3_chunked_prefill", args.workgroups or None, False, args.page)
+    rec, outs, pools = {}, [], []
+    for folded in (False, True):
+        s = PrefillStep(w, folded)
+        w.O.zero_()
+        w.pool.zero_()
+        s.step(0)
+        torch.cuda.synchronize()
+        outs.append(w.O.clone())
+        pools.append(w.pool.clone())
+        for i in range(warmup):
+            s.step(i)
+        torch.cuda.synchronize()
+        t0 = time.perf_counter()
+        for i in range(steps):
+            s.step(i)
+        torch.cuda.synchronize()
+        tag = "folded" if folded else "three_calls"
+        rec[tag + "_eager_us"] = round((time.perf_counter() - t0) / steps * 1e6, 2)
+        rec[tag + "_graph_us"] = graph_replay(s, torch, steps=2, replays=4).get("us_per_step")
+    rec["identical_output"] = bool(torch.equal(outs[0].view(torch.int16), outs[1].view(torch.int16)))
+    rec["identical_pool"] = bool(torch.equal(pools[0].view(torch.int16), pools[1].view(torch.int16)))
+    parts = 1 if w.n_parts else 0
+    rec["dispatches_per_chunk"] = {"three_calls": 4 + parts, "folded": 2 + parts}   # prep, staging copy, attention, [merge,] append | prep, attention[, merge]
+    out = {"metric": "chunked prefill attention step, prep + attention (+ append)", "unit": "us", "steps": steps, "config": "c3_chunked_prefill", **rec}
+    if emit:
+        print(json.dumps(out), flush=True)
+    return out
+
+
 def decode_step_fusion(args, torch, names=("c1_single_decode", "c2_batched_decode", "c4_decode_sliding", "c4_decode_global"), emit=True):
     """Step time of the attention part of a decode layer with and without the prep fused into the attention kernel:
     eager wall time per step and the time per step of 16 steps replayed from one HIP graph."""
@@ -358,8 +466,8 @@ def make_workload(name, workgroups=None, contiguous=False, page=16):
         kind = name[3:-4]
         return LayerMix(name, make_workload(f"c4_{kind}_sliding", workgroups, contiguous, page),
                         make_workload(f"c4_{kind}_global", workgroups, contiguous, page))
-    if name == "c3_chunked_prefill":   # the whole of config 3 as one step
-        return ChunkedPrefill(name, bt=page, workgroups=workgroups)
+    if name in ("c3_chunked_prefill", "c3_chunked_prefill_kb"):   # the whole of config 3 as one step; _kb: rows handed over as Kb / Vb
+        return ChunkedPrefill(name, bt=page, workgroups=workgroups, rows_in_pool=not name.endswith("_kb"))
     if name == "c3_attn_prep":   # the rows of one C3 prefill chunk, Qwen3-Omni arrangement (82_qwen3_omni.metal:30-88)
         return PrepWorkload(name, "omni", 40, 8, 128, BF16, 2048, bt=page)
     if name == "c4_attn_prep":   # the rows of one C4 prefill pass, Qwen3.5 arrangement (40_attention.metal:9-102)
@@ -402,7 +510,8 @@ def measured_traffic(workload):
     WRITE_SIZE counters (each scaled by what the same counter reads for a plain 256 MiB copy); the
     summaries under profiles/ show the runs. A step of several launches (the chunked prefill, the layer mixes) is
     the sum over its launches. None for a workload that has not been measured."""
-    parts = {"c3_chunked_prefill": ["c3_prefill_p0", "c3_prefill_p2048", "c3_prefill_p4096", "c3_prefill_p6144"],   # one launch per chunk
+    chunks = ["c3_prefill_p0", "c3_prefill_p2048", "c3_prefill_p4096", "c3_prefill_p6144"]   # one launch per chunk
+    parts = {"c3_chunked_prefill": chunks, "c3_chunked_prefill_kb": chunks,
              "c4_decode_mix": ["c4_decode_sliding"] * 5 + ["c4_decode_global"],
              "c4_prefill_mix": ["c4_prefill_sliding"] * 5 + ["c4_prefill_global"]}.get(workload, [workload])
     try:
@@ -425,7 +534,7 @@ def traffic_source():
 
 WORKLOADS = ["c1_single_decode", "c2_batched_decode", "c3_prefill_p0", "c3_prefill_p2048", "c3_prefill_p4096",
              "c3_prefill_p6144", "c4_decode_sliding", "c4_decode_global", "c4_prefill_sliding", "c4_prefill_global",
-             "c5_verify", "c4_decode_mix", "c4_prefill_mix", "c3_chunked_prefill", "c3_attn_prep", "c4_attn_prep",
+             "c5_verify", "c4_decode_mix", "c4_prefill_mix", "c3_chunked_prefill", "c3_chunked_prefill_kb", "c3_attn_prep", "c4_attn_prep",
              "c4_head_gate", "c4_head_gate_dots", "g4_global512_decode", "g4_global512_prefill"]
 
 
@@ -697,13 +806,15 @@ def spin(torch, ms):
     torch.cuda._sleep(int(_SPIN["per_ms"] * ms))
 
 
-def kernel_times(w, torch, n, first_step=0):
+def kernel_times(w, torch, n, first_step=0, step_seconds=0.0):
     """Durations of the dominant kernel's launches over n steps, in milliseconds [n][launches per step], from HIP
     event pairs handed to the launches themselves (esp_attn_time_next -> hipExtLaunchKernelGGL: the first event is
     a marker in front of the dispatch, the second the dispatch's own end). The steps are enqueued behind a few
     milliseconds of spinning, so marker and dispatch are both in the queue when the GPU reaches them: taken while
     the GPU waits for the host instead (the host needs longer to enqueue an armed step than the GPU to run it),
-    the pair also spans the host's time between the two enqueues and reads 4 to 7 us long."""
+    the pair also spans the host's time between the two enqueues and reads 4 to 7 us long. (No spinning in front of
+    steps of 200 us and more: the host stays ahead of those by itself, and an idle stretch would let a chip that
+    runs at the clock its power budget allows cool down and read faster than it sustains.)"""
     nev = getattr(w, "launches_per_step", 1)
     evs = [[(torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)) for _ in range(nev)] for _ in range(n)]
     for pairs in evs:  # a first record creates the HIP events behind the torch objects
@@ -711,7 +822,8 @@ def kernel_times(w, torch, n, first_step=0):
             a.record()
             b.record()
     torch.cuda.synchronize()
-    spin(torch, 3.0 + 0.15 * n * nev)
+    if step_seconds < 2e-4:   # a step the host cannot enqueue faster than the GPU runs it; longer ones keep the queue full by themselves
+        spin(torch, 3.0 + 0.15 * n * nev)
     for i, ev in enumerate(evs):
         w.step(first_step + i, ev[0] if nev == 1 else ev)
     torch.cuda.synchronize()
@@ -719,10 +831,20 @@ def kernel_times(w, torch, n, first_step=0):
 
 
 def timed_run(w, torch, steps, warmup, kernel_samples=None):
-    """warmup untimed steps, then exactly `steps` timed ones between two device synchronisations with nothing but
-    the steps in the loop: wall seconds per step. The dominant kernel's own durations are taken afterwards, in a
+    """30 ms of the workload's own steps to wake the device, `warmup` untimed steps, then exactly `steps` timed ones
+    between two device synchronisations with nothing but the steps in the loop: wall seconds per step. The dominant kernel's own durations are taken afterwards, in a
     loop of their own (kernel_times), so that the instrumentation is not part of what the wall clock sees.
     Returns (wall seconds per step, kernel milliseconds [samples][launches per step])."""
+    # A GPU that has sat idle while the host built the workload takes milliseconds to leave its low-power state,
+    # longer than a handful of 30 us warm-up steps last: keep it busy with the workload's own steps for 30 ms first.
+    t0 = time.perf_counter()
+    i = 0
+    while time.perf_counter() - t0 < (0.03 if w.bound == "hbm" else 0.1):   # matrix-bound passes also settle at the clock their power allows
+        w.step(i)
+        i += 1
+        if i % 64 == 0:
+            torch.cuda.synchronize()
+    torch.cuda.synchronize()
     for i in range(warmup):
         w.step(i)
     torch.cuda.synchronize()
@@ -732,7 +854,7 @@ def timed_run(w, torch, steps, warmup, kernel_samples=None):
     torch.cuda.synchronize()
     wall = (time.perf_counter() - t0) / steps
     n = kernel_samples or max(8, min(steps, 40))
-    return wall, kernel_times(w, torch, n, warmup + steps)
+    return wall, kernel_times(w, torch, n, warmup + steps, wall)
 
 
 def kernel_name(w):
@@ -953,6 +1075,11 @@ def run_all(args, torch):
     kernel roofline, a parity spot check and a CPU baseline of its own), and the machine's measured ceilings."""
     K, W = args.steps, args.warmup
     cpu = not args.no_cpu
+    # The machine's own ceilings, for orientation only (no fraction is stated against them): a plain read kernel at
+    # the sizes of C2 / C5 / C4 global, and the matrix cores alone. Measured first: a GPU that has sat idle takes
+    # milliseconds to leave its low-power state, more than the W warm-up steps of a 30 us pass last.
+    ceil = Ceilings()
+    ceilings = {"hbm_read": ceil.hbm_read(), "mfma_issue": ceil.mfma_issue()}
     w = make_workload("c2_batched_decode", args.workgroups or None, args.tables == "contiguous", args.page)
     wall, per_launch = timed_run(w, torch, K, W)
     out = headline(w, wall, per_launch, K, W)
@@ -1020,10 +1147,8 @@ def run_all(args, torch):
     # the decode step from the fp32 projection to O: esp_attn_prep + esp_attn_forward against esp_attn_decode_fused
     fa = argparse.Namespace(**{**vars(args), "steps": 100, "warmup": 10})
     out["decode_step"] = decode_step_fusion(fa, torch, ("c1_single_decode", "c2_batched_decode", "c4_decode_sliding"), emit=False)["configs"]
-    # The machine's own ceilings, for orientation only (no fraction is stated against them): a plain read kernel at
-    # the sizes of C2 / C5 / C4 global, and the matrix cores alone.
-    ceil = Ceilings()
-    out["ceilings"] = {"hbm_read": ceil.hbm_read(), "mfma_issue": ceil.mfma_issue()}
+    out["prefill_step"] = prefill_step_fusion(args, torch, emit=False)
+    out["ceilings"] = ceilings
     out["traffic_source"] = traffic_source()
     print(json.dumps(out), flush=True)
 
@@ -1035,7 +1160,7 @@ def main():
     ap.add_argument("--warmup", type=int, default=20)
     ap.add_argument("--workload", default="all",
                     help="all (default): the batched decode as the headline, the chunked prefill, one record per benchmark "
-                         "configuration and the measured ceilings; or one of: hbm_read_ceiling, mfma_issue_ceiling, prefill_step_ceiling, decode_step_fusion, " + ", ".join(WORKLOADS))
+                         "configuration and the measured ceilings; or one of: hbm_read_ceiling, mfma_issue_ceiling, prefill_step_ceiling, decode_step_fusion, prefill_step_fusion, " + ", ".join(WORKLOADS))
     ap.add_argument("--workgroups", type=int, default=0, help="planner split target (0: ask esp_attn_plan_hint)")
     ap.add_argument("--tables", default="scattered", choices=["scattered", "contiguous"],
                     help="block tables: a seeded permutation of the pool (the benchmark's definition) or address order")
@@ -1062,6 +1187,8 @@ def main():
         return run_all(args, torch)
     if args.workload == "decode_step_fusion":
         return decode_step_fusion(args, torch)
+    if args.workload == "prefill_step_fusion":
+        return prefill_step_fusion(args, torch)
     if args.workload == "hbm_read_ceiling":
         print(json.dumps({"metric": "plain read GB/s", "unit": "GB/s", "peak": HBM_PEAK_GBS, "sizes": Ceilings().hbm_read()}), flush=True)
         return

@@ -190,6 +190,7 @@ class DevicePass:
         self.static = static
         self.n_trees, self.n_tiles, self.n_jobs = len(trees), len(tiles), len(jobs)
         self.n_parts, self.n_rows = n_parts, n_rows
+        self.trees_host, self.tiles_host, self.jobs_host = trees, tiles, jobs
         self.trees = to_dev(np.ascontiguousarray(trees, dtype=abi.TREE_DT), device)
         self.tiles = to_dev(np.ascontiguousarray(tiles, dtype=abi.TILE_DT), device)
         self.jobs = to_dev(np.ascontiguousarray(jobs, dtype=abi.COMBINE_DT), device) if len(jobs) else None
