@@ -115,15 +115,17 @@ class Workload:
         self.alg_bytes = vis_keys * Hkv * HD * 2 * es + 2 * n_rows * H * HD * es + ((vis_keys + bt - 1) // bt) * 4
         self.alg_flops = 4 * HD * H * pairs
 
-    def step(self, i, ev=None):
-        """Enqueue one pass. ev: (start, end) events that take the dominant kernel's begin and end."""
+    def step(self, i, merge=True):
+        """Enqueue one pass: attention + split-K merge, one call."""
         dp = self.passes[i % self.n_sets]
-        if ev:
-            self.device.time_next(ev[0], ev[1])  # the launch of the attention kernel records into them
         if self.rows_in_pool:
-            dp.run(self.Q, None, None, self.pool, self.O)
+            dp.run(self.Q, None, None, self.pool, self.O, merge=merge)
         else:
-            dp.run(self.Q, self.Kb, self.Vb, self.pool, self.O)  # attention + split-K merge, one call
+            dp.run(self.Q, self.Kb, self.Vb, self.pool, self.O, merge=merge)
+
+    def launch(self, i, l=0):
+        """The pass's dominant kernel alone: the attention without the merge that follows it."""
+        self.step(i, merge=False)
 
 
 class PrepWorkload:
@@ -166,11 +168,12 @@ class PrepWorkload:
         self.alg_bytes = n_rows * (elems * 4 + elems * 2 + 2 * Hkv * HD * 2 + 16 + 16)  # X, Q K V, pool entries, pos, table
         self.alg_flops = 0
 
-    def step(self, i, ev=None):
-        if ev:
-            self.device.time_next(ev[0], ev[1])
+    def step(self, i):
         self.device.attn_prep(self.params, self.X[i % self.n_sets], self.qn_w, self.kn_w, self.pos, self.inv_freq, self.rope_sel,
                               self.Q, self.Kb, self.Vb, self.table, self.pool, self.n_rows)
+
+    def launch(self, i, l=0):
+        self.step(i)
 
 
 class GateWorkload:
@@ -203,12 +206,13 @@ class GateWorkload:
         self.alg_bytes = n_rows * D * 2 + H * D * 2 + (n_rows * H * 4 if dots_only else 2 * n_rows * H * HD * 2)
         self.alg_flops = 0
 
-    def step(self, i, ev=None):
-        if ev:
-            self.device.time_next(ev[0], ev[1])
+    def step(self, i):
         k = i % self.n_sets
         self.device.head_gate(self.params, None if self.dots_only else self.Os[k], self.X[k], self.Wg,
                               self.dots if self.dots_only else None, self.n_rows)
+
+    def launch(self, i, l=0):
+        self.step(i)
 
 
 class ChunkedPrefill:
@@ -264,11 +268,17 @@ class ChunkedPrefill:
         self.alg_flops = 4 * HD * H * pairs
         self.alg_bytes = 0
 
-    def step(self, i, ev=None):
+    def launch(self, i, l=0):
+        """The attention kernel of chunk l alone (the pool holds the sequence from the steps before)."""
+        dp, saves, rows = self.sets[i % self.n_sets][l]
+        if self.rows_in_pool:
+            dp.run(self.Q[rows], None, None, self.pool, self.O[rows], merge=False)
+        else:
+            dp.run(self.Q[rows], self.Kb[rows], self.Vb[rows], self.pool, self.O[rows], merge=False)
+
+    def step(self, i):
         d = self.device
         for c, (dp, saves, rows) in enumerate(self.sets[i % self.n_sets]):
-            if ev:
-                d.time_next(ev[c][0], ev[c][1])
             if self.rows_in_pool:
                 d.kv_save(self.params, self.Kb[rows], self.Vb[rows], self.pool, saves, rows.stop - rows.start)
                 dp.run(self.Q[rows], None, None, self.pool, self.O[rows])
@@ -295,10 +305,13 @@ class LayerMix:
         self.alg_flops = 5 * sliding.alg_flops + full.alg_flops
         self.O = full.O
 
-    def step(self, i, ev=None):
+    def step(self, i):
         for l in range(6):
             w = self.full if l == 5 else self.sliding
-            w.step(6 * i + l, ev[l] if ev else None)
+            w.step(6 * i + l)
+
+    def launch(self, i, l=0):
+        (self.full if l == 5 else self.sliding).launch(i)
 
 
 class DecodeStep:
@@ -329,7 +342,7 @@ class DecodeStep:
         for dp in w.passes:   # the position array serves the prep too: every pass holds it, windowed or not
             dp.pos = self.pos
 
-    def step(self, i, ev=None):
+    def step(self, i):
         w, d = self.w, self.device
         k = i % w.n_sets
         dp, X = w.passes[k], self.X[i % len(self.X)]
@@ -369,7 +382,7 @@ class PrefillStep:
         self.passes = [[device.DevicePass(w.params, dp.trees_host, dp.tiles_host, dp.jobs_host, dp.n_parts, dp.n_rows, table_of(chunks), None, None,
                                           rows_in_pool=folded) for dp, _, _ in chunks] for chunks in w.sets]
 
-    def step(self, i, ev=None):
+    def step(self, i):
         w, d = self.w, self.device
         k = i % w.n_sets
         for c, (dp0, saves, rows) in enumerate(w.sets[k]):
@@ -806,28 +819,31 @@ def spin(torch, ms):
     torch.cuda._sleep(int(_SPIN["per_ms"] * ms))
 
 
-def kernel_times(w, torch, n, first_step=0, step_seconds=0.0):
-    """Durations of the dominant kernel's launches over n steps, in milliseconds [n][launches per step], from HIP
-    event pairs handed to the launches themselves (esp_attn_time_next -> hipExtLaunchKernelGGL: the first event is
-    a marker in front of the dispatch, the second the dispatch's own end). The steps are enqueued behind a few
-    milliseconds of spinning, so marker and dispatch are both in the queue when the GPU reaches them: taken while
-    the GPU waits for the host instead (the host needs longer to enqueue an armed step than the GPU to run it),
-    the pair also spans the host's time between the two enqueues and reads 4 to 7 us long. (No spinning in front of
-    steps of 200 us and more: the host stays ahead of those by itself, and an idle stretch would let a chip that
-    runs at the clock its power budget allows cool down and read faster than it sustains.)"""
+def kernel_times(w, torch, n, first_step=0, step_seconds=0.0, reps=5):
+    """Durations of the dominant kernel's launches, in milliseconds [reps][launches per step]: for every launch of
+    a step, `reps` runs of that launch alone (w.launch: the attention without the merge behind it) repeated back to
+    back, timed by two events around the run and divided by the count. Consecutive launches of one stream follow
+    each other without a gap (the trace shows the next dispatch beginning where the last one ends), so the quotient
+    is the dispatch's own begin-to-end time, and nothing is inserted between the launches that could perturb them:
+    an event pair handed to every launch (hipExtLaunchKernelGGL) puts a marker in front of each dispatch, which the
+    trace shows costs the stream 9 to 14 us per launch and makes the kernel itself read 2 to 6 % longer. Runs of
+    short launches are enqueued behind a few milliseconds of spinning, so that the queue never runs dry."""
     nev = getattr(w, "launches_per_step", 1)
-    evs = [[(torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)) for _ in range(nev)] for _ in range(n)]
-    for pairs in evs:  # a first record creates the HIP events behind the torch objects
-        for a, b in pairs:
+    per = max(step_seconds / nev, 2e-6)
+    count = int(min(200, max(8, round(3e-3 / per))))   # launches per run: about 3 ms
+    out = np.zeros((reps, nev))
+    for l in range(nev):
+        for r in range(reps):
+            a, b = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+            if per < 2e-4:
+                spin(torch, 1.0 + 0.02 * count)
             a.record()
+            for i in range(count):
+                w.launch(first_step + r * count + i, l)
             b.record()
-    torch.cuda.synchronize()
-    if step_seconds < 2e-4:   # a step the host cannot enqueue faster than the GPU runs it; longer ones keep the queue full by themselves
-        spin(torch, 3.0 + 0.15 * n * nev)
-    for i, ev in enumerate(evs):
-        w.step(first_step + i, ev[0] if nev == 1 else ev)
-    torch.cuda.synchronize()
-    return np.array([[a.elapsed_time(b) for a, b in pairs] for pairs in evs])
+            torch.cuda.synchronize()
+            out[r, l] = a.elapsed_time(b) / count
+    return out
 
 
 def timed_run(w, torch, steps, warmup, kernel_samples=None):
@@ -853,8 +869,7 @@ def timed_run(w, torch, steps, warmup, kernel_samples=None):
         w.step(warmup + i)
     torch.cuda.synchronize()
     wall = (time.perf_counter() - t0) / steps
-    n = kernel_samples or max(8, min(steps, 40))
-    return wall, kernel_times(w, torch, n, warmup + steps, wall)
+    return wall, kernel_times(w, torch, steps, warmup + steps, wall)
 
 
 def kernel_name(w):
