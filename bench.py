@@ -492,6 +492,9 @@ def make_workload(name, workgroups=None, contiguous=False, page=16):
     if name == "c2_batched_decode":
         lens = synth.c2_lengths()
         return Workload_(name, 32, 4, 128, F16, page, [(L, 1) for L in lens], pool_pages=(65536) * 16 // page, seed=2)
+    if name.startswith("c2_equal_"):   # config 2's geometry with 16 sequences of one length: what a decode pass costs beside its bytes
+        L = int(name[len("c2_equal_"):])
+        return Workload_(name, 32, 4, 128, F16, page, [(L, 1)] * 16, pool_pages=(65536) * 16 // page, seed=2)
     if name == "c4_decode_sliding":
         return Workload_(name, 16, 8, 256, F16, page, [(16384, 1)] * 8, window=1024, pool_pages=(8 * 1025 * 4) * 16 // page, seed=4)
     if name == "c4_decode_global":
@@ -1175,7 +1178,7 @@ def main():
     ap.add_argument("--warmup", type=int, default=20)
     ap.add_argument("--workload", default="all",
                     help="all (default): the batched decode as the headline, the chunked prefill, one record per benchmark "
-                         "configuration and the measured ceilings; or one of: hbm_read_ceiling, mfma_issue_ceiling, prefill_step_ceiling, decode_step_fusion, prefill_step_fusion, " + ", ".join(WORKLOADS))
+                         "configuration and the measured ceilings; or c2_equal_<tokens> (16 equal sequences), or one of: hbm_read_ceiling, mfma_issue_ceiling, prefill_step_ceiling, decode_step_fusion, prefill_step_fusion, " + ", ".join(WORKLOADS))
     ap.add_argument("--workgroups", type=int, default=0, help="planner split target (0: ask esp_attn_plan_hint)")
     ap.add_argument("--tables", default="scattered", choices=["scattered", "contiguous"],
                     help="block tables: a seeded permutation of the pool (the benchmark's definition) or address order")
