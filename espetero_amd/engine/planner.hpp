@@ -260,6 +260,18 @@ inline void plan_tiles(AttnPlan& A, int groups, int window, const int32_t* pos, 
     }
     A.combine.push_back({t.base + rt.r, std::min(R, t.M - rt.r), part0, used});
   }
+  // Streaming kernel, balanced rule: every workgroup of the pass is resident at once and the hardware starts them
+  // in record order over a few microseconds. The tiles that own their tree's batch keys go first - behind their
+  // stream of cached keys they have a serial tail (the batch rows through the masked path) that the others'
+  // streaming then covers - and the rest follow by cached range, longest first. (Measured on the batched decode of
+  // 16 ragged sequences: 26.6 -> 25.8 us; with the owners of the batch keys last instead, 26.9 us.) The records'
+  // partial-record indices stay as assigned, so the merge order does not change.
+  if (o.balanced && o.item_steps == 0) {
+    std::stable_sort(A.tiles.begin(), A.tiles.end(), [](const esp_tile& x, const esp_tile& y) {
+      if (x.last != y.last) return x.last > y.last;
+      return (x.k1 - x.k0) > (y.k1 - y.k0);
+    });
+  }
 }
 
 }  // namespace espetero::engine

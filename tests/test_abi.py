@@ -173,17 +173,18 @@ def test_validate_accepts_a_planned_pass_and_names_the_first_bad_record():
         with pytest.raises(abi.EspError, match=match):
             device.validate(p, tiles, trees, jobs, n_parts, n_rows, blocks, pool_blocks)
 
+    i0 = int(np.flatnonzero(tiles["tree"] == 0)[0])   # a record of the first tree (4 rows, 1000 cached keys), wherever the planner lists it
     t = tiles.copy(); t[1]["tree"] = 3
     bad("tile 1: tree 3 of 3", tiles=t)
-    t = tiles.copy(); t[0]["part"] = n_parts
-    bad("tile 0: partial record", tiles=t)
-    t = tiles.copy(); t[0]["r0"] = 4
-    bad("tile 0: first row 4 outside", tiles=t)
-    t = tiles.copy(); t[0]["pad"] = 7
-    bad("tile 0: pad 7", tiles=t)
-    t = tiles.copy(); t[0]["k1"] = 1001
-    bad("tile 0: cached range", tiles=t)
-    t = tiles.copy(); t[-1]["b0"] = 9
+    t = tiles.copy(); t[i0]["part"] = n_parts
+    bad(f"tile {i0}: partial record", tiles=t)
+    t = tiles.copy(); t[i0]["r0"] = 4
+    bad(f"tile {i0}: first row 4 outside", tiles=t)
+    t = tiles.copy(); t[i0]["pad"] = 7
+    bad(f"tile {i0}: pad 7", tiles=t)
+    t = tiles.copy(); t[i0]["k1"] = 1001
+    bad(f"tile {i0}: cached range", tiles=t)
+    t = tiles.copy(); t[i0]["b0"] = 9
     bad("first batch key 9", tiles=t)
     split = [i for i in range(len(tiles)) if tiles[i]["part"] >= 0]
     t = tiles.copy(); t[split[1]]["part"] = t[split[0]]["part"]
