@@ -506,6 +506,9 @@ def make_workload(name, workgroups=None, contiguous=False, page=16):
     # gemma.h:125-150), on config 4's sequences: what config 4's "global" layers are in the real model.
     if name == "g4_global512_decode":
         return Workload_(name, 16, 2, 512, F16, page, [(16384, 1)] * 8, pool_pages=(8 * 1025 * 4) * 16 // page, seed=6)
+    if name in ("g4_global512_verify", "g4_global512_verify_2row_tiles"):   # 4-row verify trees there: 32 packed rows in one pass over K / V, or as two 2-row tiles
+        return Workload_(name, 16, 2, 512, F16, page, [(16384, 4)] * 8, rows_per_tile=4 if name.endswith("verify") else 2,
+                        desc_fn=lambda M: synth.verify_desc(M, 1), pool_pages=(8 * 1025 * 4) * 16 // page, seed=6)
     if name == "g4_global512_prefill":
         return Workload_(name, 16, 2, 512, F16, page, [(15360, 1024)] * 8, rows_per_tile=128, pool_pages=(8 * 1024 * 2) * 16 // page,
                         seed=6, bound="mfma")
@@ -551,7 +554,8 @@ def traffic_source():
 WORKLOADS = ["c1_single_decode", "c2_batched_decode", "c3_prefill_p0", "c3_prefill_p2048", "c3_prefill_p4096",
              "c3_prefill_p6144", "c4_decode_sliding", "c4_decode_global", "c4_prefill_sliding", "c4_prefill_global",
              "c5_verify", "c4_decode_mix", "c4_prefill_mix", "c3_chunked_prefill", "c3_chunked_prefill_kb", "c3_attn_prep", "c4_attn_prep",
-             "c4_head_gate", "c4_head_gate_dots", "g4_global512_decode", "g4_global512_prefill"]
+             "c4_head_gate", "c4_head_gate_dots", "g4_global512_decode", "g4_global512_verify", "g4_global512_verify_2row_tiles",
+             "g4_global512_prefill"]
 
 
 def cpu_baseline(w, budget_s=20.0):

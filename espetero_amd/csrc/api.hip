@@ -78,7 +78,8 @@ int check_params(const esp_attn_params* p, char* err, size_t errlen) {
 int family(const esp_attn_params* p) {
   const int packed = p->rows_per_tile * (p->H / p->Hkv);
   const int nc = (packed + 15) / 16;
-  if (nc == 1 || (nc == 2 && p->head_dim == 128)) return nc;  // two column tiles fit the registers at head dim 128 only
+  // two column tiles: in one wavefront's registers at head dim 128, as two wavefront pairs of one workgroup at head dim 512
+  if (nc == 1 || (nc == 2 && (p->head_dim == 128 || p->head_dim == 512))) return nc;
   return -1;
 }
 

@@ -29,7 +29,8 @@
 // threadgroup memory the same way, 80_gemma.metal:272-282), both run the same softmax and
 // each accumulates its 256 output dims. A workgroup is one such pair (128 threads, two
 // workgroups per compute unit), so the barrier ties no more than the two wavefronts
-// that need each other.
+// that need each other - or, for 17 to 32 packed rows, two pairs with one column tile each
+// that walk the same units together, so that K and V come from memory once for both.
 #include <type_traits>
 
 #include "common.hpp"
@@ -134,12 +135,17 @@ struct Unit {  // operands of one unit of SBU 16-key sub-blocks
 // head, which it also appends to the pool): no prep dispatch in front, no Q / Kb / Vb round trip through
 // memory. For passes whose trees have at most rows_per_tile <= 4 rows (decode, short verify trees).
 template <int DT, int HD, int NC, int SBU, int BT, int OCC, int FUSED>
-__global__ __launch_bounds__(HD >= 512 ? 128 : 256, OCC) void attn_stream_kernel(const KArgs a, const PrepArgs pa) {
+__global__ __launch_bounds__(HD >= 512 ? 128 * NC : 256, OCC) void attn_stream_kernel(const KArgs a, const PrepArgs pa) {
   constexpr bool PAIR = HD >= 512;      // two wavefronts per unit, HW dims each
   constexpr int HW = PAIR ? HD / 2 : HD;
   constexpr int NS = PAIR ? 1 : 4;       // unit streams of the workgroup
-  constexpr int NW = PAIR ? 2 : 4;       // wavefronts of the workgroup
-  static_assert(!PAIR || (NC == 1 && SBU == 1), "paired wavefronts: one column tile, 16-key units");
+  constexpr int NW = PAIR ? 2 * NC : 4;  // wavefronts of the workgroup
+  // Column tiles a wavefront holds. Paired wavefronts have registers for one; a second column tile (32 packed rows:
+  // a 4-row verify tree at 8 query heads per KV head) is a second pair of the same workgroup that walks the same
+  // units in step with the first - one barrier per unit ties all four wavefronts - so that its requests for the
+  // unit's K and V meet the first pair's in L2 and the pool is read from memory once.
+  constexpr int NCW = PAIR ? 1 : NC;
+  static_assert(!PAIR || SBU == 1, "paired wavefronts: 16-key units");
   static_assert(!PAIR || !FUSED, "the fused prologue is built for one wavefront per head");
   constexpr int kFusedRows = 4;  // most rows of a tile on the fused path
   constexpr int KK = HW / 32, MT = HW / 16, LDO = HD + 4, UK = 16 * SBU, USH = SBU == 2 ? 5 : 4;
@@ -151,6 +157,7 @@ __global__ __launch_bounds__(HD >= 512 ? 128 : 256, OCC) void attn_stream_kernel
   const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
   const int strm = PAIR ? 0 : wave;          // which of the NS unit streams
   const int dw = PAIR ? (wave & 1) * HW : 0; // first dim of this wavefront's share of the head
+  const int cbase = PAIR ? 16 * (wave >> 1) : 0;  // first packed row (column) of this wavefront's column tiles
   const int c16 = lane & 15, q4 = lane >> 4;
   esp_tile tile = a.tiles[blockIdx.y];
   const esp_tree tree = a.trees[tile.tree];
@@ -225,13 +232,13 @@ __global__ __launch_bounds__(HD >= 512 ? 128 : 256, OCC) void attn_stream_kernel
   }
 
   // ---- this lane's packed rows: Q fragments, position, descriptor
-  u32x4 qf[NC][KK];
-  int rr[NC], qpos[NC];
-  int4 dsc[NC];
-  bool ok[NC];
+  u32x4 qf[NCW][KK];
+  int rr[NCW], qpos[NCW];
+  int4 dsc[NCW];
+  bool ok[NCW];
 #pragma unroll
-  for (int c = 0; c < NC; ++c) {
-    const int col = 16 * c + c16;
+  for (int c = 0; c < NCW; ++c) {
+    const int col = cbase + 16 * c + c16;
     const int m = col / a.G, hg = col - m * a.G;
     ok[c] = col < a.cols && m < rows_live;
     rr[c] = rr0 + m;
@@ -261,9 +268,17 @@ __global__ __launch_bounds__(HD >= 512 ? 128 : 256, OCC) void attn_stream_kernel
     int lo_key = tile.k0;  // first key every row sees
     if (a.window > 0) {
       int qm = INT32_MIN;
+      if constexpr (PAIR && NC > 1) {
+        // The pairs of the workgroup hold different rows but pass the same barriers: the range every row sees
+        // is taken over all rows of the tile, by every wavefront alike.
+        for (int m = lane; m < rows_live; m += 64) qm = max(qm, a.pos[tile.r0 + m].x);
 #pragma unroll
-      for (int c = 0; c < NC; ++c)
-        if (ok[c]) qm = max(qm, qpos[c]);
+        for (int o = 32; o >= 16; o >>= 1) qm = max(qm, __shfl_xor(qm, o));
+      } else {
+#pragma unroll
+        for (int c = 0; c < NCW; ++c)
+          if (ok[c]) qm = max(qm, qpos[c]);
+      }
 #pragma unroll
       for (int o = 8; o >= 1; o >>= 1) qm = max(qm, __shfl_xor(qm, o));
       qm = __builtin_amdgcn_readfirstlane(qm);  // the 16 columns repeat in every quarter of the wavefront
@@ -274,10 +289,10 @@ __global__ __launch_bounds__(HD >= 512 ? 128 : 256, OCC) void attn_stream_kernel
   }
   const int n_lo = ui0 - cp0, n_edge = n_cached - (ui1 - ui0);
   int k_last = -1, bp0 = 0, n_batch = 0;  // batch range: set once the cached range has been streamed
-  f32x4 acc[NC][MT];
-  float m_run[NC], l_run[NC];  // running max in log2 units of the scaled score; this lane's share of the sum
+  f32x4 acc[NCW][MT];
+  float m_run[NCW], l_run[NCW];  // running max in log2 units of the scaled score; this lane's share of the sum
 #pragma unroll
-  for (int c = 0; c < NC; ++c) {
+  for (int c = 0; c < NCW; ++c) {
     m_run[c] = -INFINITY;
     l_run[c] = 0.0f;
 #pragma unroll
@@ -301,10 +316,15 @@ __global__ __launch_bounds__(HD >= 512 ? 128 : 256, OCC) void attn_stream_kernel
       constexpr int ks = 32, vs = 16 * kVtDim;
       // Every cached byte is read once per pass: non-temporal loads keep the stream from displacing
       // what the caches could still serve (measured: 184 -> 164 us on 1 GB of keys at head dim 256).
+      // (Two pairs that walk the same units want the opposite: the first pair's lines must still be in L2 when the
+      // second pair asks for them, so those loads are ordinary ones.)
+      constexpr bool kOnce = !(PAIR && NC > 1);
 #pragma unroll
-      for (int kk = 0; kk < KK; ++kk) U.k[sb][kk] = __builtin_nontemporal_load(reinterpret_cast<const u32x4*>(kp + ks * kk));
+      for (int kk = 0; kk < KK; ++kk)
+        U.k[sb][kk] = kOnce ? __builtin_nontemporal_load(reinterpret_cast<const u32x4*>(kp + ks * kk)) : *reinterpret_cast<const u32x4*>(kp + ks * kk);
 #pragma unroll
-      for (int mt = 0; mt < MT; ++mt) U.v[sb][mt] = __builtin_nontemporal_load(reinterpret_cast<const u32x2*>(vp + vs * mt));
+      for (int mt = 0; mt < MT; ++mt)
+        U.v[sb][mt] = kOnce ? __builtin_nontemporal_load(reinterpret_cast<const u32x2*>(vp + vs * mt)) : *reinterpret_cast<const u32x2*>(vp + vs * mt);
     }
   };
 
@@ -367,9 +387,9 @@ __global__ __launch_bounds__(HD >= 512 ? 128 : 256, OCC) void attn_stream_kernel
   // in between, which the partner reaches only after it has read the slot.
   int n_done = 0;  // units this wavefront has computed
   f32x4* xch = reinterpret_cast<f32x4*>(smem + NS * NC * 16 * (LDO + 2));
-  auto scores = [&](const Unit<HW, SBU>& U, f32x4 (&s)[NC][SBU]) {
+  auto scores = [&](const Unit<HW, SBU>& U, f32x4 (&s)[NCW][SBU]) {
 #pragma unroll
-    for (int c = 0; c < NC; ++c)
+    for (int c = 0; c < NCW; ++c)
 #pragma unroll
       for (int sb = 0; sb < SBU; ++sb) {
         s[c][sb] = f32x4{0, 0, 0, 0};
@@ -386,12 +406,12 @@ __global__ __launch_bounds__(HD >= 512 ? 128 : 256, OCC) void attn_stream_kernel
     }
   };
   // Online softmax over a unit's scores x (log2 units, -inf where masked), then O^T += V^T . P^T.
-  auto softmax_pv = [&](const Unit<HW, SBU>& U, f32x4 (&x)[NC][SBU], const float (&mx_in)[NC]) {
+  auto softmax_pv = [&](const Unit<HW, SBU>& U, f32x4 (&x)[NCW][SBU], const float (&mx_in)[NCW]) {
     bool any_change = false;
-    u32x2 pb[NC][SBU];
-    float corr[NC];
+    u32x2 pb[NCW][SBU];
+    float corr[NCW];
 #pragma unroll
-    for (int c = 0; c < NC; ++c) {
+    for (int c = 0; c < NCW; ++c) {
       float mx = mx_in[c];
       mx = fmaxf(mx, __shfl_xor(mx, 16));
       mx = fmaxf(mx, __shfl_xor(mx, 32));
@@ -415,7 +435,7 @@ __global__ __launch_bounds__(HD >= 512 ? 128 : 256, OCC) void attn_stream_kernel
     }
     if (__any(any_change)) {
 #pragma unroll
-      for (int c = 0; c < NC; ++c)
+      for (int c = 0; c < NCW; ++c)
 #pragma unroll
         for (int mt = 0; mt < MT; ++mt) acc[c][mt] *= corr[c];
     }
@@ -424,22 +444,22 @@ __global__ __launch_bounds__(HD >= 512 ? 128 : 256, OCC) void attn_stream_kernel
       if constexpr (SBU == 2) {
         const u32x4 va = {U.v[0][mt].x, U.v[0][mt].y, U.v[1][mt].x, U.v[1][mt].y};
 #pragma unroll
-        for (int c = 0; c < NC; ++c)
+        for (int c = 0; c < NCW; ++c)
           acc[c][mt] = mfma16x32<DT>(va, u32x4{pb[c][0].x, pb[c][0].y, pb[c][1].x, pb[c][1].y}, acc[c][mt]);
       } else {
 #pragma unroll
-        for (int c = 0; c < NC; ++c) acc[c][mt] = mfma16x16<DT>(U.v[0][mt], pb[c][0], acc[c][mt]);
+        for (int c = 0; c < NCW; ++c) acc[c][mt] = mfma16x16<DT>(U.v[0][mt], pb[c][0], acc[c][mt]);
       }
     }
   };
 
   // Interior unit: every key visible to every row.
   auto compute_interior = [&](const Unit<HW, SBU>& U) {
-    f32x4 s[NC][SBU];
+    f32x4 s[NCW][SBU];
     scores(U, s);
-    float mx[NC];
+    float mx[NCW];
 #pragma unroll
-    for (int c = 0; c < NC; ++c) {
+    for (int c = 0; c < NCW; ++c) {
       mx[c] = -INFINITY;
 #pragma unroll
       for (int sb = 0; sb < SBU; ++sb)
@@ -471,11 +491,11 @@ __global__ __launch_bounds__(HD >= 512 ? 128 : 256, OCC) void attn_stream_kernel
         }
       }
     }
-    f32x4 s[NC][SBU];
+    f32x4 s[NCW][SBU];
     scores(U, s);
     // The first readers of s sit behind the branches of the visibility rules below.
 #pragma unroll
-    for (int c = 0; c < NC; ++c)
+    for (int c = 0; c < NCW; ++c)
 #pragma unroll
       for (int sb = 0; sb < SBU; ++sb) mfma_settle(s[c][sb]);
     int kpos[SBU][4];
@@ -488,9 +508,9 @@ __global__ __launch_bounds__(HD >= 512 ? 128 : 256, OCC) void attn_stream_kernel
           kpos[sb][e] = a.pos[tree.base + min(j, tree.M - 1)].x;
         }
     }
-    float mx[NC];
+    float mx[NCW];
 #pragma unroll
-    for (int c = 0; c < NC; ++c) {
+    for (int c = 0; c < NCW; ++c) {
       mx[c] = -INFINITY;
 #pragma unroll
       for (int sb = 0; sb < SBU; ++sb)
@@ -548,9 +568,16 @@ __global__ __launch_bounds__(HD >= 512 ? 128 : 256, OCC) void attn_stream_kernel
       // Last batch key any row of the tile sees: its last row, a root it sees whole
       // (anc_len), the end of its image (bidi).
       int kl = -1;
+      if constexpr (PAIR && NC > 1) {  // over all rows of the tile: every pair scans the same batch units
+        for (int m = lane; m < rows_live; m += 64) {
+          const int4 dm = a.desc ? a.desc[tile.r0 + m] : make_int4(0, 0, 0, 0);
+          kl = max(kl, max(rr0 + m, max(dm.z - 1, a.bidi ? dm.w - 1 : -1)));
+        }
+      } else {
 #pragma unroll
-      for (int c = 0; c < NC; ++c)
-        if (ok[c]) kl = max(kl, max(rr[c], max(dsc[c].z - 1, a.bidi ? dsc[c].w - 1 : -1)));
+        for (int c = 0; c < NCW; ++c)
+          if (ok[c]) kl = max(kl, max(rr[c], max(dsc[c].z - 1, a.bidi ? dsc[c].w - 1 : -1)));
+      }
 #pragma unroll
       for (int o = 32; o >= 1; o >>= 1) kl = max(kl, __shfl_xor(kl, o));
       // fused: the batch keys are the tile's own rows in LDS, never more than the tile holds
@@ -580,20 +607,20 @@ __global__ __launch_bounds__(HD >= 512 ? 128 : 256, OCC) void attn_stream_kernel
   float* o_sh = smem;                          // [NS][NC * 16][LDO]
   float* ml_sh = smem + NS * NC * 16 * LDO;    // [NS][NC * 16][2]
 #pragma unroll
-  for (int c = 0; c < NC; ++c) {
+  for (int c = 0; c < NCW; ++c) {
     float l = l_run[c];
     l += __shfl_xor(l, 16);
     l += __shfl_xor(l, 32);
     l_run[c] = l;
     if (q4 == 0) {
-      ml_sh[(strm * NC * 16 + 16 * c + c16) * 2] = m_run[c];
-      ml_sh[(strm * NC * 16 + 16 * c + c16) * 2 + 1] = l;
+      ml_sh[(strm * NC * 16 + cbase + 16 * c + c16) * 2] = m_run[c];
+      ml_sh[(strm * NC * 16 + cbase + 16 * c + c16) * 2 + 1] = l;
     }
   }
   __syncthreads();
 #pragma unroll
-  for (int c = 0; c < NC; ++c) {
-    const int col = 16 * c + c16;
+  for (int c = 0; c < NCW; ++c) {
+    const int col = cbase + 16 * c + c16;
     float M = -INFINITY;
 #pragma unroll
     for (int w = 0; w < NS; ++w) M = fmaxf(M, ml_sh[(w * NC * 16 + col) * 2]);
@@ -663,15 +690,15 @@ __global__ __launch_bounds__(256) void attn_combine_kernel(const KArgs a, const 
 }
 
 size_t stream_smem_bytes(int HD, int NC) {
-  if (HD >= 512) return size_t(NC * 16) * (HD + 4 + 2) * sizeof(float) + 2 * 2 * 64 * 16;  // one stream + the partial S^T slots
+  if (HD >= 512) return size_t(NC * 16) * (HD + 4 + 2) * sizeof(float) + 2 * (2 * NC) * 64 * 16;  // one stream + the partial S^T slots of every wavefront
   return size_t(4 * NC * 16) * (HD + 4 + 2) * sizeof(float);
 }
 
 // Resident workgroups per CU of each variant: the single-column-tile head_dim-128 kernel
 // fits two; the wider ones need more than 256 VGPRs and run one.
 constexpr int stream_occ(int HD, int NC) { return (HD == 128 && NC == 1) ? 2 : 1; }  // wavefronts per SIMD
-// Head dim 512: workgroups of two wavefronts, one per SIMD: two fill a compute unit.
-int stream_workgroups_per_cu(int HD, int NC) { return HD >= 512 ? 2 : stream_occ(HD, NC); }
+// Head dim 512: workgroups of one wavefront pair per column tile, one wavefront per SIMD: two pairs fill a compute unit.
+int stream_workgroups_per_cu(int HD, int NC) { return HD >= 512 ? 2 / NC : stream_occ(HD, NC); }
 
 template <int DT, int HD, int NC, int FUSED>
 static hipError_t launch_stream_t(const KArgs& a, const PrepArgs& pa, int n_tiles, hipStream_t st) {
@@ -683,7 +710,7 @@ static hipError_t launch_stream_t(const KArgs& a, const PrepArgs& pa, int n_tile
   const auto k = a.bt == 16 ? k16 : kbt;
   const hipError_t e = a.bt == 16 ? allow_dynamic_lds<k16>(smem) : allow_dynamic_lds<kbt>(smem);
   if (e != hipSuccess) return e;
-  launch_timed(k, dim3(a.Hkv, n_tiles), dim3(HD >= 512 ? 128 : 256), smem, st, a, pa);
+  launch_timed(k, dim3(a.Hkv, n_tiles), dim3(HD >= 512 ? 128 * NC : 256), smem, st, a, pa);
   return hipGetLastError();
 }
 
@@ -708,14 +735,16 @@ hipError_t stream_init_attributes() {
   if (e == hipSuccess) e = stream_attributes_t<ESP_F16, 128, 2>();
   if (e == hipSuccess) e = stream_attributes_t<ESP_F16, 256, 1>();
   if (e == hipSuccess) e = stream_attributes_t<ESP_F16, 512, 1>();
+  if (e == hipSuccess) e = stream_attributes_t<ESP_F16, 512, 2>();
   if (e == hipSuccess) e = stream_attributes_t<ESP_BF16, 128, 1>();
   if (e == hipSuccess) e = stream_attributes_t<ESP_BF16, 128, 2>();
   if (e == hipSuccess) e = stream_attributes_t<ESP_BF16, 256, 1>();
   if (e == hipSuccess) e = stream_attributes_t<ESP_BF16, 512, 1>();
+  if (e == hipSuccess) e = stream_attributes_t<ESP_BF16, 512, 2>();
   return e;
 }
 
-// dt, HD, NC are validated by the caller: (HD, NC) in {(128, 1), (128, 2), (256, 1), (512, 1)}; with a prep
+// dt, HD, NC are validated by the caller: (HD, NC) in {(128, 1), (128, 2), (256, 1), (512, 1), (512, 2)}; with a prep
 // argument block (the fused prologue) head dim 512 is not served.
 hipError_t launch_stream(int dt, int HD, int NC, const KArgs& a, const PrepArgs* pa, int n_tiles, hipStream_t st) {
   static const PrepArgs none{};
@@ -729,9 +758,11 @@ hipError_t launch_stream(int dt, int HD, int NC, const KArgs& a, const PrepArgs*
   ESP_STREAM_CASE(ESP_BF16, 128, 2)
   ESP_STREAM_CASE(ESP_BF16, 256, 1)
 #undef ESP_STREAM_CASE
-  if (HD == 512 && NC == 1 && !pa) {
-    if (dt == ESP_F16) return launch_stream_t<ESP_F16, 512, 1, 0>(a, none, n_tiles, st);
-    if (dt == ESP_BF16) return launch_stream_t<ESP_BF16, 512, 1, 0>(a, none, n_tiles, st);
+  if (HD == 512 && !pa) {
+    if (dt == ESP_F16 && NC == 1) return launch_stream_t<ESP_F16, 512, 1, 0>(a, none, n_tiles, st);
+    if (dt == ESP_BF16 && NC == 1) return launch_stream_t<ESP_BF16, 512, 1, 0>(a, none, n_tiles, st);
+    if (dt == ESP_F16 && NC == 2) return launch_stream_t<ESP_F16, 512, 2, 0>(a, none, n_tiles, st);
+    if (dt == ESP_BF16 && NC == 2) return launch_stream_t<ESP_BF16, 512, 2, 0>(a, none, n_tiles, st);
   }
   return hipErrorInvalidValue;
 }

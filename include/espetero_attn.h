@@ -97,7 +97,7 @@ typedef struct esp_attn_params {
   int32_t H;             /* query heads */
   int32_t Hkv;           /* KV heads; H % Hkv == 0, group G = H / Hkv */
   int32_t head_dim;      /* 128, 256 or 512 (512: the g4_attention512_s* / g4_attention_dec512_g* instantiations,
-                            80_:355-358, :561-564; at most 16 packed rows on the streaming kernel, 64-row tiles
+                            80_:355-358, :561-564; up to 32 packed rows on the streaming kernel like the other head dims, 64-row tiles
                             on the tiled one: esp_attn_plan_hint's max_rows) */
   int32_t dtype;         /* ESP_F16 | ESP_BF16: element type of Q, Kb, Vb, pool and O */
   int32_t q_ld;          /* Q / O row stride in elements (>= H * head_dim) */

@@ -59,6 +59,13 @@ def test_stream_kernel_matches_checker(kw):
     dict(seqs=((900, 1), (40, 1)), H=4, Hkv=1, window=128, rows_per_tile=1),        # window (not a Gemma shape; same code)
     dict(seqs=((90, 7),), H=4, Hkv=2, rows_per_tile=8),                             # G = 2, 8-row tiles: batch keys
     dict(seqs=((700, 4), (33, 4)), H=8, Hkv=1, rows_per_tile=2, desc_fn=lambda M: synth.verify_desc(M, 1)),  # a 4-row verify tree as two 2-row tiles
+    # 32 packed rows: two wavefront pairs of one workgroup, one column tile each, walking the same units
+    dict(seqs=((700, 4), (33, 4), (0, 3)), H=8, Hkv=1, rows_per_tile=4, desc_fn=lambda M: synth.verify_desc(M, 1)),  # a 4-row verify tree in one pass
+    dict(seqs=((5000, 4), (900, 2)), H=16, Hkv=2, rows_per_tile=4, dtype=abi.ESP_BF16),                # split + merge, ragged last tile, bf16
+    dict(seqs=((300, 1), (77, 1)), H=32, Hkv=1, rows_per_tile=1),                                        # G = 32
+    dict(seqs=((900, 7), (40, 3)), H=12, Hkv=3, window=128, rows_per_tile=8),                           # G = 4, 8-row tiles: the pairs hold different rows under a window
+    dict(seqs=((900, 4), (2000, 4)), H=8, Hkv=1, window=256, ring_layer=True, rows_per_tile=4, desc_fn=lambda M: synth.verify_desc(M, 2)),
+    dict(seqs=((200, 8),), H=4, Hkv=1, rows_per_tile=8, bt=64, bidi=1, desc_fn=lambda M: synth.image_desc(M, 2, 6)),   # image span across the two pairs' rows
 ])
 def test_stream_kernel_head_dim_512(kw):
     _check(small_case(seed=37, HD=512, fill_unused=True, **kw))
@@ -200,7 +207,7 @@ def test_sharp_softmax_with_a_moving_maximum(kw, dtype):
     dict(seqs=((128, 128),), bt=64, H=4, Hkv=2),
     dict(seqs=((100, 140),), H=2, Hkv=1, bidi=1, desc_fn=lambda M: synth.image_desc(M, 10, 90)),   # bidirectional span
     dict(seqs=((1203, 64), (700, 40)), bt=64, H=4, Hkv=2, fill_unused=True),  # long cached ranges, ragged end
-    dict(seqs=((100, 1), (33, 1)), H=32, Hkv=1, rows_per_tile=1),       # G = 32: more packed rows than the streaming kernel takes at 512
+    dict(seqs=((100, 2), (33, 1)), H=32, Hkv=1, rows_per_tile=2),       # G = 32, two rows: more packed rows (64) than the streaming kernel takes
     dict(seqs=((150, 20),), H=4, Hkv=2, rows_per_tile=24),              # tiles smaller than the kernel's 64 rows
 ])
 def test_tiled_kernel_head_dim_512(kw):

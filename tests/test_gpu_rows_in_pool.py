@@ -56,6 +56,7 @@ def test_tiled_kernel_reads_its_rows_from_the_pool(kw):
     dict(seqs=((1030, 4), (90, 4)), rows_per_tile=4, desc_fn=lambda M: synth.verify_desc(M, 1)),   # a root and its chain
     dict(seqs=((777, 1), (100, 1)), H=4, Hkv=2, HD=256, rows_per_tile=1),
     dict(seqs=((300, 2),), H=8, Hkv=2, HD=512, rows_per_tile=2, dtype=abi.ESP_BF16),
+    dict(seqs=((300, 4), (50, 4)), H=8, Hkv=1, HD=512, rows_per_tile=4, desc_fn=lambda M: synth.verify_desc(M, 1)),   # two wavefront pairs
     dict(seqs=((400, 6), (64, 2)), H=4, Hkv=2, rows_per_tile=8, bt=64),            # short causal chunks on the streaming kernel
     dict(seqs=((900, 1), (2000, 1)), window=256, ring_layer=True, rows_per_tile=1),  # rings: a decode row overwrites what no row sees
     dict(seqs=((5000, 1), (900, 1)), H=32, Hkv=4, rows_per_tile=1, split=256),     # split ranges: the last part owns the row
