@@ -157,19 +157,45 @@ __global__ __launch_bounds__(256, OCC) void attn_tiled_kernel(const KArgs a, int
   const bool in_pool = a.Kb == nullptr;
   const int pool_shift = tree.P - tree.base;  // pool position of absolute row r: r + pool_shift
 
-  // Windowed layers: do this tile's batch keys need the per-key position test at all? Not when
-  // the oldest position among them is inside the window of the row with the largest position.
+  // Windowed layers: do this tile's batch keys need a window test at all? Not when the oldest position among
+  // them is inside the window of the row with the largest position. Where they do and their positions rise by
+  // one per row (position of row j = j + pos_shift: a plain chunk of prompt), the window is one more lower
+  // bound in row numbers, j >= qpos - w_off, and a step whose rows lie at or above bw_lo is inside every row's
+  // window; only other position patterns (trees) take the per-key position test.
   bool batch_window = false;
+  int w_off = 1 << 30, bw_lo = INT32_MIN;
   if (a.window > 0 && n_b > 0) {
-    int kp = INT32_MAX;
-    for (int j = tile.b0 + int(threadIdx.x); j <= k_last; j += 256) kp = min(kp, a.pos[tree.base + j].x);
+    int kp = INT32_MAX, dmin = INT32_MAX, dmax = INT32_MIN;
+    for (int j = tile.b0 + int(threadIdx.x); j <= k_last; j += 256) {
+      const int p = a.pos[tree.base + j].x;
+      kp = min(kp, p);
+      dmin = min(dmin, p - j);
+      dmax = max(dmax, p - j);
+    }
 #pragma unroll
-    for (int o = 32; o >= 1; o >>= 1) kp = min(kp, __shfl_xor(kp, o));
+    for (int o = 32; o >= 1; o >>= 1) {
+      kp = min(kp, __shfl_xor(kp, o));
+      dmin = min(dmin, __shfl_xor(dmin, o));
+      dmax = max(dmax, __shfl_xor(dmax, o));
+    }
     __syncthreads();  // every wavefront has read the facts above
-    if (lane == 0) red[wave][0] = kp;
+    if (lane == 0) {
+      red[wave][0] = kp;
+      red[wave][1] = dmin;
+      red[wave][2] = dmax;
+    }
     __syncthreads();
-    kp = min(min(red[0][0], red[1][0]), min(red[2][0], red[3][0]));
-    batch_window = qpos_max - __builtin_amdgcn_readfirstlane(kp) >= a.window;
+    kp = __builtin_amdgcn_readfirstlane(min(min(red[0][0], red[1][0]), min(red[2][0], red[3][0])));
+    dmin = __builtin_amdgcn_readfirstlane(min(min(red[0][1], red[1][1]), min(red[2][1], red[3][1])));
+    dmax = __builtin_amdgcn_readfirstlane(max(max(red[0][2], red[1][2]), max(red[2][2], red[3][2])));
+    if (qpos_max - kp >= a.window) {
+      if (dmin == dmax) {
+        w_off = a.window - 1 + dmin;
+        bw_lo = qpos_max - w_off;
+      } else {
+        batch_window = true;
+      }
+    }
   }
 
   // Block ids of this wavefront's cached sub-blocks, 64 steps at a time: lane l holds the
@@ -392,7 +418,7 @@ __global__ __launch_bounds__(256, OCC) void attn_tiled_kernel(const KArgs a, int
         half_full = j0 >= tile.k0 && j0 + 32 <= tile.k1 && (a.window == 0 || qpos_max - j0 < a.window);
       } else if (s0 >= n_c && s0 + 2 <= n_sb) {
         const int j0 = ((a0 + s0 - n_c) << 4) - tree.base;
-        half_full = !batch_window && j0 >= seg_max && j0 + 31 <= rr0 + 32 * wave && j0 >= tile.b0;
+        half_full = !batch_window && j0 >= seg_max && j0 + 31 <= rr0 + 32 * wave && j0 >= tile.b0 && j0 >= bw_lo;
       } else {
         half_full = false;
       }
@@ -412,7 +438,7 @@ __global__ __launch_bounds__(256, OCC) void attn_tiled_kernel(const KArgs a, int
         } else if (batch) {
           // b0 is the first batch key any row of the tile sees (the window's lower edge; 0 without one). The
           // first sub-block starts at a multiple of 16 rows at or below it: what lies below b0 is invisible.
-          lo = max(d.x, tile.b0);
+          lo = max(max(d.x, tile.b0), qpos - w_off);
           hi = min(k_last, (a.bidi && d.w > 0) ? max(rr, d.w - 1) : rr);
           anc = min(d.z, k_last + 1);
         } else {
@@ -667,7 +693,7 @@ __global__ __launch_bounds__(256, OCC) void attn_tiled_kernel(const KArgs a, int
     int_lo = lo_key <= first ? 0 : (lo_key - first + 63) >> 6;
     c_hi = ((tile.k1 >> 4) - c0) >> 2;  // steps wholly inside the cached range
     if (n_b > 0 && !batch_window && !anc_any && seg_max != INT32_MAX) {
-      const int lo_b = max(max(tile.b0, seg_max), 0);
+      const int lo_b = max(max(max(tile.b0, seg_max), bw_lo), 0);
       const int g_lo = (tree.base + lo_b + 15) >> 4;           // first group of 16 rows wholly at or above lo_b
       const int g_hi = ((tree.base + rr0) >> 4) - 1;           // last group wholly below the tile's first row
       const int s_lo = n_c + g_lo - a0, s_hi = n_c + g_hi - a0;  // as sub-blocks of the range

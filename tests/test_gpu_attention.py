@@ -242,6 +242,32 @@ def test_tiled_kernel_one_row_remainder_tile_on_a_windowed_layer(HD, rows):
                           window=window, ring_layer=ring, fill_unused=not ring))
 
 
+@pytest.mark.parametrize("HD,rows,dtype", [(128, 128, abi.ESP_F16), (128, 64, abi.ESP_BF16), (256, 128, abi.ESP_BF16),
+                                           (256, 32, abi.ESP_F16), (512, 64, abi.ESP_F16)])
+@pytest.mark.parametrize("positions", ["consecutive", "pairs", "step_back"])
+def test_tiled_kernel_chunk_longer_than_the_window(HD, rows, dtype, positions):
+    """A chunk several windows long: most tiles' batch keys straddle the window's lower edge. Positions that rise by
+    one per row take the window as a bound in row numbers; positions that repeat (two rows per position) or step
+    back in the middle of the chunk take the per-key position test. The split target also cuts the cached range."""
+    from gpu_utils import run_case
+    window = 200
+    c = small_case(seed=47, H=6, Hkv=3, HD=HD, bt=32, dtype=dtype, seqs=((333, 700), (50, 290), (0, 450)), rows_per_tile=rows,
+                   window=window)
+    if positions != "consecutive":
+        for t in c.trees:
+            P, M, base = int(t["P"]), int(t["M"]), int(t["base"])
+            j = np.arange(M)
+            c.pos[base:base + M, 0:3] = (P + (j // 2 if positions == "pairs" else np.where(j < M // 2, j, j - 37)))[:, None]
+    _check(c, host.options_mi355x(rows, 64))
+    if HD != 512 and positions == "consecutive":   # the same chunk with its rows read from the pool
+        from test_gpu_rows_in_pool import pool_case
+        pc = pool_case(seed=48, H=6, Hkv=3, HD=HD, bt=32, dtype=dtype, seqs=((320, 700), (60, 450)), rows_per_tile=rows, window=window)
+        print(f"rows in pool: {pc.meta['seqs']}", flush=True)
+        got = run_case(pc, host.options_mi355x(rows, 64), rows_in_pool=True)
+        err = max_abs(got, oracle_direct(pc, threads=8), dtype)
+        assert err <= tol_for(dtype), f"rows in pool: max abs {err}"
+
+
 def test_tiled_kernel_split_tiles_and_combine():
     """A single long-context tile group is split over key ranges and merged."""
     c = small_case(seed=42, seqs=((3000, 100),), H=4, Hkv=2, rows_per_tile=128)
