@@ -50,6 +50,9 @@ def _draw(rng):
         seqs = [(max(P, 1), M) for P, M in seqs]
     split = int(rng.choice([0, 3, 8, 64, 700, 5000]))
     gate = bool(rng.integers(0, 4) == 0)
+    # drawn last, so that the shapes above are those of earlier versions of this sweep: on windowed layers, now and then,
+    # positions that do not rise by one per row (two rows per position, as siblings of a tree have)
+    kw["paired_positions"] = bool(window and kind in ("prefill", "smallchunk", "verify") and rng.integers(0, 3) == 0)
     return kind, tuple(seqs), R, split, gate, kw
 
 
@@ -62,7 +65,12 @@ def test_random_shapes_match_the_checker(chunk):
         kind, seqs, R, split, gate, kw = _draw(rng)
         print(f"it={it} kind={kind} seqs={seqs} R={R} split={split} gate={gate} "
               f"{ {k: v for k, v in kw.items() if k != 'desc_fn'} }", flush=True)
+        paired = kw.pop("paired_positions")
         c = small_case(seed=9000 + it, seqs=seqs, rows_per_tile=R, **kw)
+        if paired:
+            for t in c.trees:
+                P, M, base = int(t["P"]), int(t["M"]), int(t["base"])
+                c.pos[base:base + M, 0:3] = (P + np.arange(M) // 2)[:, None]
         p = c.params
         keep = None
         if gate:
