@@ -994,6 +994,7 @@ class Ceilings:
         self.lib.esp_ceiling_hbm_read.argtypes = [V, V, I, I, I, I, V, V, V, V]
         self.lib.esp_ceiling_mfma_issue.argtypes = [I, I, I, I, I, V, V, V, V]
         self.lib.esp_ceiling_prefill_step.argtypes = [I, I, I, I, I, V, V, V, V, V, V]
+        self.lib.esp_ceiling_prefill_step256.argtypes = [I, I, I, I, V, V, V, V, V, V]
 
     def _events(self, n):
         t = self.torch
@@ -1091,6 +1092,35 @@ class Ceilings:
         return out
 
 
+    SHAPES256 = ("4 wavefronts x 32 rows, one per SIMD (as built)", "8 wavefronts as 4 pairs, P through LDS",
+                 "8 wavefronts x 16 rows, v_mfma_f32_16x16x32")
+    LOADS256 = ("no staging loads", "64 KB per step staged behind the barrier", "one load behind each of the first 16 matrix instructions")
+
+    def prefill_step256(self, cases=((0, 0), (0, 1), (0, 2), (1, 0), (1, 1), (2, 0), (2, 1)), iters=1500):
+        """The 256-dim prefill step as bare instruction streams in three shapes of the workgroup, one workgroup per
+        compute unit: TFLOP/s, cycles per step (64 keys x 128 rows) and the clock, both read inside the kernel."""
+        t = self.torch
+        src = t.full(((8 << 20) + 65536,), 0x3c, dtype=t.uint8, device="cuda")
+        st = self.C.c_void_p(t.cuda.current_stream().cuda_stream)
+        out = []
+        for shape, loads in cases:
+            outbuf = t.zeros(N_CU * 512, dtype=t.float32, device="cuda")
+            clk = t.zeros(2 * N_CU, dtype=t.int64, device="cuda")
+            evs = self._events(4)
+            for a, b in evs:
+                rc = self.lib.esp_ceiling_prefill_step256(shape, loads, N_CU, iters, self.C.c_void_p(outbuf.data_ptr()), self.C.c_void_p(src.data_ptr()),
+                                                          self.C.c_void_p(clk.data_ptr()), st, self.C.c_void_p(a.cuda_event), self.C.c_void_p(b.cuda_event))
+                assert rc == 0, rc
+            t.cuda.synchronize()
+            ms = float(np.median([a.elapsed_time(b) for a, b in evs][1:]))
+            ck = clk.cpu().numpy().reshape(N_CU, 2).astype(np.float64)
+            out.append({"shape": self.SHAPES256[shape], "loads": self.LOADS256[loads],
+                        "TFLOPs": round(N_CU * iters * 256 * 32768 / ms / 1e9, 1),
+                        "cycles_per_step": round(float(ck[:, 0].mean()) / iters, 0),
+                        "clock_GHz": round(float((ck[:, 0] / (ck[:, 1] / 100e6)).mean()) / 1e9, 3)})
+        return out
+
+
 def run_all(args, torch):
     """The default run: the batched paged decode as the headline (its K timed steps are the line's steps), the
     chunked causal prefill as the other half of the metric, one record per benchmark configuration (each with its
@@ -1182,7 +1212,7 @@ def main():
     ap.add_argument("--warmup", type=int, default=20)
     ap.add_argument("--workload", default="all",
                     help="all (default): the batched decode as the headline, the chunked prefill, one record per benchmark "
-                         "configuration and the measured ceilings; or c2_equal_<tokens> (16 equal sequences), or one of: hbm_read_ceiling, mfma_issue_ceiling, prefill_step_ceiling, decode_step_fusion, prefill_step_fusion, " + ", ".join(WORKLOADS))
+                         "configuration and the measured ceilings; or c2_equal_<tokens> (16 equal sequences), or one of: hbm_read_ceiling, mfma_issue_ceiling, prefill_step_ceiling, prefill_step256_ceiling, decode_step_fusion, prefill_step_fusion, " + ", ".join(WORKLOADS))
     ap.add_argument("--workgroups", type=int, default=0, help="planner split target (0: ask esp_attn_plan_hint)")
     ap.add_argument("--tables", default="scattered", choices=["scattered", "contiguous"],
                     help="block tables: a seeded permutation of the pool (the benchmark's definition) or address order")
@@ -1221,6 +1251,10 @@ def main():
     if args.workload == "prefill_step_ceiling":
         print(json.dumps({"metric": "the prefill kernels' step as a bare instruction stream, TFLOP/s", "unit": "TFLOP/s",
                           "peak": MFMA_PEAK_TFLOPS, "stages": Ceilings().prefill_step()}), flush=True)
+        return
+    if args.workload == "prefill_step256_ceiling":
+        print(json.dumps({"metric": "the 256-dim prefill step as a bare instruction stream, three workgroup shapes, TFLOP/s", "unit": "TFLOP/s",
+                          "peak": MFMA_PEAK_TFLOPS, "streams": Ceilings().prefill_step256()}), flush=True)
         return
     w = make_workload(args.workload, args.workgroups or None, args.tables == "contiguous", args.page)
     K, W = args.steps, args.warmup

@@ -15,6 +15,7 @@ namespace {
 
 using u32x4 = uint32_t __attribute__((ext_vector_type(4)));
 using f32x16 = float __attribute__((ext_vector_type(16)));
+using f32x4 = float __attribute__((ext_vector_type(4)));
 using bf16x8 = __bf16 __attribute__((ext_vector_type(8)));
 
 // Every wavefront reads whole pages, 16 bytes per lane per load, DEPTH pages in flight; page p of the
@@ -214,6 +215,246 @@ __global__ __launch_bounds__(256, ROWS == 2 ? 1 : 2) void step_kernel(float* out
   out[blockIdx.x * 256 + threadIdx.x] = r;
 }
 
+// The head-dim-256 prefill step as bare instruction streams: per step a compute unit multiplies 64 keys with 128 query
+// rows of one 256-dim head (256 v_mfma_f32_32x32x16 or as many flops in 16x16x32), every A operand read from LDS,
+// 32 scores per row-lane of softmax work, one barrier, 64 KB staged from `src` into LDS. Three shapes of the workgroup:
+//   0  4 wavefronts x 32 rows, one per SIMD: the kernel as built (64 matrix instructions per wavefront and step)
+//   1  8 wavefronts as 4 pairs: a wavefront takes half of the step's keys through Q K^T and the softmax, hands its
+//      packed P to its partner through LDS and multiplies all 64 keys' P with its half of the dims
+//   2  8 wavefronts x 16 rows on v_mfma_f32_16x16x32: every wavefront a whole head, reading all of K and V^T
+// LOADS: 0 none, 1 all behind the barrier, 2 (shape 0) one behind each of the step's first 16 matrix instructions.
+__device__ __forceinline__ void stage_one(const char* base, uint32_t lane_off, uint32_t lds_addr) {
+  lds_addr = uint32_t(__builtin_amdgcn_readfirstlane(int(lds_addr)));
+  const uint64_t b64 = reinterpret_cast<uint64_t>(base);
+  const uint32_t b_lo = uint32_t(__builtin_amdgcn_readfirstlane(int(uint32_t(b64))));
+  const uint32_t b_hi = uint32_t(__builtin_amdgcn_readfirstlane(int(uint32_t(b64 >> 32))));
+  base = reinterpret_cast<const char*>(uint64_t(b_lo) | (uint64_t(b_hi) << 32));
+  asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, %2" : : "s"(lds_addr), "v"(lane_off), "s"(base) : "memory");
+}
+__device__ __forceinline__ uint32_t step256_rnd(uint32_t x) {
+  x = x * 2654435761u + 12345u;
+  x ^= x >> 15;
+  x *= 2246822519u;
+  x ^= x >> 13;
+  return (x & 0x807f807fu) | 0x3e803e80u | ((x >> 3) & 0x01000100u);
+}
+__device__ __forceinline__ const char* step256_src(const char* src, int it, int wave, int per_wave) {
+  return src + ((size_t(blockIdx.x) * 977 * 16 + size_t(it) * 65536) & ((size_t(8) << 20) - 1 - 131071)) + size_t(wave) * per_wave;
+}
+
+template <int LOADS>
+__global__ __launch_bounds__(256, 1) void step256_kernel(float* out, int iters, const char* src, unsigned long long* clk) {
+  const unsigned long long c0 = __builtin_readcyclecounter(), r0 = __builtin_amdgcn_s_memrealtime();
+  extern __shared__ __attribute__((aligned(16))) char lds[];  // 64 KB of operands, 64 KB of staging space
+  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+  const u32x4 b = {step256_rnd(threadIdx.x + 11), step256_rnd(threadIdx.x + 13), step256_rnd(threadIdx.x + 17), step256_rnd(threadIdx.x + 19)};
+  f32x16 c[8] = {};
+  float v[16];
+#pragma unroll
+  for (int i = 0; i < 16; ++i) v[i] = -float(threadIdx.x + i) * 1e-3f;
+  for (int i = threadIdx.x; i < 16384; i += 256) reinterpret_cast<uint32_t*>(lds)[i] = step256_rnd(i * 7 + blockIdx.x);
+  __syncthreads();
+  using lds_ptr = const __attribute__((address_space(3))) u32x4*;
+  const uint32_t lds0 = uint32_t(uintptr_t(lds)), base = lds0 + lane * 16;
+  auto mm = [](u32x4 x, u32x4 y, f32x16 z) { return __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(bf16x8, x), __builtin_bit_cast(bf16x8, y), z, 0, 0, 0); };
+  u32x4 ring[2][8];
+#pragma unroll
+  for (int j = 0; j < 8; ++j) ring[0][j] = *reinterpret_cast<lds_ptr>(base + j * 1024);
+  for (int it = 0; it < iters; ++it) {
+    const char* sp = step256_src(src, it, wave, 16384);
+    const uint32_t dst = lds0 + 65536 + wave * 16384;
+#pragma unroll
+    for (int g = 0; g < 8; ++g) {
+#pragma unroll
+      for (int j = 0; j < 8; ++j) ring[(g + 1) & 1][j] = *reinterpret_cast<lds_ptr>(base + ((g + 1) & 7) * 8192 + j * 1024);
+      __builtin_amdgcn_s_waitcnt(0xC07F | (8 << 8));
+#pragma unroll
+      for (int j = 0; j < 8; ++j) {
+        c[g] = mm(ring[g & 1][j], b, c[g]);
+        if (g >= 2 && g < 6) {  // the softmax's share: 32 scores per lane and step beside 32 of the matrix instructions
+          v[(2 * j) & 15] = __builtin_amdgcn_exp2f(v[(2 * j) & 15] - c[7][0]);
+          v[(2 * j + 5) & 15] += v[(2 * j + 7) & 15];
+          asm volatile("" : "+v"(v[(2 * j) & 15]));
+        }
+        if constexpr (LOADS == 2) {
+          if (g < 2) stage_one(sp + (8 * g + j) * 1024, lane * 16, dst + (8 * g + j) * 1024);
+        }
+        __builtin_amdgcn_sched_barrier(0);
+      }
+    }
+    if constexpr (LOADS != 0) asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+    __syncthreads();
+    if constexpr (LOADS == 1) {
+#pragma unroll
+      for (int q = 0; q < 16; ++q) stage_one(sp + q * 1024, lane * 16, dst + q * 1024);
+    }
+  }
+  asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+  if (threadIdx.x == 0 && clk) {
+    clk[2 * blockIdx.x] = __builtin_readcyclecounter() - c0;
+    clk[2 * blockIdx.x + 1] = __builtin_amdgcn_s_memrealtime() - r0;
+  }
+  float r = 0;
+#pragma unroll
+  for (int i = 0; i < 16; ++i) r += c[0][i] + c[1][i] + c[2][i] + c[3][i] + c[4][i] + c[5][i] + c[6][i] + c[7][i] + v[i];
+  out[blockIdx.x * 256 + threadIdx.x] = r;
+}
+
+template <int LOADS>
+__global__ __launch_bounds__(512, 1) void step256_pairs_kernel(float* out, int iters, const char* src, unsigned long long* clk) {
+  const unsigned long long c0 = __builtin_readcyclecounter(), r0 = __builtin_amdgcn_s_memrealtime();
+  extern __shared__ __attribute__((aligned(16))) char lds[];  // 64 KB of operands, 64 KB of staging space, 16 KB of exchange
+  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+  u32x4 q[16];
+#pragma unroll
+  for (int i = 0; i < 16; ++i) q[i] = u32x4{step256_rnd(threadIdx.x + 11 * i), step256_rnd(threadIdx.x + 13 * i), step256_rnd(threadIdx.x + 17), step256_rnd(threadIdx.x + 19)};
+  f32x16 acc[4] = {};
+  float l_run = 0.f;
+  const float m_run = 3.0f;
+  for (int i = threadIdx.x; i < 16384; i += 512) reinterpret_cast<uint32_t*>(lds)[i] = step256_rnd(i * 7 + blockIdx.x);
+  __syncthreads();
+  using lds_ptr = const __attribute__((address_space(3))) u32x4*;
+  const uint32_t lds0 = uint32_t(uintptr_t(lds)), base = lds0 + lane * 16;
+  u32x4* xch = reinterpret_cast<u32x4*>(lds + 131072);
+  auto mm = [](u32x4 x, u32x4 y, f32x16 z) { return __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(bf16x8, x), __builtin_bit_cast(bf16x8, y), z, 0, 0, 0); };
+  auto pk = [](float a, float b) { return (__builtin_bit_cast(uint32_t, a) >> 16) | (__builtin_bit_cast(uint32_t, b) & 0xffff0000u); };
+  u32x4 ring[2][8];
+  u32x4 pb[4] = {};
+  for (int it = 0; it < iters; ++it) {
+    const char* sp = step256_src(src, it, wave, 8192);
+    const uint32_t dst = lds0 + 65536 + wave * 8192;
+    // Q K^T of this wavefront's 32 keys and their softmax
+#pragma unroll
+    for (int j = 0; j < 8; ++j) ring[0][j] = *reinterpret_cast<lds_ptr>(base + (wave & 1) * 16384 + j * 1024);
+#pragma unroll
+    for (int j = 0; j < 8; ++j) ring[1][j] = *reinterpret_cast<lds_ptr>(base + (wave & 1) * 16384 + 8192 + j * 1024);
+    f32x16 s = {};
+    __builtin_amdgcn_s_waitcnt(0xC07F | (8 << 8));
+#pragma unroll
+    for (int j = 0; j < 8; ++j) s = mm(ring[0][j], q[j], s);
+    __builtin_amdgcn_s_waitcnt(0xC07F);
+#pragma unroll
+    for (int j = 0; j < 8; ++j) s = mm(ring[1][j], q[8 + j], s);
+    __builtin_amdgcn_sched_barrier(0);
+    float p[16], ps = 0.f;
+#pragma unroll
+    for (int e = 0; e < 16; ++e) p[e] = __builtin_amdgcn_exp2f(__builtin_fmaf(s[e], 0.088f, -m_run));
+    pb[0] = u32x4{pk(p[0], p[1]), pk(p[2], p[3]), pk(p[4], p[5]), pk(p[6], p[7])};
+    pb[1] = u32x4{pk(p[8], p[9]), pk(p[10], p[11]), pk(p[12], p[13]), pk(p[14], p[15])};
+#pragma unroll
+    for (int e = 0; e < 16; ++e) ps += p[e];
+    l_run += ps;
+    xch[(wave * 2 + 0) * 64 + lane] = pb[0];
+    xch[(wave * 2 + 1) * 64 + lane] = pb[1];
+    asm volatile("s_waitcnt vmcnt(0) lgkmcnt(0)" ::: "memory");
+    __syncthreads();
+    if constexpr (LOADS != 0) {
+#pragma unroll
+      for (int qd = 0; qd < 8; ++qd) stage_one(sp + qd * 1024, lane * 16, dst + qd * 1024);
+    }
+    // P V: all 64 keys' P with this wavefront's 128 dims
+#pragma unroll
+    for (int j = 0; j < 8; ++j) ring[0][j] = *reinterpret_cast<lds_ptr>(base + 32768 + j * 1024);
+    pb[2] = xch[((wave ^ 1) * 2 + 0) * 64 + lane];
+    pb[3] = xch[((wave ^ 1) * 2 + 1) * 64 + lane];
+#pragma unroll
+    for (int j = 0; j < 8; ++j) ring[1][j] = *reinterpret_cast<lds_ptr>(base + 32768 + 8192 + j * 1024);
+    __builtin_amdgcn_s_waitcnt(0xC07F | (8 << 8));
+#pragma unroll
+    for (int j = 0; j < 8; ++j) acc[j & 3] = mm(ring[0][j], pb[j >> 2], acc[j & 3]);
+    __builtin_amdgcn_s_waitcnt(0xC07F);
+#pragma unroll
+    for (int j = 0; j < 8; ++j) acc[j & 3] = mm(ring[1][j], pb[2 + (j >> 2)], acc[j & 3]);
+    __builtin_amdgcn_sched_barrier(0);
+  }
+  asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+  if (threadIdx.x == 0 && clk) {
+    clk[2 * blockIdx.x] = __builtin_readcyclecounter() - c0;
+    clk[2 * blockIdx.x + 1] = __builtin_amdgcn_s_memrealtime() - r0;
+  }
+  float r = l_run;
+#pragma unroll
+  for (int i = 0; i < 16; ++i) r += acc[0][i] + acc[1][i] + acc[2][i] + acc[3][i];
+  out[blockIdx.x * 512 + threadIdx.x] = r;
+}
+
+template <int LOADS>
+__global__ __launch_bounds__(512, 1) void step256_rows16_kernel(float* out, int iters, const char* src, unsigned long long* clk) {
+  const unsigned long long c0 = __builtin_readcyclecounter(), r0 = __builtin_amdgcn_s_memrealtime();
+  extern __shared__ __attribute__((aligned(16))) char lds[];  // 64 KB of operands, 64 KB of staging space
+  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+  u32x4 q[8];
+#pragma unroll
+  for (int i = 0; i < 8; ++i) q[i] = u32x4{step256_rnd(threadIdx.x + 11 * i), step256_rnd(threadIdx.x + 13 * i), step256_rnd(threadIdx.x + 17), step256_rnd(threadIdx.x + 19)};
+  f32x4 acc[16] = {};
+  float l_run = 0.f;
+  const float m_run = 3.0f;
+  for (int i = threadIdx.x; i < 16384; i += 512) reinterpret_cast<uint32_t*>(lds)[i] = step256_rnd(i * 7 + blockIdx.x);
+  __syncthreads();
+  using lds_ptr = const __attribute__((address_space(3))) u32x4*;
+  const uint32_t lds0 = uint32_t(uintptr_t(lds)), base = lds0 + lane * 16;
+  auto mm = [](u32x4 x, u32x4 y, f32x4 z) { return __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(bf16x8, x), __builtin_bit_cast(bf16x8, y), z, 0, 0, 0); };
+  auto pk = [](float a, float b) { return (__builtin_bit_cast(uint32_t, a) >> 16) | (__builtin_bit_cast(uint32_t, b) & 0xffff0000u); };
+  u32x4 ring[2][8];
+  u32x4 pb[2] = {};
+  for (int it = 0; it < iters; ++it) {
+    const char* sp = step256_src(src, it, wave, 8192);
+    const uint32_t dst = lds0 + 65536 + wave * 8192;
+    f32x4 s[4];
+#pragma unroll
+    for (int j = 0; j < 8; ++j) ring[0][j] = *reinterpret_cast<lds_ptr>(base + j * 1024);
+#pragma unroll
+    for (int t = 0; t < 4; ++t) {  // Q K^T: 4 tiles of 16 keys, 8 slices of 32 dims each
+#pragma unroll
+      for (int j = 0; j < 8; ++j) ring[(t + 1) & 1][j] = *reinterpret_cast<lds_ptr>(base + (t + 1) * 8192 + j * 1024);
+      __builtin_amdgcn_s_waitcnt(0xC07F | (8 << 8));
+      s[t] = f32x4{0, 0, 0, 0};
+#pragma unroll
+      for (int j = 0; j < 8; ++j) s[t] = mm(ring[t & 1][j], q[j], s[t]);
+      __builtin_amdgcn_sched_barrier(0);
+    }
+    float p[16], ps = 0.f;
+#pragma unroll
+    for (int t = 0; t < 4; ++t)
+#pragma unroll
+      for (int e = 0; e < 4; ++e) p[4 * t + e] = __builtin_amdgcn_exp2f(__builtin_fmaf(s[t][e], 0.088f, -m_run));
+    pb[0] = u32x4{pk(p[0], p[1]), pk(p[2], p[3]), pk(p[4], p[5]), pk(p[6], p[7])};
+    pb[1] = u32x4{pk(p[8], p[9]), pk(p[10], p[11]), pk(p[12], p[13]), pk(p[14], p[15])};
+#pragma unroll
+    for (int e = 0; e < 16; ++e) ps += p[e];
+    l_run += ps;
+    __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+    for (int g = 0; g < 4; ++g) {  // P V: 16 tiles of 16 dims x 2 halves of the step's keys
+      if (g < 3) {
+#pragma unroll
+        for (int j = 0; j < 8; ++j) ring[(g + 1) & 1][j] = *reinterpret_cast<lds_ptr>(base + 32768 + (g + 1) * 8192 + j * 1024);
+        __builtin_amdgcn_s_waitcnt(0xC07F | (8 << 8));
+      } else {
+        __builtin_amdgcn_s_waitcnt(0xC07F);
+      }
+#pragma unroll
+      for (int j = 0; j < 8; ++j) acc[4 * g + (j >> 1)] = mm(ring[g & 1][j], pb[j & 1], acc[4 * g + (j >> 1)]);
+      __builtin_amdgcn_sched_barrier(0);
+    }
+    asm volatile("s_waitcnt vmcnt(0) lgkmcnt(0)" ::: "memory");
+    __syncthreads();
+    if constexpr (LOADS != 0) {
+#pragma unroll
+      for (int qd = 0; qd < 8; ++qd) stage_one(sp + qd * 1024, lane * 16, dst + qd * 1024);
+    }
+  }
+  asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+  if (threadIdx.x == 0 && clk) {
+    clk[2 * blockIdx.x] = __builtin_readcyclecounter() - c0;
+    clk[2 * blockIdx.x + 1] = __builtin_amdgcn_s_memrealtime() - r0;
+  }
+  float r = l_run;
+#pragma unroll
+  for (int i = 0; i < 16; ++i) r += acc[i][0] + acc[i][1] + acc[i][2] + acc[i][3];
+  out[blockIdx.x * 512 + threadIdx.x] = r;
+}
+
 template <typename K, typename... Args>
 hipError_t launch_lds(K k, size_t lds_bytes, dim3 grid, dim3 block, hipStream_t st, hipEvent_t e0, hipEvent_t e1, Args... args) {
   hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(k), hipFuncAttributeMaxDynamicSharedMemorySize, int(lds_bytes));
@@ -288,6 +529,27 @@ int esp_ceiling_prefill_step(int32_t stage, int32_t rows, int32_t random_data, i
     case 12: e = launch_lds(step_kernel<1, 2>, 65536, g, b, st, e0, e1, out, iters, 1u, random_data, s, clk); break;
     case 32: e = launch_lds(step_kernel<3, 2>, 65536, g, b, st, e0, e1, out, iters, 1u, random_data, s, clk); break;
     case 42: e = launch_lds(step_kernel<4, 2>, 65536, g, b, st, e0, e1, out, iters, 1u, random_data, s, clk); break;
+    default: return 2;
+  }
+  return e == hipSuccess ? 0 : 3;
+}
+
+int esp_ceiling_prefill_step256(int32_t shape, int32_t loads, int32_t workgroups, int32_t iters, float* out, const void* src, unsigned long long* clk,
+                                void* stream, void* start_event, void* stop_event) {
+  if (!out || workgroups <= 0 || iters <= 0 || (loads != 0 && !src)) return 1;
+  const auto st = static_cast<hipStream_t>(stream);
+  const auto e0 = static_cast<hipEvent_t>(start_event), e1 = static_cast<hipEvent_t>(stop_event);
+  const dim3 g(workgroups);
+  const char* s = static_cast<const char*>(src);
+  hipError_t e;
+  switch (shape * 10 + loads) {
+    case 0: e = launch_lds(step256_kernel<0>, 131072, g, dim3(256), st, e0, e1, out, iters, s, clk); break;
+    case 1: e = launch_lds(step256_kernel<1>, 131072, g, dim3(256), st, e0, e1, out, iters, s, clk); break;
+    case 2: e = launch_lds(step256_kernel<2>, 131072, g, dim3(256), st, e0, e1, out, iters, s, clk); break;
+    case 10: e = launch_lds(step256_pairs_kernel<0>, 147456, g, dim3(512), st, e0, e1, out, iters, s, clk); break;
+    case 11: e = launch_lds(step256_pairs_kernel<1>, 147456, g, dim3(512), st, e0, e1, out, iters, s, clk); break;
+    case 20: e = launch_lds(step256_rows16_kernel<0>, 131072, g, dim3(512), st, e0, e1, out, iters, s, clk); break;
+    case 21: e = launch_lds(step256_rows16_kernel<1>, 131072, g, dim3(512), st, e0, e1, out, iters, s, clk); break;
     default: return 2;
   }
   return e == hipSuccess ? 0 : 3;

@@ -51,6 +51,18 @@ int esp_ceiling_mfma_issue(int32_t valu_per_mfma, int32_t exp_per_mfma, int32_t 
 int esp_ceiling_prefill_step(int32_t stage, int32_t rows, int32_t random_data, int32_t workgroups, int32_t iters, float* out, const void* src,
                              unsigned long long* clk, void* stream, void* start_event, void* stop_event);
 
+/* The key step of the 256-dim prefill kernel as bare instruction streams, in three shapes of the workgroup. Per step a
+ * compute unit multiplies 64 keys with 128 query rows of one head (the flops of 256 v_mfma_f32_32x32x16), every A operand
+ * read from LDS, with 32 scores per row of softmax arithmetic and one barrier. shape: 0 = 4 wavefronts x 32 rows, one per
+ * SIMD (the kernel as built); 1 = 8 wavefronts as 4 pairs, each wavefront taking half of the step's keys through Q K^T and
+ * the softmax, handing its packed P to its partner through LDS and multiplying all 64 keys' P with its half of the dims;
+ * 2 = 8 wavefronts x 16 rows on v_mfma_f32_16x16x32, each a whole head. loads: 0 = none, 1 = the step's 64 KB staged from
+ * `src` (a device buffer of at least 8 MB + 64 KB, cache resident) straight into LDS behind the barrier, 2 (shape 0 only) =
+ * one load behind each of the step's first 16 matrix instructions. One workgroup per compute unit. clk as above.
+ * out: workgroups * 512 floats. Flops of a launch: workgroups * iters * 256 * 32768. */
+int esp_ceiling_prefill_step256(int32_t shape, int32_t loads, int32_t workgroups, int32_t iters, float* out, const void* src, unsigned long long* clk,
+                                void* stream, void* start_event, void* stop_event);
+
 #ifdef __cplusplus
 }
 #endif

@@ -35,7 +35,7 @@ def test_engine_library_exports_every_declared_symbol():
 
 def test_ceilings_library_exports_every_declared_symbol_and_refuses_bad_arguments():
     names = _declared("espetero_ceilings.h")
-    assert names == ["esp_ceiling_hbm_read", "esp_ceiling_mfma_issue", "esp_ceiling_prefill_step"]
+    assert names == ["esp_ceiling_hbm_read", "esp_ceiling_mfma_issue", "esp_ceiling_prefill_step", "esp_ceiling_prefill_step256"]
     lib = C.CDLL(os.path.join(ROOT, "espetero_amd", "csrc", "libespetero_ceilings.so"))
     for n in names:
         assert hasattr(lib, n), n
@@ -46,6 +46,8 @@ def test_ceilings_library_exports_every_declared_symbol_and_refuses_bad_argument
     assert lib.esp_ceiling_hbm_read(None, None, 4, 8192, 1, 8, None, None, None, None) == 1        # no buffer: refused on the host
     assert lib.esp_ceiling_mfma_issue(0, 0, 1, 8, 10, None, None, None, None) == 1
     assert lib.esp_ceiling_prefill_step(4, 1, 1, 8, 10, None, None, None, None, None, None) == 1
+    lib.esp_ceiling_prefill_step256.argtypes = [I, I, I, I, V, V, V, V, V, V]
+    assert lib.esp_ceiling_prefill_step256(0, 1, 8, 10, None, None, None, None, None, None) == 1
 
 
 def test_record_layouts_match_the_reference_structs():
