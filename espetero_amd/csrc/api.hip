@@ -378,7 +378,9 @@ int esp_attn_validate(const esp_attn_params* p, const esp_tile* tiles, int32_t n
                       jobs[j].r0, jobs[j].rows, t.r0);
       }
     }
-    if (t.last != 0 && t.last != 1) return fail(err, errlen, ESP_EINVAL, "tile %d: last %d (0 or 1)", i, t.last);
+    if (t.last < 0 || (t.last >= 2 && (t.last - 2 < t.b0 || t.last - 2 >= tr.M)))
+      return fail(err, errlen, ESP_EINVAL, "tile %d: last %d (0: no batch keys, 1: from b0 on, e + 2: rows b0 = %d .. e of the tree's %d)", i, t.last,
+                  t.b0, tr.M);
     if (t.b0 < 0 || t.b0 > tr.M) return fail(err, errlen, ESP_EINVAL, "tile %d: first batch key %d of %d rows", i, t.b0, tr.M);
     if (t.pad != 0 && t.pad - 1 != tr.table) return fail(err, errlen, ESP_EINVAL, "tile %d: pad %d is neither 0 nor 1 + its tree's table %d", i, t.pad, tr.table);
   }

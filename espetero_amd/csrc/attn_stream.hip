@@ -582,6 +582,7 @@ __global__ __launch_bounds__(HD >= 512 ? 128 * NC : 256, OCC) void attn_stream_k
       for (int o = 32; o >= 1; o >>= 1) kl = max(kl, __shfl_xor(kl, o));
       // fused: the batch keys are the tile's own rows in LDS, never more than the tile holds
       k_last = __builtin_amdgcn_readfirstlane(min(kl, (FUSED ? min(tree.M, rows_live) : tree.M) - 1));
+      if (tile.last >= 2) k_last = min(k_last, tile.last - 2);  // a part whose batch range ends at row last - 2 of the tree
       bp0 = tile.b0 >> USH;
       n_batch = max(0, ((k_last + UK) >> USH) - bp0);
     }

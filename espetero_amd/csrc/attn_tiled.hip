@@ -134,7 +134,8 @@ __global__ __launch_bounds__(256, OCC) void attn_tiled_kernel(const KArgs a, int
       qpos_max = max(qpos_max, red[w][3]);
     }
     // The same in every lane; saying so keeps everything derived from them in scalar registers.
-    k_last = __builtin_amdgcn_readfirstlane(min(k_last, tree.M - 1));
+    // a part whose batch range is cut ends at row last - 2 of the tree (last = 1: open, up to what its rows see)
+    k_last = __builtin_amdgcn_readfirstlane(min(min(k_last, tree.M - 1), tile.last >= 2 ? tile.last - 2 : INT32_MAX));
     seg_max = __builtin_amdgcn_readfirstlane(seg_max);
     anc_max = __builtin_amdgcn_readfirstlane(anc_max);
     qpos_max = __builtin_amdgcn_readfirstlane(qpos_max);
@@ -695,7 +696,7 @@ __global__ __launch_bounds__(256, OCC) void attn_tiled_kernel(const KArgs a, int
     if (n_b > 0 && !batch_window && !anc_any && seg_max != INT32_MAX) {
       const int lo_b = max(max(max(tile.b0, seg_max), bw_lo), 0);
       const int g_lo = (tree.base + lo_b + 15) >> 4;           // first group of 16 rows wholly at or above lo_b
-      const int g_hi = ((tree.base + rr0) >> 4) - 1;           // last group wholly below the tile's first row
+      const int g_hi = min(((tree.base + rr0) >> 4), ((tree.base + k_last + 1) >> 4)) - 1;  // last group wholly below the tile's first row (and inside the part's batch range)
       const int s_lo = n_c + g_lo - a0, s_hi = n_c + g_hi - a0;  // as sub-blocks of the range
       b_lo = (s_lo + 3) >> 2;
       b_hi = max(b_lo, (s_hi + 1) >> 2);

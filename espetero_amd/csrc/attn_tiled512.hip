@@ -94,7 +94,7 @@ __global__ __launch_bounds__(256, 1) void attn_tiled512_kernel(const KArgs a, in
     if (lane == 0) red[wave][0] = kl;
     __syncthreads();
     k_last = max(max(red[0][0], red[1][0]), max(red[2][0], red[3][0]));
-    k_last = __builtin_amdgcn_readfirstlane(min(k_last, tree.M - 1));
+    k_last = __builtin_amdgcn_readfirstlane(min(min(k_last, tree.M - 1), tile.last >= 2 ? tile.last - 2 : INT32_MAX));  // last >= 2: the part's batch range ends at row last - 2
   }
 
   // ---- the key range as 16-key sub-blocks: cached [k0, k1), then batch rows [b0, k_last]

@@ -31,6 +31,7 @@ PlanOptions to_cpp(const esp_plan_options& o) {
   p.balanced = o.balanced != 0;
   p.item_steps = o.item_steps;
   p.part_steps = o.part_steps;
+  p.cut_batch = o.cut_batch != 0;
   return p;
 }
 void to_c(const PlanOptions& p, esp_plan_options* o) {
@@ -44,6 +45,7 @@ void to_c(const PlanOptions& p, esp_plan_options* o) {
   o->balanced = p.balanced ? 1 : 0;
   o->item_steps = p.item_steps;
   o->part_steps = p.part_steps;
+  o->cut_batch = p.cut_batch ? 1 : 0;
 }
 template <class F>
 int guarded(F&& f) {

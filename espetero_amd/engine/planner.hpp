@@ -13,8 +13,11 @@
 //     (the reference rule gives a 512-token and an 8192-token sequence the same
 //     number of splits, which leaves most of 256 CUs idle while the longest
 //     sequence finishes). Boundaries stay on page multiples.
-// Only the algebra is contractual: the ranges of a tile group partition
-// [k0, P), the last range owns the batch keys, parts merge in range order.
+// Only the algebra is contractual: the cached ranges of a tile group partition
+// [k0, P), its batch ranges partition the batch keys from b0 on (one range - the
+// last part's - unless the balanced rule cuts the batch keys too: `last` = e + 2
+// ends a part's batch keys at row e of the tree, `last` = 1 leaves them open),
+// parts merge in range order.
 #pragma once
 
 #include <algorithm>
@@ -43,6 +46,9 @@ struct PlanOptions {
   // epilogue), in steps of `granule` keys.
   int item_steps = 0;
   int part_steps = 0;  // what a split part costs on top: its partial record written, read again and merged
+  // Tiled kernel, balanced rule: a tile's batch keys are cut like its cached keys (a pass of fewer workgroups than
+  // slots - one prompt's first chunk - is otherwise as long as its last tile, which scans every row of the chunk).
+  bool cut_batch = false;
 
   static PlanOptions reference() { return PlanOptions{}; }
   // rows: query rows per tile (decode 1..8 -> 8-row budget is irrelevant; prefill 64/128).
@@ -62,6 +68,7 @@ struct PlanOptions {
       o.min_span = 1024;
       o.item_steps = 6;
       o.part_steps = 8;
+      o.cut_batch = true;
     }
     return o;
   }
@@ -110,8 +117,9 @@ inline void plan_tiles(AttnPlan& A, int groups, int window, const int32_t* pos, 
   const int n_tiles = int(rts.size());
   int budget = std::max(1, o.groups_target / std::max(1, groups * n_tiles));
   int chunk_all = 0;  // balanced rule: keys per workgroup
+  auto cuttable = [&](const RowTile& rt) { return rt.span + (o.cut_batch ? rt.batch : 0) >= o.min_span; };
   auto parts_of = [&](const RowTile& rt, long long chunk) {
-    return rt.span >= o.min_span ? std::min<long long>((rt.span + rt.batch + chunk - 1) / chunk, o.max_splits) : 1;
+    return cuttable(rt) ? std::min<long long>((rt.span + rt.batch + chunk - 1) / chunk, o.max_splits) : 1;
   };
   std::vector<int> ns_of;  // tiled kernel: parts of every row tile, once chosen
   if (o.balanced && o.item_steps > 0) {
@@ -151,11 +159,11 @@ inline void plan_tiles(AttnPlan& A, int groups, int window, const int32_t* pos, 
     ns_of = cand;
     long long best = finish_time(cand);
     const long long items = 1LL * n_tiles * groups, rounds = items / slots;
-    // Fewer workgroups than slots: one chunk for every tile, the chunks that cut the longest tile into 2 .. 8
+    // No more workgroups than slots: one chunk for every tile, the chunks that cut the longest tile into 2 .. 8
     // parts (fewer parts first: ties keep them). With a round or more of whole workgroups such a split was
     // measured slower than none (two workgroups share a compute unit and the older one is served first, so the
     // slots are less alike than this hand-out takes them to be).
-    for (int parts = 2; parts <= 8 && rounds == 0; ++parts) {
+    for (int parts = 2; parts <= 8 && items <= slots; ++parts) {
       const long long c = std::max(c_lo, (c_hi + parts - 1) / parts) * o.granule;
       for (int i = 0; i < n_tiles; ++i) cand[size_t(i)] = int(parts_of(rts[size_t(i)], c));
       const long long t = finish_time(cand);
@@ -236,7 +244,46 @@ inline void plan_tiles(AttnPlan& A, int groups, int window, const int32_t* pos, 
     const int step = (per + o.granule - 1) / o.granule * o.granule;
     const int part0 = A.parts;
     int used = 0;
-    if (o.balanced) {
+    if (o.balanced && o.cut_batch && span < (ns - 1) * step) {
+      // Some cut falls among the batch keys: walk cached keys [k0, P) and then batch rows [b0, b0 + batch) in parts of
+      // `step`, cached cuts on page multiples, batch cuts on multiples of the granule in the tree's rows. A part that
+      // ends among the batch rows says where (`last` = its last row + 2); the last part's batch range stays open, so
+      // rows that see beyond their own tile (ancestors, image spans) find those keys there.
+      const int b_end = rt.b0 + rt.batch;  // one past the tile's last row
+      int k = rt.k0, b = rt.b0;
+      for (int p = 0; p < ns && (k < t.P || b < b_end); ++p) {
+        const bool is_last = p + 1 == ns;
+        int k1 = t.P, b1 = b_end;
+        if (!is_last) {
+          int room = step;
+          if (k < t.P) {
+            k1 = std::min(t.P, k + room);
+            if (k1 < t.P) k1 = std::min(t.P, std::max(k + o.granule, k1 / o.granule * o.granule));
+            room -= k1 - k;
+          }
+          if (k1 < t.P) {
+            b1 = b;  // all of it cached keys
+          } else {
+            b1 = std::min(b_end, b + std::max(room, 0));
+            if (b1 < b_end) b1 = std::min(b_end, std::max(b + (k1 > k ? 0 : o.granule), b1 / o.granule * o.granule));
+            if (b1 < b) b1 = b;
+          }
+        }
+        if (k1 == k && b1 == b) continue;
+        const bool rest = b1 >= b_end;  // nothing left for a later part: this one is the group's last
+        const int last = b1 > b ? (rest ? 1 : b1 + 1) : (rest && k1 >= t.P ? 1 : 0);
+        A.tiles.push_back({rt.tree, t.base + rt.r, k, k1, A.parts++, last, b, pad});
+        k = k1;
+        b = b1;
+        ++used;
+        if (rest && k >= t.P) break;
+      }
+      if (used == 1) {  // nothing was cut after all
+        A.tiles.back().part = -1;
+        --A.parts;
+        continue;
+      }
+    } else if (o.balanced) {
       // ns parts: all but the last are `step` cached keys on page multiples; the last keeps the
       // rest of the cached range (possibly nothing) and the batch keys.
       int k = rt.k0;

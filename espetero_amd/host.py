@@ -11,7 +11,8 @@ from . import abi
 class PlanOptions(C.Structure):
     _fields_ = [("rows_per_tile", C.c_int32), ("groups_target", C.c_int32), ("split", C.c_int32),
                 ("min_chunk", C.c_int32), ("granule", C.c_int32), ("max_splits", C.c_int32),
-                ("min_span", C.c_int32), ("balanced", C.c_int32), ("item_steps", C.c_int32), ("part_steps", C.c_int32)]
+                ("min_span", C.c_int32), ("balanced", C.c_int32), ("item_steps", C.c_int32), ("part_steps", C.c_int32),
+                ("cut_batch", C.c_int32)]
 
 
 class TreeSpec(C.Structure):

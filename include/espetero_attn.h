@@ -69,8 +69,11 @@ typedef struct esp_tile {
   int32_t k0;   /* cached-key range [k0, k1) */
   int32_t k1;
   int32_t part; /* -1: write O; else index of the partial record this tile writes */
-  int32_t last; /* also scan the tree's batch keys (this pass's own rows) */
-  int32_t b0;   /* first batch key (relative row) any row of the tile may see */
+  int32_t last; /* 0: cached keys only; 1 (the reference's value): also the tree's batch keys (this pass's own rows) from b0 on;
+                   e + 2: also the batch keys b0 .. e and no further (no counterpart in the reference, whose planner never cuts
+                   the batch keys: this library's balanced rule does when a pass has fewer workgroups than the chip has room
+                   for; the parts of such a group partition the batch keys as they partition the cached ones) */
+  int32_t b0;   /* first batch key (relative row) any row of the tile may see; of a part with a cut batch range, its first */
   int32_t pad;  /* 0 (the reference's value), or 1 + the tree's `table`: lets a kernel skip the tree lookup */
 } esp_tile;
 

@@ -262,6 +262,8 @@ int esp_oracle_attn_tiles(const esp_attn_params* p, const uint16_t* Q, const uin
       if (p->bidi && w - 1 > k_last) k_last = w - 1;
     }
     if (anc_max - 1 > k_last) k_last = anc_max - 1; /* noncausal roots, 40_:220 */
+    /* a part whose batch range is cut (this library's balanced planner; the reference never does): rows b0 .. last - 2 */
+    if (tile->last >= 2 && tile->last - 2 < k_last) k_last = tile->last - 2;
     const int n_slot_blocks = (tile->k1 - tile->k0 + OBK - 1) / OBK;
     const int bb0 = tile->last ? tile->b0 / OBK : 0;
     int n_batch_blocks = tile->last ? (k_last + OBK) / OBK - bb0 : 0;
@@ -289,7 +291,7 @@ int esp_oracle_attn_tiles(const esp_attn_params* p, const uint16_t* Q, const uin
             float mx = -INFINITY;
             for (int kc = 0; kc < OBK; ++kc) {
               const int j = j0 + kc;
-              int vis = j < j_end;
+              int vis = j < j_end && (in_slot || j >= tile->b0); /* below b0 no row of the tile sees anything */
               if (vis) vis = in_slot ? cached_visible(p, pos, row, j) : batch_visible(p, d, pos, t, rr, j);
               sv[kc] = -INFINITY;
               vrow[kc] = NULL;

@@ -268,6 +268,39 @@ def test_tiled_kernel_chunk_longer_than_the_window(HD, rows, dtype, positions):
         assert err <= tol_for(dtype), f"rows in pool: max abs {err}"
 
 
+@pytest.mark.parametrize("kw", [
+    dict(seqs=((0, 1500),), H=4, Hkv=2, dtype=abi.ESP_BF16),                        # a first chunk: batch keys only, ragged end
+    dict(seqs=((130, 1100), (0, 700)), H=4, Hkv=2, HD=256),                         # a part that ends the cached keys and begins the batch keys
+    dict(seqs=((0, 1400),), H=4, Hkv=2, HD=256, window=300, dtype=abi.ESP_BF16),    # cuts on both sides of the window's lower edge
+    dict(seqs=((40, 1300),), H=2, Hkv=2, bt=64, bidi=1, desc_fn=lambda M: synth.image_desc(M, 500, 900)),   # rows that see beyond their own tile
+    dict(seqs=((0, 1200),), H=2, Hkv=1, HD=512, rows_per_tile=64),                  # head dim 512
+    dict(seqs=((16, 1400),), H=4, Hkv=2, rows_in_pool=True),                        # the rows read from the pool
+])
+def test_tiled_kernel_cuts_the_batch_keys_of_a_tile(kw):
+    """The balanced rule cuts a tile's batch keys like its cached keys when a pass has few workgroups (a part whose batch
+    range ends early carries last = its last row + 2). Forced here by a cost model without fixed costs; held to the
+    checker, and to the uncut plan within the merge's own rounding."""
+    from gpu_utils import plan, run_case
+    in_pool = kw.pop("rows_in_pool", False)
+    R = kw.pop("rows_per_tile", 128)
+    if in_pool:
+        from test_gpu_rows_in_pool import pool_case
+        c = pool_case(49, rows_per_tile=R, **kw)
+    else:
+        c = small_case(seed=49, rows_per_tile=R, **kw)
+    o = host.options_mi355x(R, 256)
+    o.item_steps, o.part_steps, o.min_chunk, o.min_span = 1, 0, 128, 256
+    tiles, _, n_parts = plan(c, o)
+    cut = [x for x in tiles if int(x["last"]) >= 2]
+    assert cut and n_parts > 0, "the plan has no part with a cut batch range"
+    print(f"case seqs={c.meta['seqs']} R={R}: {len(tiles)} records, {len(cut)} with a cut batch range", flush=True)
+    got = run_case(c, o, rows_in_pool=in_pool)
+    err = max_abs(got, oracle_direct(c, threads=8), c.params.dtype)
+    assert err <= tol_for(c.params.dtype), f"max abs {err}"
+    whole = run_case(c, None, rows_in_pool=in_pool)
+    assert np.abs(f32(got, c.params.dtype) - f32(whole, c.params.dtype)).max() <= 2e-3
+
+
 def test_tiled_kernel_split_tiles_and_combine():
     """A single long-context tile group is split over key ranges and merged."""
     c = small_case(seed=42, seqs=((3000, 100),), H=4, Hkv=2, rows_per_tile=128)

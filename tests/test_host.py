@@ -129,8 +129,9 @@ def test_split_algebra_holds_for_both_rules(seed):
 @pytest.mark.parametrize("seed", range(8))
 def test_tiled_kernel_plans_partition_every_tile(seed):
     """The balanced rule for 128-row tiles (chosen by simulating the hand-out of workgroups to slots): whatever it
-    picks - no split, one chunk for all tiles, or only the shortest tiles cut - the ranges of a tile partition
-    [0, P), the last part owns the batch keys, parts are numbered in record order and every merge job names them."""
+    picks - no split, one chunk for all tiles, or only the shortest tiles cut - the cached ranges of a tile partition
+    [0, P), its batch ranges partition the batch rows (one open range in the last part, or cut ranges in front of it),
+    parts are numbered in record order and every merge job names them."""
     rng = np.random.default_rng(900 + seed)
     n = int(rng.integers(1, 5))
     trees, base = [], 0
@@ -145,19 +146,26 @@ def test_tiled_kernel_plans_partition_every_tile(seed):
     for x in tiles:
         by.setdefault((int(x["tree"]), int(x["r0"])), []).append(x)
     assert set(by) == {(ti, b + r) for ti, (b, P, _, m) in enumerate(trees) for r in range(0, m, 128)}
-    numbered = []
+    numbered, cut = [], 0
     for (ti, r0), xs in by.items():
-        P = trees[ti][1]
-        k = 0
+        base, P, _, m = trees[ti]
+        k, b = 0, 0      # cached keys and batch rows handed out so far
         for i, x in enumerate(xs):
-            assert int(x["k0"]) == k and (int(x["k1"]) > k or P == k)
+            last = int(x["last"])
+            assert int(x["k0"]) == k and int(x["k1"]) >= k
             assert int(x["k0"]) % o.granule == 0
             k = int(x["k1"])
-            assert int(x["last"]) == (1 if i == len(xs) - 1 else 0)
+            if last:                                   # the part takes batch rows from where the one before it stopped
+                assert k == P and int(x["b0"]) == b
+                if last >= 2:                          # ... up to row last - 2, on a granule boundary, and a later part goes on
+                    assert i < len(xs) - 1 and last - 2 >= b and (last - 1) % o.granule == 0
+                    b, cut = last - 1, cut + 1
+            assert (last == 1) == (i == len(xs) - 1)   # the group's last part leaves its batch range open
+            assert int(x["k1"]) > int(x["k0"]) or last  # no empty part
             assert (int(x["part"]) == -1) == (len(xs) == 1)
             if len(xs) > 1:
                 numbered.append(int(x["part"]))
-        assert k == P
+        assert k == P and b < min(m, r0 - base + 128)  # the open part begins inside the tile's own batch rows
     assert numbered == list(range(parts))          # in record order, which is the order the kernel's grid reverses
     assert sum(int(j["nparts"]) for j in jobs) == parts and all(int(j["nparts"]) >= 2 for j in jobs)
 

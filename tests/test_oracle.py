@@ -13,7 +13,7 @@ import numpy as np
 import pytest
 import torch
 
-from espetero_amd import abi, synth
+from espetero_amd import abi, host, synth
 from oracle import binding as ob
 from oracle import host_oracle as ho
 
@@ -224,6 +224,24 @@ def test_tiles_and_combine_match_direct(split, groups):
         assert parts == 0
     else:
         assert parts > 0
+    got = ob.attn_tiles(c.params, c.Q, c.Kb, c.Vb, c.pool_ref, c.blocks, c.desc, c.pos, tiles, c.trees, jobs, parts)
+    assert max_abs(got, oracle_direct(c), c.params.dtype) <= 1e-3
+
+
+@pytest.mark.parametrize("kw", [
+    dict(seqs=((0, 300),)),                                                            # batch keys only
+    dict(seqs=((70, 200), (0, 150))),                                                  # a part that ends the cached keys and begins the batch keys
+    dict(seqs=((0, 260),), window=60),                                                 # cuts around the window's lower edge
+    dict(seqs=((20, 220),), bidi=1, desc_fn=lambda M: synth.image_desc(M, 90, 170)),   # rows that see beyond their own tile
+])
+def test_cut_batch_ranges_match_direct(kw):
+    """The balanced planner's cut of a tile's batch keys (parts with last = their last row + 2, then one open part):
+    the partial records of such parts, merged, equal the row-by-row call."""
+    c = small_case(seed=24, H=4, Hkv=2, rows_per_tile=64, **kw)
+    o = host.options_mi355x(64, 256)
+    o.item_steps, o.part_steps, o.min_chunk, o.min_span, o.granule = 1, 0, 32, 64, 32
+    tiles, jobs, parts = host.plan_tiles(c.trees, c.params.Hkv, c.params.window, c.pos if c.params.window else None, o)
+    assert any(int(x["last"]) >= 2 for x in tiles) and parts > 0
     got = ob.attn_tiles(c.params, c.Q, c.Kb, c.Vb, c.pool_ref, c.blocks, c.desc, c.pos, tiles, c.trees, jobs, parts)
     assert max_abs(got, oracle_direct(c), c.params.dtype) <= 1e-3
 
