@@ -78,6 +78,8 @@ class Workload:
         self.trees, self.desc, self.pos = trees, desc, pos
         resident, groups = device.plan_hint(p)
         opts = host.options_mi355x(rows_per_tile, workgroups or resident)
+        for k, v in PLAN_TWEAK.items():   # experiments from the command line (--cut-batch, --plan-costs)
+            setattr(opts, k, v)
         self.tiles, self.jobs, self.n_parts = host.plan_tiles(trees, groups, window, pos if window > 0 else None, opts)
         # Block tables: disjoint slices of one seeded permutation of the pool, one slice per
         # rotation set, so a step never finds the previous step's pages in a cache.
@@ -518,6 +520,10 @@ def make_workload(name, workgroups=None, contiguous=False, page=16):
     if name == "c4_prefill_sliding":
         return Workload_(name, 16, 8, 256, F16, page, [(15360, 1024)] * 8, window=1024, rows_per_tile=128,
                         pool_pages=(8 * 1024 * 2) * 16 // page, seed=4, bound="mfma")
+    if name == "one_prompt_first_chunk":   # config 4's global layer on one prompt's first 2048 rows: 16 tiles x 16 heads, one per compute unit
+        return Workload_(name, 16, 8, 256, F16, page, [(0, 2048)], rows_per_tile=128, pool_pages=4096 * 16 // page, seed=4, bound="mfma")
+    if name == "one_prompt_first_chunk_hd128":   # the same rows on 16 heads of 128 dims: half of the slots of the narrower kernel
+        return Workload_(name, 16, 8, 128, BF16, page, [(0, 2048)], rows_per_tile=128, pool_pages=4096 * 16 // page, seed=4, bound="mfma")
     if name == "c4_prefill_global":
         return Workload_(name, 16, 8, 256, F16, page, [(15360, 1024)] * 8, rows_per_tile=128, pool_pages=(8 * 1024 * 2) * 16 // page, seed=4,
                         bound="mfma")
@@ -551,11 +557,14 @@ def traffic_source():
         return None
 
 
+PLAN_TWEAK = {}   # fields of the planner's options set from the command line
+
+
 WORKLOADS = ["c1_single_decode", "c2_batched_decode", "c3_prefill_p0", "c3_prefill_p2048", "c3_prefill_p4096",
              "c3_prefill_p6144", "c4_decode_sliding", "c4_decode_global", "c4_prefill_sliding", "c4_prefill_global",
              "c5_verify", "c4_decode_mix", "c4_prefill_mix", "c3_chunked_prefill", "c3_chunked_prefill_kb", "c3_attn_prep", "c4_attn_prep",
              "c4_head_gate", "c4_head_gate_dots", "g4_global512_decode", "g4_global512_verify", "g4_global512_verify_2row_tiles",
-             "g4_global512_prefill"]
+             "g4_global512_prefill", "one_prompt_first_chunk", "one_prompt_first_chunk_hd128"]
 
 
 def cpu_baseline(w, budget_s=20.0):
@@ -1214,6 +1223,8 @@ def main():
                     help="all (default): the batched decode as the headline, the chunked prefill, one record per benchmark "
                          "configuration and the measured ceilings; or c2_equal_<tokens> (16 equal sequences), or one of: hbm_read_ceiling, mfma_issue_ceiling, prefill_step_ceiling, prefill_step256_ceiling, decode_step_fusion, prefill_step_fusion, " + ", ".join(WORKLOADS))
     ap.add_argument("--workgroups", type=int, default=0, help="planner split target (0: ask esp_attn_plan_hint)")
+    ap.add_argument("--cut-batch", action="store_true", help="experiment: let the planner cut a tile's batch keys too (esp_plan_options.cut_batch)")
+    ap.add_argument("--plan-costs", default="", help="experiment: the planner's item_steps,part_steps (e.g. 3,4) instead of its own")
     ap.add_argument("--tables", default="scattered", choices=["scattered", "contiguous"],
                     help="block tables: a seeded permutation of the pool (the benchmark's definition) or address order")
     ap.add_argument("--page", type=int, default=16, help="tokens per KV block (the benchmark's definition: 16)")
@@ -1223,6 +1234,10 @@ def main():
     args = ap.parse_args()
     if args.gpus != 1:
         raise SystemExit("bench.py measures one GPU: this path has no multi-GPU leg (run with --gpus 1)")
+    if args.cut_batch:
+        PLAN_TWEAK["cut_batch"] = 1
+    if args.plan_costs:
+        PLAN_TWEAK["item_steps"], PLAN_TWEAK["part_steps"] = (int(x) for x in args.plan_costs.split(","))
 
     import torch
     from espetero_amd import device

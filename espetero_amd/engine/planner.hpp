@@ -48,6 +48,9 @@ struct PlanOptions {
   int part_steps = 0;  // what a split part costs on top: its partial record written, read again and merged
   // Tiled kernel, balanced rule: a tile's batch keys are cut like its cached keys (a pass of fewer workgroups than
   // slots - one prompt's first chunk - is otherwise as long as its last tile, which scans every row of the chunk).
+  // Off in mi355x(): measured on one 2048-row first chunk, 16 heads, the attention kernel gets shorter (head dim 256:
+  // 88 -> 77 us, head dim 128: 45 -> 35 us) and the step with the merge of the partial records behind it does not
+  // (86 -> 95 us, 45 -> 45 us).
   bool cut_batch = false;
 
   static PlanOptions reference() { return PlanOptions{}; }
@@ -68,7 +71,6 @@ struct PlanOptions {
       o.min_span = 1024;
       o.item_steps = 6;
       o.part_steps = 8;
-      o.cut_batch = true;
     }
     return o;
   }
@@ -159,11 +161,11 @@ inline void plan_tiles(AttnPlan& A, int groups, int window, const int32_t* pos, 
     ns_of = cand;
     long long best = finish_time(cand);
     const long long items = 1LL * n_tiles * groups, rounds = items / slots;
-    // No more workgroups than slots: one chunk for every tile, the chunks that cut the longest tile into 2 .. 8
+    // Fewer workgroups than slots (with cut_batch: no more than slots): one chunk for every tile, the chunks that cut the longest tile into 2 .. 8
     // parts (fewer parts first: ties keep them). With a round or more of whole workgroups such a split was
     // measured slower than none (two workgroups share a compute unit and the older one is served first, so the
     // slots are less alike than this hand-out takes them to be).
-    for (int parts = 2; parts <= 8 && items <= slots; ++parts) {
+    for (int parts = 2; parts <= 8 && (rounds == 0 || (o.cut_batch && items <= slots)); ++parts) {
       const long long c = std::max(c_lo, (c_hi + parts - 1) / parts) * o.granule;
       for (int i = 0; i < n_tiles; ++i) cand[size_t(i)] = int(parts_of(rts[size_t(i)], c));
       const long long t = finish_time(cand);

@@ -40,8 +40,9 @@ typedef struct esp_plan_options {
                             split chunk is the one whose workgroups finish earliest when handed to those slots in
                             dispatch order; this is a workgroup's fixed cost in steps of `granule` keys */
   int32_t part_steps;    /* the same rule: what a split part costs on top (its partial record and the merge) */
-  int32_t cut_batch;     /* the same rule: a tile's batch keys are cut like its cached keys where that finishes earlier (a part
-                            whose batch range ends early carries esp_tile.last = its last row + 2) */
+  int32_t cut_batch;     /* the same rule: a tile's batch keys are cut like its cached keys where the hand-out says that finishes
+                            earlier (a part whose batch range ends early carries esp_tile.last = its last row + 2); 0 in
+                            esp_plan_options_mi355x: the merge dispatch costs what the shorter kernel wins */
 } esp_plan_options;
 
 /* The reference's constants. */

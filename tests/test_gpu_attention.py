@@ -277,9 +277,9 @@ def test_tiled_kernel_chunk_longer_than_the_window(HD, rows, dtype, positions):
     dict(seqs=((16, 1400),), H=4, Hkv=2, rows_in_pool=True),                        # the rows read from the pool
 ])
 def test_tiled_kernel_cuts_the_batch_keys_of_a_tile(kw):
-    """The balanced rule cuts a tile's batch keys like its cached keys when a pass has few workgroups (a part whose batch
-    range ends early carries last = its last row + 2). Forced here by a cost model without fixed costs; held to the
-    checker, and to the uncut plan within the merge's own rounding."""
+    """With cut_batch the balanced rule cuts a tile's batch keys like its cached keys (a part whose batch range ends
+    early carries last = its last row + 2). Switched on here, with a cost model without fixed costs so that it cuts;
+    held to the checker, and to the uncut plan within the merge's own rounding."""
     from gpu_utils import plan, run_case
     in_pool = kw.pop("rows_in_pool", False)
     R = kw.pop("rows_per_tile", 128)
@@ -289,7 +289,7 @@ def test_tiled_kernel_cuts_the_batch_keys_of_a_tile(kw):
     else:
         c = small_case(seed=49, rows_per_tile=R, **kw)
     o = host.options_mi355x(R, 256)
-    o.item_steps, o.part_steps, o.min_chunk, o.min_span = 1, 0, 128, 256
+    o.cut_batch, o.item_steps, o.part_steps, o.min_chunk, o.min_span = 1, 1, 0, 128, 256
     tiles, _, n_parts = plan(c, o)
     cut = [x for x in tiles if int(x["last"]) >= 2]
     assert cut and n_parts > 0, "the plan has no part with a cut batch range"

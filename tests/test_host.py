@@ -126,22 +126,7 @@ def test_split_algebra_holds_for_both_rules(seed):
         assert seen == parts
 
 
-@pytest.mark.parametrize("seed", range(8))
-def test_tiled_kernel_plans_partition_every_tile(seed):
-    """The balanced rule for 128-row tiles (chosen by simulating the hand-out of workgroups to slots): whatever it
-    picks - no split, one chunk for all tiles, or only the shortest tiles cut - the cached ranges of a tile partition
-    [0, P), its batch ranges partition the batch rows (one open range in the last part, or cut ranges in front of it),
-    parts are numbered in record order and every merge job names them."""
-    rng = np.random.default_rng(900 + seed)
-    n = int(rng.integers(1, 5))
-    trees, base = [], 0
-    for _ in range(n):
-        P, m = int(rng.integers(0, 40) * 256), int(rng.integers(1, 2500))
-        trees.append((base, P, 0, m))
-        base += m
-    groups, slots = int(rng.choice([8, 16, 40])), int(rng.choice([256, 512]))
-    o = host.options_mi355x(128, slots)
-    tiles, jobs, parts = host.plan_tiles(np.array(trees, abi.TREE_DT), groups, 0, None, o)
+def _check_tiled_partition(trees, tiles, jobs, parts, o):
     by = {}
     for x in tiles:
         by.setdefault((int(x["tree"]), int(x["r0"])), []).append(x)
@@ -168,6 +153,47 @@ def test_tiled_kernel_plans_partition_every_tile(seed):
         assert k == P and b < min(m, r0 - base + 128)  # the open part begins inside the tile's own batch rows
     assert numbered == list(range(parts))          # in record order, which is the order the kernel's grid reverses
     assert sum(int(j["nparts"]) for j in jobs) == parts and all(int(j["nparts"]) >= 2 for j in jobs)
+    return cut
+
+
+@pytest.mark.parametrize("seed", range(8))
+def test_tiled_kernel_plans_partition_every_tile(seed):
+    """The balanced rule for 128-row tiles (chosen by simulating the hand-out of workgroups to slots): whatever it
+    picks - no split, one chunk for all tiles, or only the shortest tiles cut - the cached ranges of a tile partition
+    [0, P), its batch ranges partition the batch rows (one open range in the last part, or cut ranges in front of it),
+    parts are numbered in record order and every merge job names them."""
+    rng = np.random.default_rng(900 + seed)
+    n = int(rng.integers(1, 5))
+    trees, base = [], 0
+    for _ in range(n):
+        P, m = int(rng.integers(0, 40) * 256), int(rng.integers(1, 2500))
+        trees.append((base, P, 0, m))
+        base += m
+    groups, slots = int(rng.choice([8, 16, 40])), int(rng.choice([256, 512]))
+    o = host.options_mi355x(128, slots)
+    if seed % 2:   # with the batch keys open to cuts, and fixed costs low enough that some are made
+        o.cut_batch, o.item_steps, o.part_steps = 1, int(rng.choice([1, 3, 6])), int(rng.choice([0, 4, 8]))
+    tiles, jobs, parts = host.plan_tiles(np.array(trees, abi.TREE_DT), groups, 0, None, o)
+    _check_tiled_partition(trees, tiles, jobs, parts, o)
+
+
+@pytest.mark.parametrize("trees,groups,slots", [
+    ([(0, 0, 0, 2048)], 16, 256),                      # one prompt's first chunk: batch rows only
+    ([(0, 0, 0, 1500)], 8, 256),                       # ragged end
+    ([(0, 384, 0, 2048)], 16, 256),                    # a part that ends the cached keys and begins the batch rows
+    ([(0, 0, 0, 1100), (1100, 256, 0, 900)], 8, 512),  # two prompts
+    ([(0, 0, 0, 4096)], 4, 256),
+])
+def test_cut_batch_plans_partition_the_batch_rows(trees, groups, slots):
+    """With cut_batch (and fixed costs low enough that cuts are made) a tile's batch rows are cut like its cached keys:
+    parts with last = their last row + 2 in front of one open part, batch ranges that follow each other without a gap."""
+    o = host.options_mi355x(128, slots)
+    o.cut_batch, o.item_steps, o.part_steps = 1, 2, 2
+    tiles, jobs, parts = host.plan_tiles(np.array(trees, abi.TREE_DT), groups, 0, None, o)
+    assert _check_tiled_partition(trees, tiles, jobs, parts, o) > 0
+    o.cut_batch = 0
+    tiles, _, _ = host.plan_tiles(np.array(trees, abi.TREE_DT), groups, 0, None, o)
+    assert all(int(x["last"]) in (0, 1) for x in tiles)
 
 
 def test_a_round_and_a_quarter_of_workgroups_is_cut_at_its_short_end():

@@ -239,7 +239,7 @@ def test_cut_batch_ranges_match_direct(kw):
     the partial records of such parts, merged, equal the row-by-row call."""
     c = small_case(seed=24, H=4, Hkv=2, rows_per_tile=64, **kw)
     o = host.options_mi355x(64, 256)
-    o.item_steps, o.part_steps, o.min_chunk, o.min_span, o.granule = 1, 0, 32, 64, 32
+    o.cut_batch, o.item_steps, o.part_steps, o.min_chunk, o.min_span, o.granule = 1, 1, 0, 32, 64, 32
     tiles, jobs, parts = host.plan_tiles(c.trees, c.params.Hkv, c.params.window, c.pos if c.params.window else None, o)
     assert any(int(x["last"]) >= 2 for x in tiles) and parts > 0
     got = ob.attn_tiles(c.params, c.Q, c.Kb, c.Vb, c.pool_ref, c.blocks, c.desc, c.pos, tiles, c.trees, jobs, parts)
