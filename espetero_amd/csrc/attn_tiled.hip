@@ -419,7 +419,8 @@ __global__ __launch_bounds__(256, OCC) void attn_tiled_kernel(const KArgs a, int
         half_full = j0 >= tile.k0 && j0 + 32 <= tile.k1 && (a.window == 0 || qpos_max - j0 < a.window);
       } else if (s0 >= n_c && s0 + 2 <= n_sb) {
         const int j0 = ((a0 + s0 - n_c) << 4) - tree.base;
-        half_full = !batch_window && j0 >= seg_max && j0 + 31 <= rr0 + 32 * wave && j0 >= tile.b0 && j0 >= bw_lo;
+        // (j0 + 31 <= k_last matters where the part's batch range ends early: without a cut every row of the tile lies below k_last)
+        half_full = !batch_window && j0 >= seg_max && j0 + 31 <= min(rr0 + 32 * wave, k_last) && j0 >= tile.b0 && j0 >= bw_lo;
       } else {
         half_full = false;
       }

@@ -275,6 +275,11 @@ def test_tiled_kernel_chunk_longer_than_the_window(HD, rows, dtype, positions):
     dict(seqs=((40, 1300),), H=2, Hkv=2, bt=64, bidi=1, desc_fn=lambda M: synth.image_desc(M, 500, 900)),   # rows that see beyond their own tile
     dict(seqs=((0, 1200),), H=2, Hkv=1, HD=512, rows_per_tile=64),                  # head dim 512
     dict(seqs=((16, 1400),), H=4, Hkv=2, rows_in_pool=True),                        # the rows read from the pool
+    # a second tree whose rows begin 4 rows into a group of 16: a cut at a multiple of 64 of its own rows then falls inside a
+    # staged sub-block, whose keys behind the cut belong to the next part (a random sweep found them counted twice by the
+    # rows far enough below: the whole-half-step shortcut did not look at where the part's batch range ends)
+    dict(seqs=((634, 244), (1295, 369)), H=32, Hkv=2, HD=256, dtype=abi.ESP_BF16, fill_unused=True, wg=5000),
+    dict(seqs=((0, 250), (100, 900)), H=4, Hkv=2, dtype=abi.ESP_BF16, wg=5000),
 ])
 def test_tiled_kernel_cuts_the_batch_keys_of_a_tile(kw):
     """With cut_batch the balanced rule cuts a tile's batch keys like its cached keys (a part whose batch range ends
@@ -282,13 +287,13 @@ def test_tiled_kernel_cuts_the_batch_keys_of_a_tile(kw):
     held to the checker, and to the uncut plan within the merge's own rounding."""
     from gpu_utils import plan, run_case
     in_pool = kw.pop("rows_in_pool", False)
-    R = kw.pop("rows_per_tile", 128)
+    R, wg = kw.pop("rows_per_tile", 128), kw.pop("wg", 256)
     if in_pool:
         from test_gpu_rows_in_pool import pool_case
         c = pool_case(49, rows_per_tile=R, **kw)
     else:
         c = small_case(seed=49, rows_per_tile=R, **kw)
-    o = host.options_mi355x(R, 256)
+    o = host.options_mi355x(R, wg)
     o.cut_batch, o.item_steps, o.part_steps, o.min_chunk, o.min_span = 1, 1, 0, 128, 256
     tiles, _, n_parts = plan(c, o)
     cut = [x for x in tiles if int(x["last"]) >= 2]
