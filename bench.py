@@ -520,6 +520,12 @@ def make_workload(name, workgroups=None, contiguous=False, page=16):
     if name == "c4_prefill_sliding":
         return Workload_(name, 16, 8, 256, F16, page, [(15360, 1024)] * 8, window=1024, rows_per_tile=128,
                         pool_pages=(8 * 1024 * 2) * 16 // page, seed=4, bound="mfma")
+    if name == "c4_prefill_sliding_chunk2048":   # config 4's sliding layer with the reference's own chunk (2048 rows): twice the window
+        return Workload_(name, 16, 8, 256, F16, page, [(14336, 2048)] * 4, window=1024, rows_per_tile=128,
+                        pool_pages=(8 * 1024 * 2) * 16 // page, seed=4, bound="mfma")
+    if name == "c4_prefill_sliding_window512":   # ... and with a window half the chunk
+        return Workload_(name, 16, 8, 256, F16, page, [(15360, 1024)] * 8, window=512, rows_per_tile=128,
+                        pool_pages=(8 * 1024 * 2) * 16 // page, seed=4, bound="mfma")
     if name == "one_prompt_first_chunk":   # config 4's global layer on one prompt's first 2048 rows: 16 tiles x 16 heads, one per compute unit
         return Workload_(name, 16, 8, 256, F16, page, [(0, 2048)], rows_per_tile=128, pool_pages=4096 * 16 // page, seed=4, bound="mfma")
     if name == "one_prompt_first_chunk_hd128":   # the same rows on 16 heads of 128 dims: half of the slots of the narrower kernel
@@ -564,7 +570,8 @@ WORKLOADS = ["c1_single_decode", "c2_batched_decode", "c3_prefill_p0", "c3_prefi
              "c3_prefill_p6144", "c4_decode_sliding", "c4_decode_global", "c4_prefill_sliding", "c4_prefill_global",
              "c5_verify", "c4_decode_mix", "c4_prefill_mix", "c3_chunked_prefill", "c3_chunked_prefill_kb", "c3_attn_prep", "c4_attn_prep",
              "c4_head_gate", "c4_head_gate_dots", "g4_global512_decode", "g4_global512_verify", "g4_global512_verify_2row_tiles",
-             "g4_global512_prefill", "one_prompt_first_chunk", "one_prompt_first_chunk_hd128"]
+             "g4_global512_prefill", "one_prompt_first_chunk", "one_prompt_first_chunk_hd128", "c4_prefill_sliding_chunk2048",
+             "c4_prefill_sliding_window512"]
 
 
 def cpu_baseline(w, budget_s=20.0):

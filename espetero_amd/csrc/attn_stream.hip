@@ -44,7 +44,10 @@ namespace esp {
 // LP lanes share one output (consecutive lanes of a wavefront, `lp` = this lane's place among them): lane lp
 // merges records lp, lp + LP, .. in that order, and the LP running triples (max, sum, O) are then merged pairwise
 // across the lanes. One lane (LP = 1) is the plain merge in part order.
-template <int DT, int HD, int LP = 1>
+// MAXN: the most records in flight at a time. 32 serves decode passes (a group of up to 16 parts in one round of loads);
+// 8 costs a quarter of the registers, and with them four times the wavefronts per SIMD, which is what the merges of
+// prefill tiles want: few parts per group, many outputs, a kernel that lives on bytes in flight.
+template <int DT, int HD, int LP = 1, int MAXN = 32>
 __device__ __forceinline__ void merge_records(const KArgs& a, const esp_combine& job, int r, int h, int d, int lp = 0) {
   const int kvh = h / a.G, hg = h - kvh * a.G;
   const int col = r * a.G + hg;
@@ -102,6 +105,9 @@ __device__ __forceinline__ void merge_records(const KArgs& a, const esp_combine&
     if (lp != 0) return;
   } else if (job.nparts <= 2) {  // the split of a prefill tile: two records, nothing to repeat
     merge(0, std::integral_constant<int, 2>{});
+  } else if constexpr (MAXN <= 8) {
+    if (job.nparts <= 4) merge(0, std::integral_constant<int, 4>{});
+    else for (int s = 0; s < job.nparts; s += 8) merge(s, std::integral_constant<int, 8>{});
   } else if (job.nparts <= 8) {
     merge(0, std::integral_constant<int, 8>{});
   } else if (job.nparts <= 16) {
@@ -673,7 +679,7 @@ __global__ __launch_bounds__(HD >= 512 ? 128 * NC : 256, OCC) void attn_stream_k
 // The merge as its own dispatch: LP threads per (job, row, head, 4 dims). One thread each is what a pass of many
 // tile groups wants; a pass of few groups with many parts each (one long sequence decoded alone: 1024 outputs of 65
 // records) would leave all but a handful of compute units idle, so there 8 lanes share an output.
-template <int DT, int HD, int LP>
+template <int DT, int HD, int LP, int MAXN = 32>
 __global__ __launch_bounds__(256) void attn_combine_kernel(const KArgs a, const esp_combine* jobs, int n_jobs) {
   const int per_job = a.R * a.H * (HD / 4);
   const long tid_g = long(blockIdx.x) * 256 + threadIdx.x;
@@ -687,7 +693,7 @@ __global__ __launch_bounds__(256) void attn_combine_kernel(const KArgs a, const 
   const int h = rem / (HD / 4), d = (rem % (HD / 4)) * 4;
   const esp_combine job = jobs[ji];
   if (r >= job.rows) return;
-  merge_records<DT, HD, LP>(a, job, r, h, d, lp);
+  merge_records<DT, HD, LP, MAXN>(a, job, r, h, d, lp);
 }
 
 size_t stream_smem_bytes(int HD, int NC) {
@@ -774,6 +780,8 @@ static void launch_combine_t(const KArgs& a, const esp_combine* jobs, int n_jobs
   // more than 8 records per group on average and few outputs: share each output among 8 lanes
   if (n_parts > 8 * n_jobs && n * 8 <= (1L << 22)) {
     hipLaunchKernelGGL((attn_combine_kernel<DT, HD, 8>), dim3((unsigned)((n * 8 + 255) / 256)), dim3(256), 0, st, a, jobs, n_jobs);
+  } else if (a.R > 32) {  // tiles of the tiled kernels: many outputs, few parts each
+    hipLaunchKernelGGL((attn_combine_kernel<DT, HD, 1, 8>), dim3((unsigned)((n + 255) / 256)), dim3(256), 0, st, a, jobs, n_jobs);
   } else {
     hipLaunchKernelGGL((attn_combine_kernel<DT, HD, 1>), dim3((unsigned)((n + 255) / 256)), dim3(256), 0, st, a, jobs, n_jobs);
   }
