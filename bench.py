@@ -249,6 +249,8 @@ class ChunkedPrefill:
         perm = np.random.default_rng(seed).permutation(self.pool_pages).astype(np.int32)
         resident, groups = device.plan_hint(p)
         opts = host.options_mi355x(p.rows_per_tile, workgroups or resident)
+        for k, v in PLAN_TWEAK.items():
+            setattr(opts, k, v)
         self.sets, self.tiles, self.n_parts = [], [], 0
         for s_ in range(self.n_sets):
             table = perm[s_ * n_pages:(s_ + 1) * n_pages]
