@@ -1112,9 +1112,13 @@ class Ceilings:
 
     SHAPES256 = ("4 wavefronts x 32 rows, one per SIMD (as built)", "8 wavefronts as 4 pairs, P through LDS",
                  "8 wavefronts x 16 rows, v_mfma_f32_16x16x32")
-    LOADS256 = ("no staging loads", "64 KB per step staged behind the barrier", "one load behind each of the first 16 matrix instructions")
+    LOADS256 = ("no staging loads", "64 KB per step staged behind the barrier", "one load behind each of the first 16 matrix instructions",
+                "a second barrier in mid-step, each wavefront's loads beside two groups of matrix instructions of its own",
+                "no staging loads, operand reads one by one behind the matrix instructions",
+                "one load behind each of the first 16 matrix instructions, operand reads one by one",
+                "64 KB per step staged behind the barrier, operand reads one by one")
 
-    def prefill_step256(self, cases=((0, 0), (0, 1), (0, 2), (1, 0), (1, 1), (2, 0), (2, 1)), iters=1500):
+    def prefill_step256(self, cases=((0, 0), (0, 1), (0, 2), (0, 3), (0, 4), (0, 5), (0, 6), (1, 0), (1, 1), (2, 0), (2, 1)), iters=1500):
         """The 256-dim prefill step as bare instruction streams in three shapes of the workgroup, one workgroup per
         compute unit: TFLOP/s, cycles per step (64 keys x 128 rows) and the clock, both read inside the kernel."""
         t = self.torch

@@ -222,7 +222,9 @@ __global__ __launch_bounds__(256, ROWS == 2 ? 1 : 2) void step_kernel(float* out
 //   1  8 wavefronts as 4 pairs: a wavefront takes half of the step's keys through Q K^T and the softmax, hands its
 //      packed P to its partner through LDS and multiplies all 64 keys' P with its half of the dims
 //   2  8 wavefronts x 16 rows on v_mfma_f32_16x16x32: every wavefront a whole head, reading all of K and V^T
-// LOADS: 0 none, 1 all behind the barrier, 2 (shape 0) one behind each of the step's first 16 matrix instructions.
+// LOADS: 0 none, 1 all behind the barrier, 2 (shape 0) one behind each of the step's first 16 matrix instructions,
+// 3 (shape 0) a second barrier in mid-step and each wavefront's loads beside groups of its own; 4, 5, 6 (shape 0): 0, 2, 1
+// with the operand reads one by one behind the matrix instructions.
 __device__ __forceinline__ void stage_one(const char* base, uint32_t lane_off, uint32_t lds_addr) {
   lds_addr = uint32_t(__builtin_amdgcn_readfirstlane(int(lds_addr)));
   const uint64_t b64 = reinterpret_cast<uint64_t>(base);
@@ -242,11 +244,13 @@ __device__ __forceinline__ const char* step256_src(const char* src, int it, int 
   return src + ((size_t(blockIdx.x) * 977 * 16 + size_t(it) * 65536) & ((size_t(8) << 20) - 1 - 131071)) + size_t(wave) * per_wave;
 }
 
-template <int LOADS>
-__global__ __launch_bounds__(256, 1) void step256_kernel(float* out, int iters, const char* src, unsigned long long* clk) {
+template <int LOADS, int W>
+__device__ __forceinline__ void step256_body(float* out, int iters, const char* src, unsigned long long* clk) {
   const unsigned long long c0 = __builtin_readcyclecounter(), r0 = __builtin_amdgcn_s_memrealtime();
   extern __shared__ __attribute__((aligned(16))) char lds[];  // 64 KB of operands, 64 KB of staging space
-  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+  const int lane = threadIdx.x & 63, wave = W >= 0 ? W : int(threadIdx.x >> 6);
+  constexpr bool RI = LOADS >= 4;                                          // operand reads interleaved one by one
+  constexpr int LD = LOADS == 4 ? 0 : LOADS == 5 ? 2 : LOADS == 6 ? 1 : LOADS;  // where the staging loads go
   const u32x4 b = {step256_rnd(threadIdx.x + 11), step256_rnd(threadIdx.x + 13), step256_rnd(threadIdx.x + 17), step256_rnd(threadIdx.x + 19)};
   f32x16 c[8] = {};
   float v[16];
@@ -266,25 +270,40 @@ __global__ __launch_bounds__(256, 1) void step256_kernel(float* out, int iters, 
 #pragma unroll
     for (int g = 0; g < 8; ++g) {
 #pragma unroll
-      for (int j = 0; j < 8; ++j) ring[(g + 1) & 1][j] = *reinterpret_cast<lds_ptr>(base + ((g + 1) & 7) * 8192 + j * 1024);
-      __builtin_amdgcn_s_waitcnt(0xC07F | (8 << 8));
+      for (int j = 0; j < 8; ++j)
+        if constexpr (!RI) ring[(g + 1) & 1][j] = *reinterpret_cast<lds_ptr>(base + ((g + 1) & 7) * 8192 + j * 1024);
+      if constexpr (!RI) __builtin_amdgcn_s_waitcnt(0xC07F | (8 << 8));
 #pragma unroll
       for (int j = 0; j < 8; ++j) {
+        // reads one by one behind the matrix instructions: operand j of this group went out eight reads ago, and
+        // seven younger ones are in flight when it is needed
+        if constexpr (RI) __builtin_amdgcn_s_waitcnt(0xC07F | (7 << 8));
         c[g] = mm(ring[g & 1][j], b, c[g]);
+        if constexpr (RI) ring[(g + 1) & 1][j] = *reinterpret_cast<lds_ptr>(base + ((g + 1) & 7) * 8192 + j * 1024);
         if (g >= 2 && g < 6) {  // the softmax's share: 32 scores per lane and step beside 32 of the matrix instructions
           v[(2 * j) & 15] = __builtin_amdgcn_exp2f(v[(2 * j) & 15] - c[7][0]);
           v[(2 * j + 5) & 15] += v[(2 * j + 7) & 15];
           asm volatile("" : "+v"(v[(2 * j) & 15]));
         }
-        if constexpr (LOADS == 2) {
+        if constexpr (LD == 2) {
           if (g < 2) stage_one(sp + (8 * g + j) * 1024, lane * 16, dst + (8 * g + j) * 1024);
+        }
+        if constexpr (LOADS == 3) {  // wavefront w: half of its loads beside group w, the other half beside group 4 + w
+          if ((g & 3) == W) stage_one(sp + (8 * (g >> 2) + j) * 1024, lane * 16, dst + (8 * (g >> 2) + j) * 1024);
         }
         __builtin_amdgcn_sched_barrier(0);
       }
+      if constexpr (LOADS == 3) {
+        if (g == 3) {  // the barrier in mid-step: the loads issued a step ago have landed, the later 16 stay in flight
+          asm volatile("s_waitcnt vmcnt(16)" ::: "memory");
+          __syncthreads();
+        }
+      }
     }
-    if constexpr (LOADS != 0) asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+    if constexpr (LOADS == 3) asm volatile("s_waitcnt vmcnt(16)" ::: "memory");
+    else if constexpr (LD != 0) asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
     __syncthreads();
-    if constexpr (LOADS == 1) {
+    if constexpr (LD == 1) {
 #pragma unroll
       for (int q = 0; q < 16; ++q) stage_one(sp + q * 1024, lane * 16, dst + q * 1024);
     }
@@ -298,6 +317,19 @@ __global__ __launch_bounds__(256, 1) void step256_kernel(float* out, int iters, 
 #pragma unroll
   for (int i = 0; i < 16; ++i) r += c[0][i] + c[1][i] + c[2][i] + c[3][i] + c[4][i] + c[5][i] + c[6][i] + c[7][i] + v[i];
   out[blockIdx.x * 256 + threadIdx.x] = r;
+}
+template <int LOADS>
+__global__ __launch_bounds__(256, 1) void step256_kernel(float* out, int iters, const char* src, unsigned long long* clk) {
+  if constexpr (LOADS == 3) {  // a copy of the stream per wavefront, so that which groups carry its loads is fixed in the code
+    switch (__builtin_amdgcn_readfirstlane(threadIdx.x >> 6)) {
+      case 0: step256_body<LOADS, 0>(out, iters, src, clk); break;
+      case 1: step256_body<LOADS, 1>(out, iters, src, clk); break;
+      case 2: step256_body<LOADS, 2>(out, iters, src, clk); break;
+      default: step256_body<LOADS, 3>(out, iters, src, clk); break;
+    }
+  } else {
+    step256_body<LOADS, -1>(out, iters, src, clk);
+  }
 }
 
 template <int LOADS>
@@ -546,6 +578,10 @@ int esp_ceiling_prefill_step256(int32_t shape, int32_t loads, int32_t workgroups
     case 0: e = launch_lds(step256_kernel<0>, 131072, g, dim3(256), st, e0, e1, out, iters, s, clk); break;
     case 1: e = launch_lds(step256_kernel<1>, 131072, g, dim3(256), st, e0, e1, out, iters, s, clk); break;
     case 2: e = launch_lds(step256_kernel<2>, 131072, g, dim3(256), st, e0, e1, out, iters, s, clk); break;
+    case 3: e = launch_lds(step256_kernel<3>, 131072, g, dim3(256), st, e0, e1, out, iters, s, clk); break;
+    case 4: e = launch_lds(step256_kernel<4>, 131072, g, dim3(256), st, e0, e1, out, iters, s, clk); break;
+    case 5: e = launch_lds(step256_kernel<5>, 131072, g, dim3(256), st, e0, e1, out, iters, s, clk); break;
+    case 6: e = launch_lds(step256_kernel<6>, 131072, g, dim3(256), st, e0, e1, out, iters, s, clk); break;
     case 10: e = launch_lds(step256_pairs_kernel<0>, 147456, g, dim3(512), st, e0, e1, out, iters, s, clk); break;
     case 11: e = launch_lds(step256_pairs_kernel<1>, 147456, g, dim3(512), st, e0, e1, out, iters, s, clk); break;
     case 20: e = launch_lds(step256_rows16_kernel<0>, 131072, g, dim3(512), st, e0, e1, out, iters, s, clk); break;

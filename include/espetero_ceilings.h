@@ -58,7 +58,10 @@ int esp_ceiling_prefill_step(int32_t stage, int32_t rows, int32_t random_data, i
  * the softmax, handing its packed P to its partner through LDS and multiplying all 64 keys' P with its half of the dims;
  * 2 = 8 wavefronts x 16 rows on v_mfma_f32_16x16x32, each a whole head. loads: 0 = none, 1 = the step's 64 KB staged from
  * `src` (a device buffer of at least 8 MB + 64 KB, cache resident) straight into LDS behind the barrier, 2 (shape 0 only) =
- * one load behind each of the step's first 16 matrix instructions. One workgroup per compute unit. clk as above.
+ * one load behind each of the step's first 16 matrix instructions, 3 (shape 0 only) = a second barrier in mid-step and
+ * every wavefront's loads one by one beside two groups of matrix instructions that are its own (never two wavefronts
+ * loading at a time). 4, 5, 6 (shape 0 only) = 0, 2, 1 with the operand reads issued one by one, each behind the matrix
+ * instruction that frees its register, instead of a group's eight in a row. One workgroup per compute unit. clk as above.
  * out: workgroups * 512 floats. Flops of a launch: workgroups * iters * 256 * 32768. */
 int esp_ceiling_prefill_step256(int32_t shape, int32_t loads, int32_t workgroups, int32_t iters, float* out, const void* src, unsigned long long* clk,
                                 void* stream, void* start_event, void* stop_event);
