@@ -199,18 +199,30 @@ __global__ __launch_bounds__(256, OCC) void attn_tiled_kernel(const KArgs a, int
     }
   }
 
-  // Block ids of this wavefront's cached sub-blocks, 64 steps at a time: lane l holds the
-  // block of sub-block 4 (ids_step0 + l) + wave, so the per-step lookup is a lane read
-  // instead of a dependent memory access in front of every staging load.
-  int ids = 0, ids_step0 = -(1 << 30);
-  auto block_id = [&](int step) __attribute__((always_inline)) {
-    if (step < ids_step0 || step >= ids_step0 + 64) {
-      ids_step0 = step;
+  // Pool addresses of this wavefront's sub-blocks, 64 steps at a time: lane l holds the byte address of the K rows of
+  // sub-block 4 (adr_step0 + l) + wave - the block list entry, the head's place in the block and the sub-block's place
+  // in the head worked out by 64 lanes at once - so that in front of a step's staging loads stand two lane reads
+  // instead of a dependent memory access and the scalar arithmetic behind it. V^T of a 16-token sub-block lies
+  // bt rows' worth of bytes behind its K rows whatever the sub-block.
+  uint32_t kadr_lo = 0, kadr_hi = 0;
+  int adr_step0 = -(1 << 30);
+  auto pool_k = [&](int step) __attribute__((always_inline)) {
+    if (step < adr_step0 || step >= adr_step0 + 64) {
+      adr_step0 = step;
       const int sl = 4 * (step + lane) + wave;
       const int js = sl < n_c ? (c0 + sl) << 4 : (in_pool && sl < n_sb) ? ((a0 + sl - n_c) << 4) + pool_shift : -1;
-      ids = js >= 0 ? block_of(a, table, js) : 0;
+      uint64_t adr = 0;
+      if (js >= 0) {
+        const int b = block_of(a, table, js);
+        const int t0 = a.bt == 16 ? 0 : js % a.bt;
+        adr = reinterpret_cast<uint64_t>(a.pool + head_base(a, HD, b, kvh)) + uint64_t(t0) * ROWB;
+      }
+      kadr_lo = uint32_t(adr);
+      kadr_hi = uint32_t(adr >> 32);
     }
-    return __builtin_amdgcn_readlane(ids, step - ids_step0);
+    const int idx = step - adr_step0;
+    const uint32_t lo = uint32_t(__builtin_amdgcn_readlane(int(kadr_lo), idx)), hi = uint32_t(__builtin_amdgcn_readlane(int(kadr_hi), idx));
+    return reinterpret_cast<const char*>(uint64_t(lo) | (uint64_t(hi) << 32));
   };
 
   // ---- staging: per-lane constants of the load instructions
@@ -239,12 +251,8 @@ __global__ __launch_bounds__(256, OCC) void attn_tiled_kernel(const KArgs a, int
     asm volatile("" : "+v"(kc), "+v"(kr));
     const bool batch_sb = s >= n_c && (decltype(interior)::value || s < n_sb);
     if (s < n_c || (in_pool && batch_sb)) {
-      const int js = s < n_c ? (c0 + s) << 4 : ((a0 + s - n_c) << 4) + pool_shift;
-      const int b = block_id(step);
-      const int t0 = a.bt == 16 ? 0 : js % a.bt;
-      const char* hbp = reinterpret_cast<const char*>(a.pool + head_base(a, HD, b, kvh));
-      const char* kb = hbp + size_t(t0) * ROWB;
-      const char* vb = hbp + vt_elem(a.bt, HD, t0, 0) * 2;  // the 16-token sub-block: 32 HD contiguous bytes
+      const char* kb = pool_k(step);
+      const char* vb = kb + size_t(a.bt) * ROWB;  // the 16-token sub-block: 32 HD contiguous bytes
       const uint32_t kro = kr * ROWB;
 #pragma unroll
       for (int q = 0; q < KP; q += 4)
