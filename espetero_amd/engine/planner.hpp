@@ -49,8 +49,8 @@ struct PlanOptions {
   // Tiled kernel, balanced rule: a tile's batch keys are cut like its cached keys (a pass of fewer workgroups than
   // slots - one prompt's first chunk - is otherwise as long as its last tile, which scans every row of the chunk).
   // Off in mi355x(): measured on one 2048-row first chunk, 16 heads, the attention kernel gets shorter (head dim 256:
-  // 88 -> 77 us, head dim 128: 45 -> 35 us) and the step with the merge of the partial records behind it does not
-  // (86 -> 95 us, 45 -> 45 us).
+  // 80 -> 72 us, head dim 128: 42.5 -> 36.4 us) and the step with the merge of the partial records behind it does not
+  // (79.5 -> 82.9 us, 42.0 -> 43.3 us).
   bool cut_batch = false;
 
   static PlanOptions reference() { return PlanOptions{}; }
