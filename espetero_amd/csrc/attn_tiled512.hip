@@ -115,17 +115,28 @@ __global__ __launch_bounds__(256, 1) void attn_tiled512_kernel(const KArgs a, in
   // pi(4 wave + q) = pi(4 wave) + q. V^T: this wavefront brings pieces 256 wave .. + 255 of each sub-block's
   // 1024 (piece c: keys 8 (c % 2) .. + 7 of dim c / 2); position p holds piece p ^ ((p >> 4) & 1).
   const uint32_t lds_base = uint32_t(uintptr_t(lds));
-  // Block ids of the cached sub-blocks, 64 at a time: lane l holds the block of sub-block ids0 + l, so the
-  // per-step lookup is a lane read instead of a dependent memory access in front of every staging load.
-  int ids = 0, ids0 = -(1 << 30);
-  auto block_id = [&](int sidx) __attribute__((always_inline)) {
-    if (sidx < ids0 || sidx >= ids0 + 64) {
-      ids0 = sidx;
+  // Pool addresses of the sub-blocks, 64 at a time: lane l holds the byte address of the K rows of sub-block adr0 + l
+  // (block list entry, the head's place in the block, the sub-block's place in the head, worked out by 64 lanes at
+  // once), so that in front of a sub-block's staging loads stand two lane reads instead of a dependent memory access
+  // and the scalar arithmetic behind it. V^T of a sub-block lies bt rows' worth of bytes behind its K rows.
+  uint32_t kadr_lo = 0, kadr_hi = 0;
+  int adr0 = -(1 << 30);
+  auto pool_k = [&](int sidx) __attribute__((always_inline)) {
+    if (sidx < adr0 || sidx >= adr0 + 64) {
+      adr0 = sidx;
       const int sl = sidx + lane;
       const int js = sl < n_c ? (c0 + sl) << 4 : (in_pool && sl < n_sb) ? ((a0 + sl - n_c) << 4) + pool_shift : -1;
-      ids = js >= 0 ? block_of(a, table, js) : 0;
+      uint64_t adr = 0;
+      if (js >= 0) {
+        const int b = block_of(a, table, js);
+        adr = reinterpret_cast<uint64_t>(a.pool + head_base(a, kHD, b, kvh)) + uint64_t(js % a.bt) * 1024;
+      }
+      kadr_lo = uint32_t(adr);
+      kadr_hi = uint32_t(adr >> 32);
     }
-    return __builtin_amdgcn_readlane(ids, sidx - ids0);
+    const int idx = sidx - adr0;
+    const uint32_t lo = uint32_t(__builtin_amdgcn_readlane(int(kadr_lo), idx)), hi = uint32_t(__builtin_amdgcn_readlane(int(kadr_hi), idx));
+    return reinterpret_cast<const char*>(uint64_t(lo) | (uint64_t(hi) << 32));
   };
   const uint32_t kx = uint32_t(swap23(4 * wave));
   const uint32_t voff = uint32_t((lane ^ ((lane >> 4) & 1)) << 4);
@@ -137,12 +148,8 @@ __global__ __launch_bounds__(256, 1) void attn_tiled512_kernel(const KArgs a, in
       const uint32_t vdst = lds_base + stage * kStage + kKStage + t * kVSub + wave * 4096;
       const uint32_t kl = uint32_t(lane);
       if (sidx < n_c || (in_pool && sidx < n_sb)) {
-        const int js = sidx < n_c ? (c0 + sidx) << 4 : ((a0 + sidx - n_c) << 4) + pool_shift;
-        const int b = block_id(sidx);
-        const int t0 = js % a.bt;
-        const char* hbp = reinterpret_cast<const char*>(a.pool + head_base(a, kHD, b, kvh));
-        const char* kb = hbp + size_t(t0 + 4 * wave) * 1024;
-        const char* vb = hbp + vt_elem(a.bt, kHD, t0, 0) * 2 + wave * 4096;  // the 16-token sub-block: 16 KB contiguous
+        const char* kb = pool_k(sidx) + wave * 4096;
+        const char* vb = kb + size_t(a.bt) * 1024;  // the 16-token sub-block: 16 KB contiguous
         load_to_lds16_x4(kb, (kl ^ kx) << 4, (kl ^ (kx + 1)) << 4, (kl ^ (kx + 2)) << 4, (kl ^ (kx + 3)) << 4, kdst);
         load_to_lds16_x4(vb, voff, voff, voff, voff, vdst);
       } else if (sidx < n_sb) {
