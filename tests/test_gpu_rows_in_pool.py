@@ -44,6 +44,9 @@ def _both(case, options=None):
     dict(seqs=((128, 100),), H=4, Hkv=2, bidi=1, desc_fn=lambda M: synth.image_desc(M, 10, 90)),
     dict(seqs=((64, 150),), H=4, Hkv=2, HD=512, rows_per_tile=64),                 # head dim 512
     dict(seqs=((3008, 100),), H=4, Hkv=2, split=64),                               # split tiles: the last part owns the rows
+    dict(seqs=((3008, 1400),), H=2, Hkv=1),                                        # 69 steps: the 64-step address window is refilled inside the pass's own rows
+    dict(seqs=((2048, 2200),), H=2, Hkv=1, HD=256, bt=32),                         # the same at head dim 256 with 32-token blocks
+    dict(seqs=((1024, 1200),), H=2, Hkv=1, HD=512, rows_per_tile=64, bt=64),       # 512: 64 sub-blocks at a time, 139 in all
 ])
 def test_tiled_kernel_reads_its_rows_from_the_pool(kw):
     split = kw.pop("split", None)
