@@ -556,11 +556,14 @@ def measured_traffic(workload):
 
 
 def traffic_source():
-    """Where roofline.traffic comes from: the commit the rocprofv3 counter runs under profiles/ were taken at."""
+    """Where roofline.traffic comes from: the commit the rocprofv3 counter runs under profiles/ were last taken at,
+    and the commit of each workload's own runs."""
     try:
         with open(os.path.join(ROOT, "profiles", "traffic.json")) as f:
             t = json.load(f)
-        return {"file": "profiles/traffic.json", "measured_at_commit": t.get("_measured_at_commit"), "note": t.get("_note")}
+        per = {k: v.get("measured_at_commit") for k, v in t.items() if isinstance(v, dict) and "measured_at_commit" in v}
+        return {"file": "profiles/traffic.json", "measured_at_commit": t.get("_measured_at_commit"),
+                "per_workload": per, "note": t.get("_note")}
     except (OSError, ValueError):
         return None
 
