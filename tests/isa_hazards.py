@@ -1,5 +1,5 @@
-"""Checks gfx950 assembly for one class of hazard: a vector (or LDS / memory) instruction that reads the
-result of a matrix instruction, in another basic block, before the matrix pipeline has written it.
+"""Checks gfx950 assembly for one class of hazard: a vector (or LDS / memory) instruction that reads (or
+overwrites) the result of a matrix instruction, in another basic block, before the matrix pipeline has written it.
 
 Matrix instructions are not interlocked against such readers; the required distance is padded with wait
 states by the compiler, which only looks inside one basic block. A reader reached through a branch (or
@@ -85,6 +85,10 @@ def violations(lines):
                 srcs = set()
                 for a in (args if stores else args[1:]):
                     srcs |= _regs(a)
+                # (an instruction that overwrites the result registers while the matrix instruction is still in the
+                # pipeline is as bad as one that reads them early: its value is overwritten when the result lands)
+                if not stores and args and not op.startswith("s_"):
+                    srcs |= _regs(args[0])
                 if srcs & dst:
                     if crossed and HORIZON - left < need and not any(f[0] == i and f[2] == j for f in found):
                         found.append((i, " ".join([l[1]] + l[2]), j, " ".join([op] + args), HORIZON - left))

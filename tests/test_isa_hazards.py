@@ -40,10 +40,18 @@ _Z1kv:
     assert isa_hazards.violations(lines) == []          # in one block the compiler pads; not this check's business
 
 
+def _product_flags():
+    """The flags the library is built with (csrc/Makefile's HIPFLAGS): the scan is of the code that ships."""
+    text = open(os.path.join(CSRC, "Makefile")).read().replace("\\\n", " ")
+    line = next(l for l in text.splitlines() if l.startswith("HIPFLAGS"))
+    flags = line.split("=", 1)[1].replace("$(ARCH)", "gfx950").split()
+    assert "-amdgpu-mfma-vgpr-form=1" in flags and "--offload-arch=gfx950" in flags, flags
+    return [f for f in flags if f != "-fPIC"]
+
+
 def _assembly(src, out_dir):
     out = os.path.join(out_dir, src.replace(".hip", ".s"))
-    subprocess.run([HIPCC, "-O3", "-std=c++20", "--offload-arch=gfx950", "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops",
-                    "-Wno-unused-command-line-argument", "-S", "--cuda-device-only", "-o", out, os.path.join(CSRC, src)],
+    subprocess.run([HIPCC, *_product_flags(), "-S", "--cuda-device-only", "-o", out, os.path.join(CSRC, src)],
                    check=True, capture_output=True)
     return open(out).read()
 
