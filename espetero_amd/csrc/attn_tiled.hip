@@ -559,9 +559,9 @@ __global__ __launch_bounds__(256, OCC) void attn_tiled_kernel(const KArgs a, int
     }(std::make_integer_sequence<int, 8>{});
     return softmax_finish.template operator()<kt>();
   };
-  auto softmax_settle = [&](auto kt_c, float ps) __attribute__((always_inline)) {
+  auto softmax_settle = [&](auto kt_c, float ps, bool out_of_range) __attribute__((always_inline)) {
     constexpr int kt = decltype(kt_c)::value;
-    if (__any(!(ps <= p_limit))) {
+    if (out_of_range) {
       asm volatile("s_nop 0");  // a real branch: this block must not be speculated into the loop body
       f32x16& sv = s[kt];
       mfma_settle(sv);  // the tile's last matrix instruction was issued in another block
@@ -605,7 +605,11 @@ __global__ __launch_bounds__(256, OCC) void attn_tiled_kernel(const KArgs a, int
         softmax_pre(step, std::integral_constant<int, G == GK ? 0 : 1>{}, interior);
         __builtin_amdgcn_sched_barrier(0);
         // One matrix instruction, then its share of the eight slices, fenced so that the order stands.
-        constexpr int NM = GP - HEAD, KT = G == GK ? 0 : 1;
+        // The group's last matrix instructions wait until the half step's sum has been compared with its limit:
+        // they do not depend on P, and the branch on that comparison - a vector compare that the scalar unit has
+        // to wait for - then stands behind matrix instructions in flight instead of behind an idle pipe.
+        constexpr int TAILM = 2;  // (1: the same, 3: no gain - measured)
+        constexpr int NM = GP - HEAD - TAILM, KT = G == GK ? 0 : 1;
         [&]<int... M>(std::integer_sequence<int, M...>) __attribute__((always_inline)) {
           ([&]<int MI>() __attribute__((always_inline)) {
             mma_group.template operator()<G, HEAD + MI, HEAD + MI + 1>(ring[G & 1]);
@@ -616,8 +620,11 @@ __global__ __launch_bounds__(256, OCC) void attn_tiled_kernel(const KArgs a, int
           }.template operator()<M>(), ...);
         }(std::make_integer_sequence<int, NM>{});
         const float ps = softmax_finish.template operator()<KT>();
+        const bool out_of_range = __any(!(ps <= p_limit));
         __builtin_amdgcn_sched_barrier(0);
-        softmax_settle(std::integral_constant<int, G == GK ? 0 : 1>{}, ps);
+        mma_group.template operator()<G, GP - TAILM, GP>(ring[G & 1]);
+        __builtin_amdgcn_sched_barrier(0);
+        softmax_settle(std::integral_constant<int, G == GK ? 0 : 1>{}, ps, out_of_range);
       } else {
         // The first matrix instructions of the group go out before the branchy part of the softmax,
         // whose wait for the previous group's results they cover; the rest carry the arithmetic,
