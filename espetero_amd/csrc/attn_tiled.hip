@@ -477,30 +477,35 @@ __global__ __launch_bounds__(256, OCC) void attn_tiled_kernel(const KArgs a, int
         }
       }
     }
+    // The lane's maximum over the half step (head dim 256's lazy rescale; see softmax_move).
+    float x = -INFINITY;
     if constexpr (!LEAN) {
-      // Lazy rescale: the running reference m_run only moves when some lane's maximum exceeds
-      // it by more than 8 (log2 units), so P stays below 2^8 and the accumulators are rescaled
-      // a handful of times per row instead of once per step. The two lanes of a row agree on
-      // m_run because both take the maximum over the pair whenever either wants to move.
-      float x = -INFINITY;
 #pragma unroll
       for (int i = 0; i < 16; ++i) x = fmaxf(x, sv[i]);
       x *= a.scale_log2;  // scale > 0: the max commutes with it
-      if (__any(x > m_run + 8.0f)) {
-        asm volatile("s_nop 0");  // a real branch: this block must not be speculated into the loop body
-        const float m_new = fmaxf(m_run, fmaxf(x, __shfl_xor(x, 32)));
-        const float corr = (m_new == -INFINITY) ? 1.0f : fast_exp2(m_run - m_new);
-        m_run = m_new;
-        l_run *= corr;
-        if constexpr (kt == 0) {
+    }
+    return x;
+  };
+  // Lazy rescale: the running reference m_run only moves when some lane's maximum exceeds
+  // it by more than 8 (log2 units), so P stays below 2^8 and the accumulators are rescaled
+  // a handful of times per row instead of once per step. The two lanes of a row agree on
+  // m_run because both take the maximum over the pair whenever either wants to move.
+  auto softmax_move = [&](auto kt_c, float x, bool move) __attribute__((always_inline)) {
+    constexpr int kt = decltype(kt_c)::value;
+    if (move) {
+      asm volatile("s_nop 0");  // a real branch: this block must not be speculated into the loop body
+      const float m_new = fmaxf(m_run, fmaxf(x, __shfl_xor(x, 32)));
+      const float corr = (m_new == -INFINITY) ? 1.0f : fast_exp2(m_run - m_new);
+      m_run = m_new;
+      l_run *= corr;
+      if constexpr (kt == 0) {
 #pragma unroll
-          for (int nt = 0; nt < NT; ++nt) acc[nt] *= corr;
-        } else {
-          // P V of the first half step is still to be accumulated and its P is relative to the old
-          // reference: the accumulators take this factor once those products are in.
-          corr_late = corr;
-          late = true;
-        }
+        for (int nt = 0; nt < NT; ++nt) acc[nt] *= corr;
+      } else {
+        // P V of the first half step is still to be accumulated and its P is relative to the old
+        // reference: the accumulators take this factor once those products are in.
+        corr_late = corr;
+        late = true;
       }
     }
   };
@@ -629,18 +634,25 @@ __global__ __launch_bounds__(256, OCC) void attn_tiled_kernel(const KArgs a, int
         // The first matrix instructions of the group go out before the branchy part of the softmax,
         // whose wait for the previous group's results they cover; the rest carry the arithmetic,
         // one matrix instruction then its share.
-        constexpr int HEAD = 3;
+        constexpr int HEAD = 3, TAILH = 1;  // (TAILH 0: 1 % slower on full layers, 2: as 1 - measured)
+        constexpr std::integral_constant<int, G == GK ? 0 : 1> kt_c{};
         mma_group.template operator()<G, 0, HEAD>(ring[G & 1]);
         __builtin_amdgcn_sched_barrier(0);
-        softmax_pre(step, std::integral_constant<int, G == GK ? 0 : 1>{}, interior);
+        const float x = softmax_pre(step, kt_c, interior);
+        const bool move = __any(x > m_run + 8.0f);
         __builtin_amdgcn_sched_barrier(0);
-        mma_group.template operator()<G, HEAD, GP>(ring[G & 1]);
+        // (matrix instructions between the comparison and the branch on it, as at head dim 128)
+        mma_group.template operator()<G, HEAD, HEAD + TAILH>(ring[G & 1]);
+        __builtin_amdgcn_sched_barrier(0);
+        softmax_move(kt_c, x, move);
+        __builtin_amdgcn_sched_barrier(0);
+        mma_group.template operator()<G, HEAD + TAILH, GP>(ring[G & 1]);
         constexpr bool TWO = GK >= 2;  // the half step's Q K^T (or P V) is two groups: the second carries the other half
-        softmax_exp_fma.template operator()<0, TWO ? 1 : 2>(std::integral_constant<int, G == GK ? 0 : 1>{});
+        softmax_exp_fma.template operator()<0, TWO ? 1 : 2>(kt_c);
 #pragma unroll
-        for (int j = HEAD; j < GP; ++j) {
+        for (int j = HEAD + TAILH; j < GP; ++j) {
           __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
-          __builtin_amdgcn_sched_group_barrier(0x002, TWO ? 7 : 13, 0);
+          __builtin_amdgcn_sched_group_barrier(0x002, (TWO ? 35 : 65) / (GP - HEAD - TAILH), 0);
         }
       }
     } else if constexpr (!LEAN && GK >= 2 && (G == GK + 1 || G == 2 * GK + 1)) {
