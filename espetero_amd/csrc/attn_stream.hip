@@ -610,49 +610,61 @@ __global__ __launch_bounds__(HD >= 512 ? 128 * NC : 256, OCC) void attn_stream_k
     }
   }
 
-  // ---- merge the NS streams in order (paired wavefronts hold the same m and l and one half of the dims each)
+  // ---- merge the NS streams in order (paired wavefronts hold the same m and l and one half of the dims each).
+  // Every wavefront leaves its (m, l) and its accumulators as they are; behind one barrier each thread reads, for
+  // the 4 dims of a packed row it finishes, the NS references, sums and vectors in one round of LDS reads and
+  // weighs them itself. (Accumulators scaled by the writer, which first had to read every stream's reference
+  // behind a barrier of its own, cost a second barrier and two more dependent LDS round trips at the end of
+  // every workgroup's life.)
   float* o_sh = smem;                          // [NS][NC * 16][LDO]
   float* ml_sh = smem + NS * NC * 16 * LDO;    // [NS][NC * 16][2]
+  if constexpr (FUSED) __syncthreads();        // the prepared rows lie where the accumulators go: every wavefront is done with them
 #pragma unroll
   for (int c = 0; c < NCW; ++c) {
+    const int col = cbase + 16 * c + c16;
     float l = l_run[c];
     l += __shfl_xor(l, 16);
     l += __shfl_xor(l, 32);
     l_run[c] = l;
     if (q4 == 0) {
-      ml_sh[(strm * NC * 16 + cbase + 16 * c + c16) * 2] = m_run[c];
-      ml_sh[(strm * NC * 16 + cbase + 16 * c + c16) * 2 + 1] = l;
+      ml_sh[(strm * NC * 16 + col) * 2] = m_run[c];
+      ml_sh[(strm * NC * 16 + col) * 2 + 1] = l;
     }
-  }
-  __syncthreads();
-#pragma unroll
-  for (int c = 0; c < NCW; ++c) {
-    const int col = cbase + 16 * c + c16;
-    float M = -INFINITY;
-#pragma unroll
-    for (int w = 0; w < NS; ++w) M = fmaxf(M, ml_sh[(w * NC * 16 + col) * 2]);
-    const float f = (m_run[c] == -INFINITY) ? 0.0f : fast_exp2(m_run[c] - M);
     float* dst = o_sh + size_t(strm * NC * 16 + col) * LDO + dw + 4 * q4;
 #pragma unroll
-    for (int mt = 0; mt < MT; ++mt) *reinterpret_cast<f32x4*>(dst + 16 * mt) = acc[c][mt] * f;
+    for (int mt = 0; mt < MT; ++mt) *reinterpret_cast<f32x4*>(dst + 16 * mt) = acc[c][mt];
   }
   __syncthreads();
   // Each thread finishes 4 dims of one packed row at a time.
+  const int cols_live = min(a.cols, rows_live * a.G);  // packed rows m G + head, m < rows_live
   for (int i = threadIdx.x; i < NC * 16 * (HD / 4); i += NW * 64) {
     const int col = i / (HD / 4), d = (i % (HD / 4)) * 4;
-    const int m = col / a.G, hg = col - m * a.G;
-    if (col >= a.cols || m >= rows_live) continue;
-    float M = -INFINITY;
-#pragma unroll
-    for (int w = 0; w < NS; ++w) M = fmaxf(M, ml_sh[(w * NC * 16 + col) * 2]);
-    float L = 0.0f;
-    f32x4 o = {0, 0, 0, 0};
+    if (col >= cols_live) continue;  // (no division by G where a partial record is all that is written)
+    float mw[NS], lw[NS];
+    f32x4 ow[NS];
 #pragma unroll
     for (int w = 0; w < NS; ++w) {
-      const float mw = ml_sh[(w * NC * 16 + col) * 2];
-      const float f = (mw == -INFINITY) ? 0.0f : fast_exp2(mw - M);
-      L += f * ml_sh[(w * NC * 16 + col) * 2 + 1];
-      o += *reinterpret_cast<const f32x4*>(o_sh + size_t(w * NC * 16 + col) * LDO + d);
+      mw[w] = ml_sh[(w * NC * 16 + col) * 2];
+      lw[w] = ml_sh[(w * NC * 16 + col) * 2 + 1];
+      ow[w] = *reinterpret_cast<const f32x4*>(o_sh + size_t(w * NC * 16 + col) * LDO + d);
+    }
+    float M = -INFINITY;
+#pragma unroll
+    for (int w = 0; w < NS; ++w) M = fmaxf(M, mw[w]);
+    float L = 0.0f, fw[NS];
+#pragma unroll
+    for (int w = 0; w < NS; ++w) {
+      fw[w] = (mw[w] == -INFINITY) ? 0.0f : fast_exp2(mw[w] - M);
+      L += fw[w] * lw[w];
+    }
+    f32x4 o = {0, 0, 0, 0};
+    {
+#pragma clang fp contract(off)  // product, then sum: the bits of a writer that scaled and a reader that added
+#pragma unroll
+      for (int w = 0; w < NS; ++w) {
+        const f32x4 t = ow[w] * fw[w];
+        o += t;
+      }
     }
     if (tile.part >= 0) {
       const size_t rec = (size_t(tile.part) * a.Hkv + kvh) * a.cols + col;
@@ -662,6 +674,7 @@ __global__ __launch_bounds__(HD >= 512 ? 128 * NC : 256, OCC) void attn_stream_k
         a.parts_ml[rec * 2 + 1] = L;
       }
     } else {
+      const int m = col / a.G, hg = col - m * a.G;
       const int row = tile.r0 + m, h = kvh * a.G + hg;
       const float inv = L > 0.0f ? 1.0f / L : 0.0f;
       o *= inv;
