@@ -74,20 +74,13 @@ __global__ __launch_bounds__(256, OCC) void attn_tiled_kernel(const KArgs a, int
   const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
   const int l32 = lane & 31, hb = lane >> 5;
   esp_tile tile = a.tiles[tile_i];
-  const esp_tree tree = a.trees[tile.tree];
-  if (tile.k1 == INT32_MAX) tile.k1 = tree.P;  // open-ended range: up to the tree's cached length as it is now
-  const int table = tile.pad > 0 ? tile.pad - 1 : tree.table;
-  const int end = tree.base + tree.M;
-  const int rows_live = min(a.R, end - tile.r0);
-  const int rr0 = tile.r0 - tree.base;
 
-  // ---- this lane's row
+  // ---- this lane's row. Its loads need the tile's record only (a row past the tree's last one reads the pass's
+  // last row instead and is zeroed once the tree's record says so): they are in flight while that record arrives.
   const int m_row = 32 * wave + l32;
-  const bool row_ok = m_row < rows_live;
-  const int row = row_ok ? tile.r0 + m_row : tile.r0;
-  const int rr = rr0 + m_row;
-  const int4 d = a.desc ? a.desc[row] : make_int4(0, 0, 0, 0);
-  const int qpos = a.window > 0 ? a.pos[row].x : 0;
+  const int row = min(tile.r0 + m_row, a.n_rows - 1);
+  int4 d = a.desc ? a.desc[row] : make_int4(0, 0, 0, 0);
+  int qpos = a.window > 0 ? a.pos[row].x : 0;
   // Q fragments as stored. The scale (times log2 e) is applied to the fp32 score in the same fused
   // multiply-add that subtracts the row's reference: multiplying Q itself and rounding it back to the
   // storage type would cost every score a relative 2^-9 (bf16) before the exponential, which at logits
@@ -97,7 +90,108 @@ __global__ __launch_bounds__(256, OCC) void attn_tiled_kernel(const KArgs a, int
   {
     const uint16_t* qp = a.Q + size_t(row) * a.q_ld + size_t(h) * HD + 8 * hb;
 #pragma unroll
-    for (int ks = 0; ks < KS; ++ks) qf[ks] = row_ok ? *reinterpret_cast<const u32x4*>(qp + 16 * ks) : u32x4{0, 0, 0, 0};
+    for (int ks = 0; ks < KS; ++ks) qf[ks] = *reinterpret_cast<const u32x4*>(qp + 16 * ks);
+  }
+
+  const esp_tree tree = a.trees[tile.tree];
+  if (tile.k1 == INT32_MAX) tile.k1 = tree.P;  // open-ended range: up to the tree's cached length as it is now
+  const int table = tile.pad > 0 ? tile.pad - 1 : tree.table;
+  const int end = tree.base + tree.M;
+  const int rows_live = min(a.R, end - tile.r0);
+  const int rr0 = tile.r0 - tree.base;
+  const int rr = rr0 + m_row;
+
+  // ---- the key range as 16-key sub-blocks: cached [k0, k1), then batch rows [b0, k_last]
+  const int c0 = tile.k0 >> 4;
+  const int n_c = tile.k1 > tile.k0 ? ((tile.k1 + 15) >> 4) - c0 : 0;
+  const int a0 = (tree.base + tile.b0) >> 4;  // batch sub-blocks are groups of 16 absolute rows
+  // Batch rows in the pool (no Kb / Vb): the pass's rows were appended before the attention (esp_attn_prep with a
+  // row table, or esp_kv_save), row j of a tree at position P + j of the tree's own block list, and P - base is a
+  // multiple of 16 (the caller's promise; esp_attn_validate checks it). A batch sub-block - 16 absolute rows - is
+  // then one 16-token sub-block of the pool and is staged like a cached one; the masks stay in row numbers.
+  const bool in_pool = a.Kb == nullptr;
+  const int pool_shift = tree.P - tree.base;  // pool position of absolute row r: r + pool_shift
+  // Sub-blocks the tree's block list can name for this tile: the cached ones and, with the rows in the pool, the
+  // batch ones up to the tree's last row - at least those the tile will use (its batch range ends at a row that the
+  // rows' own facts give, which are still on their way here).
+  const int n_sb_list = n_c + ((in_pool && tile.last && tree.M > tile.b0) ? ((end - 1) >> 4) - a0 + 1 : 0);
+
+  // Pool addresses of this wavefront's sub-blocks, 64 steps at a time: lane l holds the byte address of the K rows of
+  // sub-block 4 (adr_step0 + l) + wave - the block list entry, the head's place in the block and the sub-block's place
+  // in the head worked out by 64 lanes at once - so that in front of a step's staging loads stand two lane reads
+  // instead of a dependent memory access and the scalar arithmetic behind it. V^T of a 16-token sub-block lies
+  // bt rows' worth of bytes behind its K rows whatever the sub-block.
+  uint32_t kadr_lo = 0, kadr_hi = 0;
+  int adr_step0 = -(1 << 30);
+  auto pool_k = [&](int step) __attribute__((always_inline)) {
+    if (step < adr_step0 || step >= adr_step0 + 64) {
+      adr_step0 = step;
+      const int sl = 4 * (step + lane) + wave;
+      const int js = sl < n_c ? (c0 + sl) << 4 : sl < n_sb_list ? ((a0 + sl - n_c) << 4) + pool_shift : -1;
+      uint64_t adr = 0;
+      if (js >= 0) {
+        const int b = block_of(a, table, js);
+        const int t0 = a.bt == 16 ? 0 : js % a.bt;
+        adr = reinterpret_cast<uint64_t>(a.pool + head_base(a, HD, b, kvh)) + uint64_t(t0) * ROWB;
+      }
+      kadr_lo = uint32_t(adr);
+      kadr_hi = uint32_t(adr >> 32);
+    }
+    const int idx = step - adr_step0;
+    const uint32_t lo = uint32_t(__builtin_amdgcn_readlane(int(kadr_lo), idx)), hi = uint32_t(__builtin_amdgcn_readlane(int(kadr_hi), idx));
+    return reinterpret_cast<const char*>(uint64_t(lo) | (uint64_t(hi) << 32));
+  };
+
+  // ---- staging: per-lane constants of the load instructions
+  // K instruction q covers rows q RPI .. of the sub-block; this lane brings chunk
+  // position `lane % CH` of row q RPI + lane / CH, i.e. global chunk position ^ pi(row).
+  const int r0 = lane / CH;
+  const uint32_t kcol0 = uint32_t(((lane % CH) ^ r0) << 4);
+  // cached keys: rows HD elements apart, i.e. instruction q's rows start 1024 q bytes further; that part
+  // travels in the instruction's immediate offset. Instruction q's lane offset is
+  // r0 ROWB + (kcol0 ^ kswz(q)); the staging code derives it where it is used.
+  auto kswz = [](int q) constexpr { return uint32_t(swap23(q * RPI) << 4); };
+  // V^T instruction q covers dims 32 q ..: this lane brings keys 8 (lane / 32) .. + 7 of dim 32 q + lane % 32.
+  // (32 V^T rows of 16 tokens are 1024 bytes, in the pool's sub-blocks and in the staged batch rows alike)
+  const uint32_t voff = uint32_t(l32 * 32 + hb * 16);
+
+  // This wavefront's sub-block of `step`, one the pool holds, into `stage`.
+  // The per-instruction lane offsets are derived here, in every call, from two registers. Computed
+  // once in front of the loops (which the compiler does with anything loop-invariant, hence the
+  // empty asm) they would occupy a register each for the whole kernel and end up in scratch
+  // memory, whose reloads wait on the same counter as the staging loads and serialise them.
+  auto stage_pool = [&](int step, int stage) __attribute__((always_inline)) {
+    const uint32_t kdst = lds_base + stage * KBUF + wave * (16 * ROWB);
+    const uint32_t vdst = lds_base + VOFF + stage * VBUF + wave * SUBV;
+    uint32_t kc = kcol0, kr = uint32_t(r0);
+    asm volatile("" : "+v"(kc), "+v"(kr));
+    const char* kb = pool_k(step);
+    const char* vb = kb + size_t(a.bt) * ROWB;  // the 16-token sub-block: 32 HD contiguous bytes
+    const uint32_t kro = kr * ROWB;
+#pragma unroll
+    for (int q = 0; q < KP; q += 4)
+      load_to_lds16_x4(kb + q * 1024, kro + (kc ^ kswz(q)), kro + (kc ^ kswz(q + 1)), kro + (kc ^ kswz(q + 2)),
+                       kro + (kc ^ kswz(q + 3)), kdst + q * 1024);
+#pragma unroll
+    for (int q = 0; q < VP; q += 4) load_to_lds16_x4(vb + q * 1024, voff, voff, voff, voff, vdst + q * 1024);
+  };
+  // Where the tile's first step is four sub-blocks of the pool whatever the rows' facts say - cached ones, or batch
+  // ones up to the tile's first row, which that row sees - its staging needs nothing of the rows: it leaves now,
+  // and the rows' facts below are worked out while it lands.
+  int n_b_sure = 0;
+  if (in_pool && tile.last) {
+    const int k_sure = min(min(rr0, tree.M - 1), tile.last >= 2 ? tile.last - 2 : INT32_MAX);
+    if (k_sure >= tile.b0) n_b_sure = ((tree.base + k_sure) >> 4) - a0 + 1;
+  }
+  const bool early = n_c + n_b_sure >= 4;
+  if (early) stage_pool(0, 0);
+
+  const bool row_ok = m_row < rows_live;
+  if (!row_ok) {
+    d = make_int4(0, 0, 0, 0);
+    qpos = 0;
+#pragma unroll
+    for (int ks = 0; ks < KS; ++ks) qf[ks] = u32x4{0, 0, 0, 0};
   }
 
   // ---- tile-wide facts about the rows (for the batch range and the no-mask fast path)
@@ -143,20 +237,10 @@ __global__ __launch_bounds__(256, OCC) void attn_tiled_kernel(const KArgs a, int
     anc_any = anc_max > 0;
   }
 
-  // ---- the key range as 16-key sub-blocks: cached [k0, k1), then batch rows [b0, k_last]
-  const int c0 = tile.k0 >> 4;
-  const int n_c = tile.k1 > tile.k0 ? ((tile.k1 + 15) >> 4) - c0 : 0;
-  const int a0 = (tree.base + tile.b0) >> 4;  // batch sub-blocks are groups of 16 absolute rows
   const int n_b = (tile.last && k_last >= tile.b0) ? ((tree.base + k_last) >> 4) - a0 + 1 : 0;
   const int n_sb = n_c + n_b;
   const int n_steps = (n_sb + 3) >> 2;
   const int n_groups = (a.n_rows + 15) >> 4;
-  // Batch rows in the pool (no Kb / Vb): the pass's rows were appended before the attention (esp_attn_prep with a
-  // row table, or esp_kv_save), row j of a tree at position P + j of the tree's own block list, and P - base is a
-  // multiple of 16 (the caller's promise; esp_attn_validate checks it). A batch sub-block - 16 absolute rows - is
-  // then one 16-token sub-block of the pool and is staged like a cached one; the masks stay in row numbers.
-  const bool in_pool = a.Kb == nullptr;
-  const int pool_shift = tree.P - tree.base;  // pool position of absolute row r: r + pool_shift
 
   // Windowed layers: do this tile's batch keys need a window test at all? Not when the oldest position among
   // them is inside the window of the row with the largest position. Where they do and their positions rise by
@@ -199,68 +283,17 @@ __global__ __launch_bounds__(256, OCC) void attn_tiled_kernel(const KArgs a, int
     }
   }
 
-  // Pool addresses of this wavefront's sub-blocks, 64 steps at a time: lane l holds the byte address of the K rows of
-  // sub-block 4 (adr_step0 + l) + wave - the block list entry, the head's place in the block and the sub-block's place
-  // in the head worked out by 64 lanes at once - so that in front of a step's staging loads stand two lane reads
-  // instead of a dependent memory access and the scalar arithmetic behind it. V^T of a 16-token sub-block lies
-  // bt rows' worth of bytes behind its K rows whatever the sub-block.
-  uint32_t kadr_lo = 0, kadr_hi = 0;
-  int adr_step0 = -(1 << 30);
-  auto pool_k = [&](int step) __attribute__((always_inline)) {
-    if (step < adr_step0 || step >= adr_step0 + 64) {
-      adr_step0 = step;
-      const int sl = 4 * (step + lane) + wave;
-      const int js = sl < n_c ? (c0 + sl) << 4 : (in_pool && sl < n_sb) ? ((a0 + sl - n_c) << 4) + pool_shift : -1;
-      uint64_t adr = 0;
-      if (js >= 0) {
-        const int b = block_of(a, table, js);
-        const int t0 = a.bt == 16 ? 0 : js % a.bt;
-        adr = reinterpret_cast<uint64_t>(a.pool + head_base(a, HD, b, kvh)) + uint64_t(t0) * ROWB;
-      }
-      kadr_lo = uint32_t(adr);
-      kadr_hi = uint32_t(adr >> 32);
-    }
-    const int idx = step - adr_step0;
-    const uint32_t lo = uint32_t(__builtin_amdgcn_readlane(int(kadr_lo), idx)), hi = uint32_t(__builtin_amdgcn_readlane(int(kadr_hi), idx));
-    return reinterpret_cast<const char*>(uint64_t(lo) | (uint64_t(hi) << 32));
-  };
-
-  // ---- staging: per-lane constants of the load instructions
-  // K instruction q covers rows q RPI .. of the sub-block; this lane brings chunk
-  // position `lane % CH` of row q RPI + lane / CH, i.e. global chunk position ^ pi(row).
-  const int r0 = lane / CH;
-  const uint32_t kcol0 = uint32_t(((lane % CH) ^ r0) << 4);
-  // cached keys: rows HD elements apart, i.e. instruction q's rows start 1024 q bytes further; that part
-  // travels in the instruction's immediate offset. Instruction q's lane offset is
-  // r0 ROWB + (kcol0 ^ kswz(q)); fill() derives it where it is used.
-  auto kswz = [](int q) constexpr { return uint32_t(swap23(q * RPI) << 4); };
-  // V^T instruction q covers dims 32 q ..: this lane brings keys 8 (lane / 32) .. + 7 of dim 32 q + lane % 32.
-  // (32 V^T rows of 16 tokens are 1024 bytes, in the pool's sub-blocks and in the staged batch rows alike)
-  const uint32_t voff = uint32_t(l32 * 32 + hb * 16);
-
   // interior: the caller knows that all four sub-blocks of the step are cached keys, or batch rows that exist.
   auto fill = [&](int step, int stage, auto interior) __attribute__((always_inline)) {
     const int s = 4 * step + wave;
-    const uint32_t kdst = lds_base + stage * KBUF + wave * (16 * ROWB);
-    const uint32_t vdst = lds_base + VOFF + stage * VBUF + wave * SUBV;
-    // The per-instruction lane offsets are derived here, in every call, from two registers. Computed
-    // once in front of the loops (which the compiler does with anything loop-invariant, hence the
-    // empty asm) they would occupy a register each for the whole kernel and end up in scratch
-    // memory, whose reloads wait on the same counter as the staging loads and serialise them.
-    uint32_t kc = kcol0, kr = uint32_t(r0);
-    asm volatile("" : "+v"(kc), "+v"(kr));
     const bool batch_sb = s >= n_c && (decltype(interior)::value || s < n_sb);
     if (s < n_c || (in_pool && batch_sb)) {
-      const char* kb = pool_k(step);
-      const char* vb = kb + size_t(a.bt) * ROWB;  // the 16-token sub-block: 32 HD contiguous bytes
-      const uint32_t kro = kr * ROWB;
-#pragma unroll
-      for (int q = 0; q < KP; q += 4)
-        load_to_lds16_x4(kb + q * 1024, kro + (kc ^ kswz(q)), kro + (kc ^ kswz(q + 1)), kro + (kc ^ kswz(q + 2)),
-                         kro + (kc ^ kswz(q + 3)), kdst + q * 1024);
-#pragma unroll
-      for (int q = 0; q < VP; q += 4) load_to_lds16_x4(vb + q * 1024, voff, voff, voff, voff, vdst + q * 1024);
+      stage_pool(step, stage);
     } else if (batch_sb) {
+      const uint32_t kdst = lds_base + stage * KBUF + wave * (16 * ROWB);
+      const uint32_t vdst = lds_base + VOFF + stage * VBUF + wave * SUBV;
+      uint32_t kc = kcol0, kr = uint32_t(r0);
+      asm volatile("" : "+v"(kc), "+v"(kr));
       const int g = a0 + (s - n_c);
       const int lim = decltype(interior)::value ? 15 : a.n_rows - 1 - 16 * g;  // batch rows past the pass's last row do not exist
       const char* kb = reinterpret_cast<const char*>(a.Kb + size_t(16 * g) * a.kv_ld + size_t(kvh) * HD);
@@ -738,7 +771,7 @@ __global__ __launch_bounds__(256, OCC) void attn_tiled_kernel(const KArgs a, int
   constexpr std::true_type inner{};
 
   if (n_steps > 0) {
-    fill(0, 0, general);
+    if (!early) fill(0, 0, general);
     wait_loads();
     fix(0, 0);
   }
