@@ -47,6 +47,9 @@ def _both(case, options=None):
     dict(seqs=((3008, 1400),), H=2, Hkv=1),                                        # 69 steps: the 64-step address window is refilled inside the pass's own rows
     dict(seqs=((2048, 2200),), H=2, Hkv=1, HD=256, bt=32),                         # the same at head dim 256 with 32-token blocks
     dict(seqs=((1024, 1200),), H=2, Hkv=1, HD=512, rows_per_tile=64, bt=64),       # 512: 64 sub-blocks at a time, 139 in all
+    dict(seqs=((16, 400),), H=4, Hkv=2),                                           # a first step of 1 cached sub-block and 3 of the pass's own
+    dict(seqs=((48, 300), (44, 140)), H=2, Hkv=1, HD=256, dtype=abi.ESP_BF16),     # 3 + 1, and (P - base = -256) 2 3/4 + 1 1/4, head dim 256
+    dict(seqs=((32, 24), (40, 330)), H=4, Hkv=2, window=96, fill_unused=True),     # P - base = 16: the cached range ends inside a sub-block; under a window
 ])
 def test_tiled_kernel_reads_its_rows_from_the_pool(kw):
     split = kw.pop("split", None)
