@@ -637,7 +637,7 @@ __global__ __launch_bounds__(256, OCC) void attn_tiled_kernel(const KArgs a, int
     if constexpr (G == GK || G == 2 * GK) {
       if constexpr (LEAN) {
         // On the mask-free path there is no branchy part and the whole group carries the arithmetic.
-        constexpr int HEAD = decltype(interior)::value ? 0 : 3;
+        constexpr int HEAD = decltype(interior)::value ? 0 : 3;  // (2, 4, 5: equal or slower - measured)
         mma_group.template operator()<G, 0, HEAD>(ring[G & 1]);
         __builtin_amdgcn_sched_barrier(0);
         softmax_pre(step, std::integral_constant<int, G == GK ? 0 : 1>{}, interior);
@@ -667,7 +667,8 @@ __global__ __launch_bounds__(256, OCC) void attn_tiled_kernel(const KArgs a, int
         // The first matrix instructions of the group go out before the branchy part of the softmax,
         // whose wait for the previous group's results they cover; the rest carry the arithmetic,
         // one matrix instruction then its share.
-        constexpr int HEAD = 3, TAILH = 1;  // (TAILH 0: 1 % slower on full layers, 2: as 1 - measured)
+        // (On steps with masks to work out five go first: 3 -> 5 is 1.3 % on sliding layers, 1 costs as much; 6 as 5.)
+        constexpr int HEAD = decltype(interior)::value ? 3 : 5, TAILH = 1;  // (TAILH 0: 1 % slower on full layers, 2: as 1 - measured)
         constexpr std::integral_constant<int, G == GK ? 0 : 1> kt_c{};
         mma_group.template operator()<G, 0, HEAD>(ring[G & 1]);
         __builtin_amdgcn_sched_barrier(0);
