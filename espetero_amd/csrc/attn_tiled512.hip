@@ -229,10 +229,21 @@ __global__ __launch_bounds__(256, 1) void attn_tiled512_kernel(const KArgs a, in
   // through two register buffers: K slices 0..7, K slices 8..15, V^T of sub-block 0, V^T of sub-block 1.
   // The reads of a group are in flight while the matrix cores consume the group before it; the V^T reads
   // do not depend on the softmax and cover the exchange of the partial scores.
+  //
+  // At the top of iteration i stage i % 2 holds step i, step i + 1 is on its way into the other stage and
+  // the first group of K slices of step i is being read. The iteration: both score groups, the exchange,
+  // the softmax - its second sub-block's share laid between the first sub-block's P V instructions - then,
+  // every operand of the step now in registers, the wait for the own loads of step i + 1, the barrier that
+  // publishes them, the request for step i + 2 into the stage just left, the first reads of step i + 1, and
+  // only then the second sub-block's P V instructions: they cover the barrier, the address arithmetic of the
+  // loads and the first read latency. (A wavefront issues in order: a matrix instruction hides only what
+  // stands right behind it.)
   u32x4 ring[2][8];
-  auto compute = [&]<int S>(int step, std::integral_constant<int, S>) __attribute__((always_inline)) {
+  auto read_k0 = [&]<int S>(std::integral_constant<int, S>) __attribute__((always_inline)) {
 #pragma unroll
     for (int j = 0; j < 8; ++j) ring[0][j] = *lds_ptr(kaddr[j] + uint32_t(S * kStage));
+  };
+  auto iter = [&]<int S>(int step, std::integral_constant<int, S>) __attribute__((always_inline)) {
 #pragma unroll
     for (int j = 0; j < 8; ++j) ring[1][j] = *lds_ptr(kaddr[j] + uint32_t(S * kStage + 256));
     __builtin_amdgcn_sched_barrier(0);
@@ -310,35 +321,40 @@ __global__ __launch_bounds__(256, 1) void attn_tiled512_kernel(const KArgs a, in
     const float m_safe = (m_run == -INFINITY) ? 0.0f : m_run;
     u32x4 pb[2];
     float ps = 0.0f;
-#pragma unroll
-    for (int t = 0; t < 2; ++t) {
+    // The row sum is that of the rounded P the products use: under a lazily moved reference the dominant P is
+    // not exactly 1, and O = sum(P~ v) / sum(P~) keeps its rounding out of a row that one key dominates.
+    auto exp_pack = [&]<int T>(std::integral_constant<int, T>) __attribute__((always_inline)) {
       float p[8];
 #pragma unroll
-      for (int e = 0; e < 8; ++e) p[e] = fast_exp2(__builtin_fmaf(s[8 * t + e], a.scale_log2, -m_safe));
-      pb[t] = u32x4{pack2<DT>(p[0], p[1]), pack2<DT>(p[2], p[3]), pack2<DT>(p[4], p[5]), pack2<DT>(p[6], p[7])};
-      // The row sum is that of the rounded P the products use: under a lazily moved reference the dominant P is
-      // not exactly 1, and O = sum(P~ v) / sum(P~) keeps its rounding out of a row that one key dominates.
+      for (int e = 0; e < 8; ++e) p[e] = fast_exp2(__builtin_fmaf(s[8 * T + e], a.scale_log2, -m_safe));
+      pb[T] = u32x4{pack2<DT>(p[0], p[1]), pack2<DT>(p[2], p[3]), pack2<DT>(p[4], p[5]), pack2<DT>(p[6], p[7])};
 #pragma unroll
-      for (int e = 0; e < 4; ++e) ps = sum2<DT>(pb[t][e], ps);
-    }
-    l_run += ps;
+      for (int e = 0; e < 4; ++e) ps = sum2<DT>(pb[T][e], ps);
+    };
+    exp_pack(std::integral_constant<int, 0>{});
     __builtin_amdgcn_sched_barrier(0);
-    // ---- O^T += V^T . P^T over this wavefront's dims
+    // ---- O^T += V^T . P^T over this wavefront's dims: the first sub-block's products, the second sub-block's
+    // exponentials between them
 #pragma unroll
     for (int nt = 0; nt < NT; ++nt) acc[nt] = mfma32x16<DT>(ring[0][nt], pb[0], acc[nt]);
+    exp_pack(std::integral_constant<int, 1>{});
+    asm volatile("" : "+v"(pb[1]), "+v"(ps));  // worked out here, not where pb[1] is first used
+#pragma unroll
+    for (int j = 0; j < NT; ++j) {
+      __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
+      __builtin_amdgcn_sched_group_barrier(0x002, 4, 0);
+    }
+    __builtin_amdgcn_sched_barrier(0);
+    l_run += ps;
+    asm volatile("s_waitcnt vmcnt(0) lgkmcnt(0)" ::: "memory");  // own loads of step + 1 landed, own reads of stage S done
+    if (step + 1 < n_steps) fix(step + 1, S ^ 1);
+    __syncthreads();
+    if (step + 2 < n_steps) fill(step + 2, S);
+    if (step + 1 < n_steps) read_k0(std::integral_constant<int, S ^ 1>{});
+    __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
     for (int nt = 0; nt < NT; ++nt) acc[nt] = mfma32x16<DT>(ring[1][nt], pb[1], acc[nt]);
-  };
-
-  // At the top of iteration i stage i % 2 holds step i and every wavefront has left the other stage: the
-  // loads of step i + 1 go straight into it while step i is in the matrix cores. The barrier at the end
-  // publishes them; the barrier inside compute() covers the exchange of the partial scores.
-  auto iter = [&]<int S>(int i, std::integral_constant<int, S> sc) __attribute__((always_inline)) {
-    if (i + 1 < n_steps) fill(i + 1, S ^ 1);
-    compute(i, sc);
-    wait_loads();
-    if (i + 1 < n_steps) fix(i + 1, S ^ 1);
-    __syncthreads();
+    __builtin_amdgcn_sched_barrier(0);
   };
   if (n_steps > 0) {
     fill(0, 0);
@@ -346,6 +362,8 @@ __global__ __launch_bounds__(256, 1) void attn_tiled512_kernel(const KArgs a, in
     fix(0, 0);
   }
   __syncthreads();
+  if (n_steps > 1) fill(1, 1);
+  if (n_steps > 0) read_k0(std::integral_constant<int, 0>{});
   {
     int i = 0;
 #pragma nounroll
