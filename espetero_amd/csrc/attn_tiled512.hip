@@ -140,14 +140,15 @@ __global__ __launch_bounds__(256, 1) void attn_tiled512_kernel(const KArgs a, in
   };
   const uint32_t kx = uint32_t(swap23(4 * wave));
   const uint32_t voff = uint32_t((lane ^ ((lane >> 4) & 1)) << 4);
-  auto fill = [&](int step, int stage) __attribute__((always_inline)) {
+  // plain: the caller knows that both sub-blocks of the step are cached keys.
+  auto fill = [&](int step, int stage, auto plain) __attribute__((always_inline)) {
 #pragma unroll
     for (int t = 0; t < 2; ++t) {
       const int sidx = 2 * step + t;
       const uint32_t kdst = lds_base + stage * kStage + (16 * t + 4 * wave) * 1024;
       const uint32_t vdst = lds_base + stage * kStage + kKStage + t * kVSub + wave * 4096;
       const uint32_t kl = uint32_t(lane);
-      if (sidx < n_c || (in_pool && sidx < n_sb)) {
+      if (decltype(plain)::value || sidx < n_c || (in_pool && sidx < n_sb)) {
         const char* kb = pool_k(sidx) + wave * 4096;
         const char* vb = kb + size_t(a.bt) * 1024;  // the 16-token sub-block: 16 KB contiguous
         load_to_lds16_x4(kb, (kl ^ kx) << 4, (kl ^ (kx + 1)) << 4, (kl ^ (kx + 2)) << 4, (kl ^ (kx + 3)) << 4, kdst);
@@ -243,7 +244,9 @@ __global__ __launch_bounds__(256, 1) void attn_tiled512_kernel(const KArgs a, in
 #pragma unroll
     for (int j = 0; j < 8; ++j) ring[0][j] = *lds_ptr(kaddr[j] + uint32_t(S * kStage));
   };
-  auto iter = [&]<int S>(int step, std::integral_constant<int, S>) __attribute__((always_inline)) {
+  // plain: steps `step` .. `step + 2` are cached keys wholly inside [k0, k1) of a layer without a window: every key is
+  // visible to every row, nothing staged needs fixing up, one kind of load.
+  auto iter = [&]<int S>(int step, std::integral_constant<int, S>, auto plain) __attribute__((always_inline)) {
 #pragma unroll
     for (int j = 0; j < 8; ++j) ring[1][j] = *lds_ptr(kaddr[j] + uint32_t(S * kStage + 256));
     __builtin_amdgcn_sched_barrier(0);
@@ -275,7 +278,7 @@ __global__ __launch_bounds__(256, 1) void attn_tiled512_kernel(const KArgs a, in
     }
     // ---- visibility
 #pragma unroll
-    for (int t = 0; t < 2; ++t) {
+    for (int t = 0; t < (decltype(plain)::value ? 0 : 2); ++t) {
       const int sidx = 2 * step + t;
       const bool cached = sidx < n_c, batch = !cached && sidx < n_sb;
       const int j0 = cached ? (c0 + sidx) << 4 : ((a0 + sidx - n_c) << 4) - tree.base;
@@ -347,31 +350,59 @@ __global__ __launch_bounds__(256, 1) void attn_tiled512_kernel(const KArgs a, in
     __builtin_amdgcn_sched_barrier(0);
     l_run += ps;
     asm volatile("s_waitcnt vmcnt(0) lgkmcnt(0)" ::: "memory");  // own loads of step + 1 landed, own reads of stage S done
-    if (step + 1 < n_steps) fix(step + 1, S ^ 1);
-    __syncthreads();
-    if (step + 2 < n_steps) fill(step + 2, S);
-    if (step + 1 < n_steps) read_k0(std::integral_constant<int, S ^ 1>{});
+    if constexpr (decltype(plain)::value) {
+      __syncthreads();
+      fill(step + 2, S, plain);
+      read_k0(std::integral_constant<int, S ^ 1>{});
+    } else {
+      if (step + 1 < n_steps) fix(step + 1, S ^ 1);
+      __syncthreads();
+      if (step + 2 < n_steps) fill(step + 2, S, plain);
+      if (step + 1 < n_steps) read_k0(std::integral_constant<int, S ^ 1>{});
+    }
     __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
     for (int nt = 0; nt < NT; ++nt) acc[nt] = mfma32x16<DT>(ring[1][nt], pb[1], acc[nt]);
     __builtin_amdgcn_sched_barrier(0);
   };
+  constexpr std::false_type general{};
+  constexpr std::true_type plain{};
   if (n_steps > 0) {
-    fill(0, 0);
+    fill(0, 0, general);
     wait_loads();
     fix(0, 0);
   }
   __syncthreads();
-  if (n_steps > 1) fill(1, 1);
+  if (n_steps > 1) fill(1, 1, general);
   if (n_steps > 0) read_k0(std::integral_constant<int, 0>{});
   {
+    // Plain iterations: pairs of steps i, i + 1 whose steps up to i + 3 are sub-blocks wholly inside the cached range.
+    int p0 = 0, p1 = 0;  // iterations [p0, p1), both even
+    if (a.window == 0 && n_c > 0) {
+      const int sb_lo = (tile.k0 & 15) ? 1 : 0, sb_hi = n_c - ((tile.k1 & 15) ? 1 : 0);  // sub-blocks [sb_lo, sb_hi) are whole
+      p0 = (((sb_lo + 1) >> 1) + 1) & ~1;
+      const int last = (sb_hi >> 1) - 3;  // last iteration i with 2 (i + 2) + 1 < sb_hi
+      p1 = last >= p0 ? p0 + ((last + 1 - p0) & ~1) : p0;
+    }
     int i = 0;
 #pragma nounroll
-    for (; i + 2 <= n_steps; i += 2) {
-      iter(i, std::integral_constant<int, 0>{});
-      iter(i + 1, std::integral_constant<int, 1>{});
+    for (; i + 2 <= min(p0, n_steps); i += 2) {
+      iter(i, std::integral_constant<int, 0>{}, general);
+      iter(i + 1, std::integral_constant<int, 1>{}, general);
     }
-    if (i < n_steps) iter(i, std::integral_constant<int, 0>{});
+    if (i == p0) {
+#pragma nounroll
+      for (; i + 2 <= p1; i += 2) {
+        iter(i, std::integral_constant<int, 0>{}, plain);
+        iter(i + 1, std::integral_constant<int, 1>{}, plain);
+      }
+    }
+#pragma nounroll
+    for (; i + 2 <= n_steps; i += 2) {
+      iter(i, std::integral_constant<int, 0>{}, general);
+      iter(i + 1, std::integral_constant<int, 1>{}, general);
+    }
+    if (i < n_steps) iter(i, std::integral_constant<int, 0>{}, general);
   }
 
   // ---- output: lane (row l32, half hb) holds dims dw + 32 nt + 8 i + 4 hb + j at acc[nt][4 i + j]

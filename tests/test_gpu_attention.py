@@ -209,6 +209,8 @@ def test_sharp_softmax_with_a_moving_maximum(kw, dtype):
     dict(seqs=((1203, 64), (700, 40)), bt=64, H=4, Hkv=2, fill_unused=True),  # long cached ranges, ragged end
     dict(seqs=((100, 2), (33, 1)), H=32, Hkv=1, rows_per_tile=2),       # G = 32, two rows: more packed rows (64) than the streaming kernel takes
     dict(seqs=((150, 20),), H=4, Hkv=2, rows_per_tile=24),              # tiles smaller than the kernel's 64 rows
+    dict(seqs=((4127, 96),), H=2, Hkv=1),                               # 258 cached sub-blocks, the last one partial: the mask-free iterations, 64 addresses at a time
+    dict(seqs=((2072, 70), (95, 3)), bt=32, H=4, Hkv=2, dtype=abi.ESP_BF16, fill_unused=True),   # the same beside a tile with too few for any
 ])
 def test_tiled_kernel_head_dim_512(kw):
     _check(small_case(seed=44, HD=512, **{"rows_per_tile": 64, **kw}))
