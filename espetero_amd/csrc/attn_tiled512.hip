@@ -21,7 +21,9 @@
 // The next step travels global memory -> the other LDS stage with global_load_lds_dwordx4
 // (no staging registers) while the current step is in the matrix cores.
 //
-// LDS layout of a stage. K: 32 rows of 1024 bytes, unpadded; the 16-byte chunk c of row r
+// LDS layout: K of stage 0, K of stage 1, V^T of stage 0, V^T of stage 1 (an operand read is a per-lane base
+// register plus an immediate, which takes 16 bits: with a stage's K and V^T side by side the second stage would lie
+// beyond it and every read of it would cost an addition). K of a stage: 32 rows of 1024 bytes, unpadded; the 16-byte chunk c of row r
 // lies at chunk position c ^ (pi(r) & 15), pi = swap of row bits 2 and 3. The lane with S^T
 // row l reads key row pi(l) at position c ^ (l & 15): 16 consecutive lanes hit 16 different
 // positions, and with the rows permuted by pi the 8 P values a lane packs for one P.V
@@ -39,7 +41,10 @@ namespace {
 constexpr int kHD = 512, kHW = 256;                  // dims of a head; dims one wavefront multiplies and accumulates
 constexpr int kKStage = 32 * kHD * 2;                // K of one stage: 32 rows
 constexpr int kVSub = kHD * 32;                      // V^T of one sub-block
-constexpr int kStage = kKStage + 2 * kVSub;
+constexpr int kVStage = 2 * kVSub;                   // V^T of one stage: two sub-blocks
+constexpr int kVBase = 2 * kKStage;                  // layout: K stage 0, K stage 1, V^T stage 0, V^T stage 1 - every operand read is
+                                                     // a per-lane base plus an immediate below 64 KB, whichever the stage
+constexpr int kStage = kKStage + kVStage;
 constexpr int kXch = 4 * 4 * 64 * 16;                // partial S^T: [wavefront][4][lane] 16-byte pieces
 constexpr int kLds = 2 * kStage + kXch + 64;         // two stages, the exchange, 16 ints
 }  // namespace
@@ -145,8 +150,8 @@ __global__ __launch_bounds__(256, 1) void attn_tiled512_kernel(const KArgs a, in
 #pragma unroll
     for (int t = 0; t < 2; ++t) {
       const int sidx = 2 * step + t;
-      const uint32_t kdst = lds_base + stage * kStage + (16 * t + 4 * wave) * 1024;
-      const uint32_t vdst = lds_base + stage * kStage + kKStage + t * kVSub + wave * 4096;
+      const uint32_t kdst = lds_base + stage * kKStage + (16 * t + 4 * wave) * 1024;
+      const uint32_t vdst = lds_base + kVBase + stage * kVStage + t * kVSub + wave * 4096;
       const uint32_t kl = uint32_t(lane);
       if (decltype(plain)::value || sidx < n_c || (in_pool && sidx < n_sb)) {
         const char* kb = pool_k(sidx) + wave * 4096;
@@ -165,7 +170,7 @@ __global__ __launch_bounds__(256, 1) void attn_tiled512_kernel(const KArgs a, in
       } else {  // past the range: K stays whatever it was (S is masked), V^T must be finite
 #pragma unroll
         for (int q = 0; q < 4; ++q)
-          *reinterpret_cast<u32x4*>(lds + stage * kStage + kKStage + t * kVSub + wave * 4096 + q * 1024 + lane * 16) = u32x4{0, 0, 0, 0};
+          *reinterpret_cast<u32x4*>(lds + kVBase + stage * kVStage + t * kVSub + wave * 4096 + q * 1024 + lane * 16) = u32x4{0, 0, 0, 0};
       }
     }
   };
@@ -200,7 +205,7 @@ __global__ __launch_bounds__(256, 1) void attn_tiled512_kernel(const KArgs a, in
       }
 #pragma unroll
       for (int q = 0; q < 4; ++q) {
-        u32x4* p = reinterpret_cast<u32x4*>(lds + stage * kStage + kKStage + t * kVSub + wave * 4096 + q * 1024 + lane * 16);
+        u32x4* p = reinterpret_cast<u32x4*>(lds + kVBase + stage * kVStage + t * kVSub + wave * 4096 + q * 1024 + lane * 16);
         *p = *p & msk;
       }
     }
@@ -217,7 +222,7 @@ __global__ __launch_bounds__(256, 1) void attn_tiled512_kernel(const KArgs a, in
     for (int j = 0; j < 8; ++j) kaddr[j] = lds_base + uint32_t(prow * 1024 + dw * 2 + (((2 * j + hb) ^ (l32 & 15)) << 4));
   }
   // V^T operand nt of sub-block t: keys 8 hb .. + 7 of dim dw + 32 nt + l32.
-  const uint32_t vaddr = lds_base + uint32_t(kKStage + (dw + l32) * 32 + ((hb ^ ((l32 >> 3) & 1)) << 4));
+  const uint32_t vaddr = lds_base + uint32_t(kVBase + (dw + l32) * 32 + ((hb ^ ((l32 >> 3) & 1)) << 4));
 
   f32x16 acc[NT];
   float m_run = -INFINITY, l_run = 0.0f;  // l_run: this lane's share (16 of every 32 keys) of the row's sum
@@ -242,13 +247,13 @@ __global__ __launch_bounds__(256, 1) void attn_tiled512_kernel(const KArgs a, in
   u32x4 ring[2][8];
   auto read_k0 = [&]<int S>(std::integral_constant<int, S>) __attribute__((always_inline)) {
 #pragma unroll
-    for (int j = 0; j < 8; ++j) ring[0][j] = *lds_ptr(kaddr[j] + uint32_t(S * kStage));
+    for (int j = 0; j < 8; ++j) ring[0][j] = *lds_ptr(kaddr[j] + uint32_t(S * kKStage));
   };
   // plain: steps `step` .. `step + 2` are cached keys wholly inside [k0, k1) of a layer without a window: every key is
   // visible to every row, nothing staged needs fixing up, one kind of load.
   auto iter = [&]<int S>(int step, std::integral_constant<int, S>, auto plain) __attribute__((always_inline)) {
 #pragma unroll
-    for (int j = 0; j < 8; ++j) ring[1][j] = *lds_ptr(kaddr[j] + uint32_t(S * kStage + 256));
+    for (int j = 0; j < 8; ++j) ring[1][j] = *lds_ptr(kaddr[j] + uint32_t(S * kKStage + 256));
     __builtin_amdgcn_sched_barrier(0);
     // s[4 i + j] is S^T row 8 i + 4 hb + j, which is key 16 (i / 2) + 8 hb + 4 (i % 2) + j of the step:
     // s[8 t + e] is key 8 hb + e of sub-block t.
@@ -259,13 +264,13 @@ __global__ __launch_bounds__(256, 1) void attn_tiled512_kernel(const KArgs a, in
     for (int j = 0; j < 8; ++j) s = mfma32x16<DT>(ring[0][j], qf[j], s);
     __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
-    for (int j = 0; j < 8; ++j) ring[0][j] = *lds_ptr(vaddr + uint32_t(S * kStage + j * 1024));
+    for (int j = 0; j < 8; ++j) ring[0][j] = *lds_ptr(vaddr + uint32_t(S * kVStage + j * 1024));
     __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
     for (int j = 0; j < 8; ++j) s = mfma32x16<DT>(ring[1][j], qf[8 + j], s);
     __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
-    for (int j = 0; j < 8; ++j) ring[1][j] = *lds_ptr(vaddr + uint32_t(S * kStage + kVSub + j * 1024));
+    for (int j = 0; j < 8; ++j) ring[1][j] = *lds_ptr(vaddr + uint32_t(S * kVStage + kVSub + j * 1024));
     // The other half of the dims: through LDS, added in the same order in both wavefronts of the pair.
 #pragma unroll
     for (int v = 0; v < 4; ++v) xch[(wave * 4 + v) * 64 + lane] = f32x4{s[4 * v], s[4 * v + 1], s[4 * v + 2], s[4 * v + 3]};
